@@ -1,0 +1,1018 @@
+// C ABI of libculsh_amd: context, scratch arena, seeded parameter generator, and the
+// orchestration of fit / query / fit_query for the three hashing families
+// (role of rplsh/rplsh.cu, pslsh/pslsh.cu, minhash/minhash.cu and of the *Core classes in
+// python/csrc/bindings.cu of the reference).
+#include <algorithm>
+#include <cmath>
+#include <cstring>
+#include <memory>
+#include <new>
+
+#include "common.hpp"
+
+namespace culsh_amd {
+
+// ---------------------------------------------------------------- errors
+static thread_local std::string g_last_error;
+
+void set_error(const char* fmt, ...) {
+    char buf[1024];
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(buf, sizeof(buf), fmt, ap);
+    va_end(ap);
+    g_last_error = buf;
+}
+
+// ---------------------------------------------------------------- arena
+static constexpr size_t ARENA_ALIGN = 256;
+
+culsh_status arena_begin(culsh_ctx* ctx) {
+    CULSH_HIP(hipSetDevice(ctx->device));
+    ctx->arena_off = 0;
+    if (ctx->arena_want > ctx->arena_cap) {  // stream is idle here: every call ends with a sync
+        if (ctx->arena) CULSH_HIP(hipFree(ctx->arena));
+        ctx->arena = nullptr;
+        ctx->arena_cap = 0;
+        const size_t want = align_up(ctx->arena_want + ctx->arena_want / 8, 1 << 20);
+        void* p = nullptr;
+        if (hipMalloc(&p, want) == hipSuccess) {
+            ctx->arena = static_cast<char*>(p);
+            ctx->arena_cap = want;
+        } else {
+            (void)hipGetLastError();  // fall back to per-allocation blocks
+        }
+    }
+    ctx->arena_want = 0;
+    return CULSH_OK;
+}
+
+culsh_status arena_alloc(culsh_ctx* ctx, size_t bytes, void** out) {
+    bytes = align_up(std::max<size_t>(bytes, 1), ARENA_ALIGN);
+    ctx->arena_want += bytes;
+    if (ctx->arena && ctx->arena_off + bytes <= ctx->arena_cap) {
+        *out = ctx->arena + ctx->arena_off;
+        ctx->arena_off += bytes;
+        return CULSH_OK;
+    }
+    void* p = nullptr;
+    CULSH_HIP(hipMalloc(&p, bytes));
+    ctx->overflow.push_back(p);
+    *out = p;
+    return CULSH_OK;
+}
+
+culsh_status arena_end(culsh_ctx* ctx) {
+    hipError_t e = hipStreamSynchronize(ctx->stream);
+    for (void* p : ctx->overflow) (void)hipFree(p);
+    ctx->overflow.clear();
+    if (e != hipSuccess) {
+        set_error("stream synchronize failed: %s", hipGetErrorString(e));
+        return CULSH_ERR_HIP;
+    }
+    return CULSH_OK;
+}
+
+culsh_status read_back_u64(culsh_ctx* ctx, const uint64_t* dev, int count, uint64_t* host) {
+    CULSH_REQUIRE(count <= 64, CULSH_ERR_INTERNAL, "read_back: too many words");
+    CULSH_HIP(hipMemcpyAsync(ctx->pinned, dev, count * sizeof(uint64_t), hipMemcpyDeviceToHost, ctx->stream));
+    CULSH_HIP(hipStreamSynchronize(ctx->stream));
+    std::memcpy(host, ctx->pinned, count * sizeof(uint64_t));
+    return CULSH_OK;
+}
+
+culsh_status read_back_u32(culsh_ctx* ctx, const uint32_t* dev, int count, uint32_t* host) {
+    CULSH_REQUIRE(count <= 128, CULSH_ERR_INTERNAL, "read_back: too many words");
+    CULSH_HIP(hipMemcpyAsync(ctx->pinned, dev, count * sizeof(uint32_t), hipMemcpyDeviceToHost, ctx->stream));
+    CULSH_HIP(hipStreamSynchronize(ctx->stream));
+    std::memcpy(host, ctx->pinned, count * sizeof(uint32_t));
+    return CULSH_OK;
+}
+
+// ---------------------------------------------------------------- seeded generator
+// splitmix64 counter streams: r[i] = sm64(key + i), key = sm64(sm64(seed) ^ sm64(stream)).
+static inline uint64_t sm64(uint64_t x) {
+    uint64_t z = x + 0x9E3779B97F4A7C15ull;
+    z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+    z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+    return z ^ (z >> 31);
+}
+enum { STREAM_PROJECTION = 1, STREAM_BIAS = 2, STREAM_HASH_A = 3, STREAM_HASH_B = 4 };
+
+void gen_raw_u64(uint64_t seed, int stream, size_t n, uint64_t* out) {
+    const uint64_t key = sm64(sm64(seed) ^ sm64(static_cast<uint64_t>(stream)));
+    for (size_t i = 0; i < n; ++i) out[i] = sm64(key + i);
+}
+
+// Box-Muller: z = sqrt(-2 ln u1) cos(2 pi u2), u1 in (0,1], u2 in [0,1), 53-bit uniforms.
+void gen_normals_f64(uint64_t seed, int stream, size_t n, double* out) {
+    const uint64_t key = sm64(sm64(seed) ^ sm64(static_cast<uint64_t>(stream)));
+    const double inv = 1.0 / 9007199254740992.0;
+    const double two_pi = 6.283185307179586476925286766559;
+    for (size_t i = 0; i < n; ++i) {
+        const double u1 = static_cast<double>((sm64(key + 2 * i) >> 11) + 1) * inv;
+        const double u2 = static_cast<double>(sm64(key + 2 * i + 1) >> 11) * inv;
+        out[i] = std::sqrt(-2.0 * std::log(u1)) * std::cos(two_pi * u2);
+    }
+}
+
+template <typename T>
+static void gen_projection(uint64_t seed, size_t count, int window, T* P) {
+    std::vector<double> z(count);
+    gen_normals_f64(seed, STREAM_PROJECTION, count, z.data());
+    for (size_t i = 0; i < count; ++i) {
+        T v = static_cast<T>(z[i]);
+        if (window > 0) v = v / static_cast<T>(window);  // pslsh/hash.cuh:85-86
+        P[i] = v;
+    }
+}
+
+template <typename T>
+static void gen_bias(uint64_t seed, size_t count, T* b) {  // uniform in (0,1], pslsh/hash.cuh:71-73
+    std::vector<uint64_t> r(count);
+    gen_raw_u64(seed, STREAM_BIAS, count, r.data());
+    for (size_t i = 0; i < count; ++i)
+        b[i] = static_cast<T>(static_cast<double>((r[i] >> 11) + 1) * (1.0 / 9007199254740992.0));
+}
+
+static void gen_minhash(uint64_t seed, size_t count, uint32_t* A, uint32_t* B) {
+    const uint64_t p = 4294967291ull;  // minhash/hash.cuh:17
+    std::vector<uint64_t> r(count);
+    gen_raw_u64(seed, STREAM_HASH_A, count, r.data());
+    for (size_t i = 0; i < count; ++i) A[i] = static_cast<uint32_t>(((r[i] >> 32) % (p - 1)) + 1);  // :27-28
+    gen_raw_u64(seed, STREAM_HASH_B, count, r.data());
+    for (size_t i = 0; i < count; ++i) B[i] = static_cast<uint32_t>((r[i] >> 32) % p);              // :30-31
+}
+
+// ---------------------------------------------------------------- object helpers
+void free_index_arrays(culsh_index* ix) {
+    if (!ix) return;
+    (void)hipFree(ix->all_candidate_indices);
+    (void)hipFree(ix->all_bucket_signatures);
+    (void)hipFree(ix->bucket_candidate_offsets);
+    (void)hipFree(ix->table_bucket_offsets);
+    (void)hipFree(ix->bucket_keys);
+    (void)hipFree(ix->P);
+    (void)hipFree(ix->b);
+    (void)hipFree(ix->A);
+    (void)hipFree(ix->B);
+    ix->all_candidate_indices = nullptr;
+    ix->all_bucket_signatures = nullptr;
+    ix->bucket_candidate_offsets = nullptr;
+    ix->table_bucket_offsets = nullptr;
+    ix->bucket_keys = nullptr;
+    ix->P = ix->b = nullptr;
+    ix->A = ix->B = nullptr;
+}
+
+void free_candidates_arrays(culsh_candidates* c) {
+    if (!c) return;
+    (void)hipFree(c->query_candidate_indices);
+    (void)hipFree(c->query_candidate_counts);
+    (void)hipFree(c->query_candidate_offsets);
+    c->query_candidate_indices = nullptr;
+    c->query_candidate_counts = nullptr;
+    c->query_candidate_offsets = nullptr;
+}
+
+struct IndexDeleter {
+    void operator()(culsh_index* p) const { free_index_arrays(p); delete p; }
+};
+struct CandDeleter {
+    void operator()(culsh_candidates* p) const { free_candidates_arrays(p); delete p; }
+};
+using IndexPtr = std::unique_ptr<culsh_index, IndexDeleter>;
+using CandPtr = std::unique_ptr<culsh_candidates, CandDeleter>;
+
+template <typename T>
+static culsh_status upload(const T* host, size_t count, T** dev) {
+    *dev = nullptr;
+    if (count == 0) return CULSH_OK;  // empty array -> nullptr (array_utils.cuh:34-36)
+    CULSH_HIP(hipMalloc(reinterpret_cast<void**>(dev), count * sizeof(T)));
+    CULSH_HIP(hipMemcpy(*dev, host, count * sizeof(T), hipMemcpyHostToDevice));
+    return CULSH_OK;
+}
+
+static culsh_status check_fit_args(culsh_ctx* ctx, const void* X, int n, int d, int T, int H, void* out) {
+    CULSH_REQUIRE(ctx && X && out, CULSH_ERR_INVALID, "null argument");
+    CULSH_REQUIRE(n > 0 && d > 0, CULSH_ERR_INVALID, "n_samples and n_features must be positive");
+    CULSH_REQUIRE(T > 0 && H > 0, CULSH_ERR_INVALID, "n_hash_tables and n_hashes must be positive");
+    CULSH_REQUIRE(T <= 65535, CULSH_ERR_LIMIT, "n_hash_tables > 65535 is not supported");
+    CULSH_REQUIRE(static_cast<long long>(n) * T < (1ll << 31), CULSH_ERR_LIMIT,
+                  "n_samples * n_hash_tables must be below 2^31 (int32 candidate positions)");
+    return CULSH_OK;
+}
+
+// ---------------------------------------------------------------- hashing to key words
+enum Family { FAM_RPLSH, FAM_PSLSH };
+
+// Dense rows -> key words [T][rows][W] in the arena.
+template <typename T>
+static culsh_status hash_dense_to_keys(culsh_ctx* ctx, Family fam, const T* X, int rows, int d, int nT, int H,
+                                       const void* P, const void* b, uint32_t** keys_out, int* W_out) {
+    const size_t N = static_cast<size_t>(rows) * nT;
+    const KeyEnc enc = (fam == FAM_RPLSH) ? ENC_BITS : ENC_BE;
+    const int S = (fam == FAM_RPLSH) ? H : 4 * H;
+    const int W = key_words(enc, S);
+    uint32_t* keys = nullptr;
+    CULSH_TRY(arena_alloc_t(ctx, N * W, &keys));
+    if constexpr (std::is_same_v<T, float>) {
+        CULSH_TRY(launch_project_f32(ctx, X, static_cast<const float*>(P), static_cast<const float*>(b), rows, d, nT,
+                                     H, fam == FAM_RPLSH ? EPI_SIGN_KEYS : EPI_FLOOR_KEYS, keys));
+    } else {
+        uint8_t* sig = nullptr;
+        CULSH_TRY(arena_alloc_t(ctx, N * S, &sig));
+        CULSH_TRY(launch_project_f64(ctx, X, static_cast<const double*>(P), static_cast<const double*>(b), rows, d,
+                                     nT, H, fam == FAM_RPLSH ? EPI_SIGN_BYTES : EPI_FLOOR_I32, sig));
+        CULSH_TRY(launch_sig_to_keys(ctx, sig, N, S, enc, W, keys));
+    }
+    *keys_out = keys;
+    *W_out = W;
+    return CULSH_OK;
+}
+
+// ---------------------------------------------------------------- candidates concatenation
+__global__ void shift_offsets_kernel(const uint64_t* __restrict__ src, uint64_t* __restrict__ dst, size_t count,
+                                     uint64_t base) {
+    const size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (i < count) dst[i] = src[i] + base;
+}
+
+// One pre-sized result instead of the reference's re-allocation per batch
+// (Candidates::merge, core/candidates.cuh:139-197); same contents.
+static culsh_status concat_candidates(culsh_ctx* ctx, const std::vector<culsh_candidates*>& parts,
+                                      culsh_candidates* out) {
+    size_t nq = 0;
+    uint64_t total = 0;
+    for (auto* p : parts) { nq += p->n_queries; total += p->n_total_candidates; }
+    CULSH_REQUIRE(nq < (1ull << 31), CULSH_ERR_LIMIT, "too many queries");
+    out->n_queries = static_cast<int>(nq);
+    out->n_total_candidates = total;
+    CULSH_HIP(hipMalloc(&out->query_candidate_counts, std::max<size_t>(1, nq) * sizeof(uint64_t)));
+    CULSH_HIP(hipMalloc(&out->query_candidate_offsets, (nq + 1) * sizeof(uint64_t)));
+    if (total) CULSH_HIP(hipMalloc(&out->query_candidate_indices, total * sizeof(int32_t)));
+    size_t q0 = 0;
+    uint64_t c0 = 0;
+    CULSH_HIP(hipMemsetAsync(out->query_candidate_offsets, 0, sizeof(uint64_t), ctx->stream));
+    for (auto* p : parts) {
+        if (p->n_total_candidates)
+            CULSH_HIP(hipMemcpyAsync(out->query_candidate_indices + c0, p->query_candidate_indices,
+                                     p->n_total_candidates * sizeof(int32_t), hipMemcpyDeviceToDevice, ctx->stream));
+        if (p->n_queries) {
+            CULSH_HIP(hipMemcpyAsync(out->query_candidate_counts + q0, p->query_candidate_counts,
+                                     p->n_queries * sizeof(uint64_t), hipMemcpyDeviceToDevice, ctx->stream));
+            // offsets[1..] of the part, shifted by the running total (candidates.cuh:178-183)
+            hipLaunchKernelGGL(shift_offsets_kernel, dim3(div_up(p->n_queries, 256)), dim3(256), 0, ctx->stream,
+                               p->query_candidate_offsets + 1, out->query_candidate_offsets + q0 + 1,
+                               static_cast<size_t>(p->n_queries), c0);
+            CULSH_LAUNCH_CHECK();
+        }
+        q0 += p->n_queries;
+        c0 += p->n_total_candidates;
+    }
+    return CULSH_OK;
+}
+
+// query over key words that are already in the arena
+static culsh_status query_keys(culsh_ctx* ctx, const uint32_t* q_keys, int nq, const culsh_index* ix,
+                               culsh_candidates* out) {
+    int32_t* matched = nullptr;
+    CULSH_TRY(arena_alloc_t(ctx, static_cast<size_t>(nq) * ix->n_hash_tables, &matched));
+    CULSH_TRY(launch_find_matching_buckets(ctx, q_keys, nq, ix, matched));
+    return query_from_matched(ctx, matched, nq, ix, out);
+}
+
+template <typename T>
+static culsh_status dense_query(culsh_ctx* ctx, Family fam, const T* Q, int nq, const culsh_index* ix,
+                                int batch_size, culsh_candidates** out) {
+    CULSH_REQUIRE(ctx && Q && ix && out, CULSH_ERR_INVALID, "null argument");
+    CULSH_REQUIRE(nq > 0, CULSH_ERR_INVALID, "n_queries must be positive");
+    CULSH_REQUIRE(ix->kind == (fam == FAM_RPLSH ? CULSH_KIND_RPLSH : CULSH_KIND_PSLSH), CULSH_ERR_INVALID,
+                  "index was built by a different hashing family");
+    const bool want_double = std::is_same_v<T, double>;
+    if (ix->is_double && !want_double) {
+        set_error("Index was fitted with float64, but query is float32");  // bindings.cu:58-60
+        return CULSH_ERR_INVALID;
+    }
+    if (!ix->is_double && want_double) {
+        set_error("Index was fitted with float32, but query is float64");  // bindings.cu:75-77
+        return CULSH_ERR_INVALID;
+    }
+    CULSH_REQUIRE(ix->P && (fam == FAM_RPLSH || ix->b), CULSH_ERR_INVALID, "index holds no hash parameters");
+    ArenaScope scope(ctx);
+    CULSH_TRY(scope.begin_status);
+    const int d = ix->n_features, nT = ix->n_hash_tables, H = ix->n_hashes;
+    if (batch_size <= 0 || batch_size >= nq) batch_size = nq;  // rplsh.cu:190-192
+    std::vector<CandPtr> parts;
+    for (int start = 0; start < nq; start += batch_size) {
+        const int bn = std::min(batch_size, nq - start);
+        const size_t mark = ctx->arena_off;
+        uint32_t* keys = nullptr;
+        int W = 0;
+        CULSH_TRY(hash_dense_to_keys<T>(ctx, fam, Q + static_cast<size_t>(start) * d, bn, d, nT, H, ix->P, ix->b,
+                                        &keys, &W));
+        CandPtr part(new (std::nothrow) culsh_candidates());
+        CULSH_REQUIRE(part, CULSH_ERR_NOMEM, "host allocation failed");
+        part->device = ctx->device;
+        CULSH_TRY(query_keys(ctx, keys, bn, ix, part.get()));
+        parts.push_back(std::move(part));
+        ctx->arena_off = mark;  // later kernels run after these on the same stream
+    }
+    if (parts.size() == 1) {
+        CULSH_TRY(arena_end(ctx));
+        *out = parts[0].release();
+        return CULSH_OK;
+    }
+    CandPtr result(new (std::nothrow) culsh_candidates());
+    CULSH_REQUIRE(result, CULSH_ERR_NOMEM, "host allocation failed");
+    result->device = ctx->device;
+    std::vector<culsh_candidates*> raw;
+    for (auto& p : parts) raw.push_back(p.get());
+    CULSH_TRY(concat_candidates(ctx, raw, result.get()));
+    CULSH_TRY(arena_end(ctx));  // parts are freed after the copies have run
+    *out = result.release();
+    return CULSH_OK;
+}
+
+// Shared tail of every fit: keys -> index (+ optional fit_query).
+static culsh_status finish_fit(culsh_ctx* ctx, uint32_t* keys, int n, int T, int H, int S, KeyEnc enc, int W,
+                               culsh_index* ix, culsh_candidates* cands_or_null) {
+    int32_t* item_to_bucket = nullptr;
+    if (cands_or_null) CULSH_TRY(arena_alloc_t(ctx, static_cast<size_t>(n) * T, &item_to_bucket));
+    CULSH_TRY(fit_index_from_keys(ctx, keys, n, T, H, S, enc, W, item_to_bucket, ix));
+    if (cands_or_null)  // core/fit_query.cuh:46-50
+        CULSH_TRY(query_from_matched(ctx, item_to_bucket, n, ix, cands_or_null));
+    return CULSH_OK;
+}
+
+template <typename T>
+static culsh_status dense_fit(culsh_ctx* ctx, Family fam, const T* X, int n, int d, int nT, int H, int window,
+                              uint64_t seed, const T* P_host, const T* b_host, culsh_index** index_out,
+                              culsh_candidates** cands_out) {
+    CULSH_TRY(check_fit_args(ctx, X, n, d, nT, H, index_out ? static_cast<void*>(index_out) : static_cast<void*>(cands_out)));
+    if (fam == FAM_PSLSH) {
+        CULSH_REQUIRE(window > 0, CULSH_ERR_INVALID, "window_size must be positive");
+        CULSH_REQUIRE((P_host == nullptr) == (b_host == nullptr), CULSH_ERR_INVALID,
+                      "projection and bias must be given together");
+    }
+    ArenaScope scope(ctx);
+    CULSH_TRY(scope.begin_status);
+    IndexPtr ix(new (std::nothrow) culsh_index());
+    CULSH_REQUIRE(ix, CULSH_ERR_NOMEM, "host allocation failed");
+    ix->device = ctx->device;
+    ix->kind = (fam == FAM_RPLSH) ? CULSH_KIND_RPLSH : CULSH_KIND_PSLSH;
+    ix->is_double = std::is_same_v<T, double>;
+    ix->window_size = (fam == FAM_PSLSH) ? window : 0;
+    const size_t TH = static_cast<size_t>(nT) * H;
+    {
+        std::vector<T> hp, hb;
+        if (!P_host) {
+            hp.resize(TH * d);
+            gen_projection<T>(seed, TH * d, fam == FAM_PSLSH ? window : 0, hp.data());
+            P_host = hp.data();
+            if (fam == FAM_PSLSH) {
+                hb.resize(TH);
+                gen_bias<T>(seed, TH, hb.data());
+                b_host = hb.data();
+            }
+        }
+        T* dP = nullptr;
+        CULSH_TRY(upload(P_host, TH * d, &dP));
+        ix->P = dP;
+        if (fam == FAM_PSLSH) {
+            T* db = nullptr;
+            CULSH_TRY(upload(b_host, TH, &db));
+            ix->b = db;
+        }
+    }
+    uint32_t* keys = nullptr;
+    int W = 0;
+    CULSH_TRY(hash_dense_to_keys<T>(ctx, fam, X, n, d, nT, H, ix->P, ix->b, &keys, &W));
+    const KeyEnc enc = (fam == FAM_RPLSH) ? ENC_BITS : ENC_BE;
+    const int S = (fam == FAM_RPLSH) ? H : 4 * H;  // rplsh.cu:37, pslsh.cu:39
+    CandPtr cands;
+    if (cands_out) {
+        cands.reset(new (std::nothrow) culsh_candidates());
+        CULSH_REQUIRE(cands, CULSH_ERR_NOMEM, "host allocation failed");
+        cands->device = ctx->device;
+    }
+    CULSH_TRY(finish_fit(ctx, keys, n, nT, H, S, enc, W, ix.get(), cands.get()));
+    ix->n_features = d;
+    ix->seed = seed;
+    CULSH_TRY(arena_end(ctx));
+    if (index_out) *index_out = ix.release();
+    if (cands_out) *cands_out = cands.release();  // the index (and P) is dropped, rplsh.cu:152-155
+    return CULSH_OK;
+}
+
+static culsh_status minhash_fit_impl(culsh_ctx* ctx, const int32_t* indices, const int32_t* indptr, int n, int d,
+                                     int nT, int H, uint64_t seed, const uint32_t* A_host, const uint32_t* B_host,
+                                     culsh_index** index_out, culsh_candidates** cands_out) {
+    CULSH_TRY(check_fit_args(ctx, indptr, n, d, nT, H, index_out ? static_cast<void*>(index_out) : static_cast<void*>(cands_out)));
+    CULSH_REQUIRE((A_host == nullptr) == (B_host == nullptr), CULSH_ERR_INVALID, "hash_a and hash_b must be given together");
+    ArenaScope scope(ctx);
+    CULSH_TRY(scope.begin_status);
+    IndexPtr ix(new (std::nothrow) culsh_index());
+    CULSH_REQUIRE(ix, CULSH_ERR_NOMEM, "host allocation failed");
+    ix->device = ctx->device;
+    ix->kind = CULSH_KIND_MINHASH;
+    const size_t TH = static_cast<size_t>(nT) * H;
+    {
+        std::vector<uint32_t> ha, hb;
+        if (!A_host) {
+            ha.resize(TH);
+            hb.resize(TH);
+            gen_minhash(seed, TH, ha.data(), hb.data());
+            A_host = ha.data();
+            B_host = hb.data();
+        }
+        CULSH_TRY(upload(A_host, TH, &ix->A));
+        CULSH_TRY(upload(B_host, TH, &ix->B));
+    }
+    const size_t N = static_cast<size_t>(n) * nT;
+    uint32_t* keys = nullptr;
+    CULSH_TRY(arena_alloc_t(ctx, N * H, &keys));
+    CULSH_TRY(launch_minhash(ctx, indices, indptr, ix->A, ix->B, n, nT, H, true, keys));
+    CandPtr cands;
+    if (cands_out) {
+        cands.reset(new (std::nothrow) culsh_candidates());
+        CULSH_REQUIRE(cands, CULSH_ERR_NOMEM, "host allocation failed");
+        cands->device = ctx->device;
+    }
+    CULSH_TRY(finish_fit(ctx, keys, n, nT, H, 4 * H, ENC_BE, H, ix.get(), cands.get()));  // minhash.cu:37
+    ix->n_features = d;
+    ix->seed = seed;
+    CULSH_TRY(arena_end(ctx));
+    if (index_out) *index_out = ix.release();
+    if (cands_out) *cands_out = cands.release();
+    return CULSH_OK;
+}
+
+static size_t elem_size_of(const culsh_index* ix, culsh_array which) {
+    switch (which) {
+        case CULSH_ARR_BUCKET_SIGNATURES: return 1;
+        case CULSH_ARR_PROJECTION:
+        case CULSH_ARR_BIAS: return ix->is_double ? 8 : 4;
+        default: return 4;
+    }
+}
+
+static culsh_status index_array(const culsh_index* ix, culsh_array which, const void** ptr, uint64_t* count) {
+    const uint64_t TH = static_cast<uint64_t>(ix->n_hash_tables) * ix->n_hashes;
+    switch (which) {
+        case CULSH_ARR_CANDIDATE_INDICES: *ptr = ix->all_candidate_indices; *count = ix->n_total_candidates; break;
+        case CULSH_ARR_BUCKET_SIGNATURES:
+            *ptr = ix->all_bucket_signatures;
+            *count = static_cast<uint64_t>(ix->n_total_buckets) * ix->sig_nbytes;
+            break;
+        case CULSH_ARR_BUCKET_CANDIDATE_OFFSETS:
+            *ptr = ix->bucket_candidate_offsets; *count = static_cast<uint64_t>(ix->n_total_buckets) + 1; break;
+        case CULSH_ARR_TABLE_BUCKET_OFFSETS:
+            *ptr = ix->table_bucket_offsets; *count = static_cast<uint64_t>(ix->n_hash_tables) + 1; break;
+        case CULSH_ARR_PROJECTION: *ptr = ix->P; *count = ix->P ? TH * ix->n_features : 0; break;
+        case CULSH_ARR_BIAS: *ptr = ix->b; *count = ix->b ? TH : 0; break;
+        case CULSH_ARR_HASH_A: *ptr = ix->A; *count = ix->A ? TH : 0; break;
+        case CULSH_ARR_HASH_B: *ptr = ix->B; *count = ix->B ? TH : 0; break;
+        default: set_error("not an index array: %d", static_cast<int>(which)); return CULSH_ERR_INVALID;
+    }
+    if (*ptr == nullptr) *count = 0;
+    return CULSH_OK;
+}
+
+}  // namespace culsh_amd
+
+using namespace culsh_amd;
+
+// ======================================================================================
+extern "C" {
+
+const char* culsh_last_error(void) { return g_last_error.c_str(); }
+const char* culsh_version(void) { return "culsh_amd 0.1.0 (gfx950)"; }
+
+culsh_status culsh_ctx_create(int device, culsh_ctx** out) {
+    CULSH_REQUIRE(out, CULSH_ERR_INVALID, "null argument");
+    *out = nullptr;
+    int count = 0;
+    CULSH_HIP(hipGetDeviceCount(&count));
+    CULSH_REQUIRE(device >= 0 && device < count, CULSH_ERR_INVALID, "device %d out of range (%d visible)", device, count);
+    CULSH_HIP(hipSetDevice(device));
+    std::unique_ptr<culsh_ctx> ctx(new (std::nothrow) culsh_ctx());
+    CULSH_REQUIRE(ctx, CULSH_ERR_NOMEM, "host allocation failed");
+    ctx->device = device;
+    hipDeviceProp_t prop;
+    CULSH_HIP(hipGetDeviceProperties(&prop, device));
+    CULSH_REQUIRE(std::strncmp(prop.gcnArchName, "gfx950", 6) == 0, CULSH_ERR_INVALID,
+                  "device %d is %s; this library is built for gfx950 only", device, prop.gcnArchName);
+    ctx->n_cus = prop.multiProcessorCount;
+    int lds_optin = 0;
+    if (hipDeviceGetAttribute(&lds_optin, hipDeviceAttributeMaxSharedMemoryPerBlock, device) != hipSuccess) {
+        (void)hipGetLastError();
+        lds_optin = 0;
+    }
+    ctx->lds_max = std::max<int>(static_cast<int>(prop.sharedMemPerBlock), lds_optin);
+    if (ctx->lds_max <= 0) ctx->lds_max = 65536;
+    CULSH_HIP(hipStreamCreate(&ctx->stream));  // default priority
+    void* pinned = nullptr;
+    if (hipHostMalloc(&pinned, 64 * sizeof(uint64_t), hipHostMallocDefault) != hipSuccess) {
+        (void)hipStreamDestroy(ctx->stream);
+        set_error("hipHostMalloc failed");
+        return CULSH_ERR_NOMEM;
+    }
+    ctx->pinned = static_cast<uint64_t*>(pinned);
+    *out = ctx.release();
+    return CULSH_OK;
+}
+
+void culsh_ctx_destroy(culsh_ctx* ctx) {
+    if (!ctx) return;
+    (void)hipSetDevice(ctx->device);
+    if (ctx->stream) {
+        (void)hipStreamSynchronize(ctx->stream);
+        (void)hipStreamDestroy(ctx->stream);
+    }
+    for (void* p : ctx->overflow) (void)hipFree(p);
+    if (ctx->arena) (void)hipFree(ctx->arena);
+    if (ctx->pinned) (void)hipHostFree(ctx->pinned);
+    delete ctx;
+}
+
+culsh_status culsh_ctx_synchronize(culsh_ctx* ctx) {
+    CULSH_REQUIRE(ctx, CULSH_ERR_INVALID, "null argument");
+    CULSH_HIP(hipStreamSynchronize(ctx->stream));
+    return CULSH_OK;
+}
+
+void* culsh_ctx_stream(culsh_ctx* ctx) { return ctx ? static_cast<void*>(ctx->stream) : nullptr; }
+
+// ---- generators
+culsh_status culsh_generate_projection_f32(uint64_t seed, int n_rows, int d, float* P) {
+    CULSH_REQUIRE(P && n_rows > 0 && d > 0, CULSH_ERR_INVALID, "bad argument");
+    gen_projection<float>(seed, static_cast<size_t>(n_rows) * d, 0, P);
+    return CULSH_OK;
+}
+culsh_status culsh_generate_projection_f64(uint64_t seed, int n_rows, int d, double* P) {
+    CULSH_REQUIRE(P && n_rows > 0 && d > 0, CULSH_ERR_INVALID, "bad argument");
+    gen_projection<double>(seed, static_cast<size_t>(n_rows) * d, 0, P);
+    return CULSH_OK;
+}
+culsh_status culsh_generate_pslsh_params_f32(uint64_t seed, int n_rows, int d, int w, float* P, float* b) {
+    CULSH_REQUIRE(P && b && n_rows > 0 && d > 0 && w > 0, CULSH_ERR_INVALID, "bad argument");
+    gen_projection<float>(seed, static_cast<size_t>(n_rows) * d, w, P);
+    gen_bias<float>(seed, n_rows, b);
+    return CULSH_OK;
+}
+culsh_status culsh_generate_pslsh_params_f64(uint64_t seed, int n_rows, int d, int w, double* P, double* b) {
+    CULSH_REQUIRE(P && b && n_rows > 0 && d > 0 && w > 0, CULSH_ERR_INVALID, "bad argument");
+    gen_projection<double>(seed, static_cast<size_t>(n_rows) * d, w, P);
+    gen_bias<double>(seed, n_rows, b);
+    return CULSH_OK;
+}
+culsh_status culsh_generate_minhash_params(uint64_t seed, int n_rows, uint32_t* A, uint32_t* B) {
+    CULSH_REQUIRE(A && B && n_rows > 0, CULSH_ERR_INVALID, "bad argument");
+    gen_minhash(seed, n_rows, A, B);
+    return CULSH_OK;
+}
+
+// ---- RPLSH
+culsh_status culsh_rplsh_fit_f32(culsh_ctx* ctx, const float* X, int n, int d, int T, int H, uint64_t seed,
+                                 const float* P, culsh_index** out) {
+    CULSH_REQUIRE(out, CULSH_ERR_INVALID, "null argument");
+    return dense_fit<float>(ctx, FAM_RPLSH, X, n, d, T, H, 0, seed, P, nullptr, out, nullptr);
+}
+culsh_status culsh_rplsh_fit_f64(culsh_ctx* ctx, const double* X, int n, int d, int T, int H, uint64_t seed,
+                                 const double* P, culsh_index** out) {
+    CULSH_REQUIRE(out, CULSH_ERR_INVALID, "null argument");
+    return dense_fit<double>(ctx, FAM_RPLSH, X, n, d, T, H, 0, seed, P, nullptr, out, nullptr);
+}
+culsh_status culsh_rplsh_query_f32(culsh_ctx* ctx, const float* Q, int nq, const culsh_index* ix, int batch,
+                                   culsh_candidates** out) {
+    return dense_query<float>(ctx, FAM_RPLSH, Q, nq, ix, batch, out);
+}
+culsh_status culsh_rplsh_query_f64(culsh_ctx* ctx, const double* Q, int nq, const culsh_index* ix, int batch,
+                                   culsh_candidates** out) {
+    return dense_query<double>(ctx, FAM_RPLSH, Q, nq, ix, batch, out);
+}
+culsh_status culsh_rplsh_fit_query_f32(culsh_ctx* ctx, const float* X, int n, int d, int T, int H, uint64_t seed,
+                                       const float* P, culsh_candidates** out) {
+    CULSH_REQUIRE(out, CULSH_ERR_INVALID, "null argument");
+    return dense_fit<float>(ctx, FAM_RPLSH, X, n, d, T, H, 0, seed, P, nullptr, nullptr, out);
+}
+culsh_status culsh_rplsh_fit_query_f64(culsh_ctx* ctx, const double* X, int n, int d, int T, int H, uint64_t seed,
+                                       const double* P, culsh_candidates** out) {
+    CULSH_REQUIRE(out, CULSH_ERR_INVALID, "null argument");
+    return dense_fit<double>(ctx, FAM_RPLSH, X, n, d, T, H, 0, seed, P, nullptr, nullptr, out);
+}
+
+// ---- p-stable
+culsh_status culsh_pslsh_fit_f32(culsh_ctx* ctx, const float* X, int n, int d, int T, int H, int w, uint64_t seed,
+                                 const float* P, const float* b, culsh_index** out) {
+    CULSH_REQUIRE(out, CULSH_ERR_INVALID, "null argument");
+    return dense_fit<float>(ctx, FAM_PSLSH, X, n, d, T, H, w, seed, P, b, out, nullptr);
+}
+culsh_status culsh_pslsh_fit_f64(culsh_ctx* ctx, const double* X, int n, int d, int T, int H, int w, uint64_t seed,
+                                 const double* P, const double* b, culsh_index** out) {
+    CULSH_REQUIRE(out, CULSH_ERR_INVALID, "null argument");
+    return dense_fit<double>(ctx, FAM_PSLSH, X, n, d, T, H, w, seed, P, b, out, nullptr);
+}
+culsh_status culsh_pslsh_query_f32(culsh_ctx* ctx, const float* Q, int nq, const culsh_index* ix, int batch,
+                                   culsh_candidates** out) {
+    return dense_query<float>(ctx, FAM_PSLSH, Q, nq, ix, batch, out);
+}
+culsh_status culsh_pslsh_query_f64(culsh_ctx* ctx, const double* Q, int nq, const culsh_index* ix, int batch,
+                                   culsh_candidates** out) {
+    return dense_query<double>(ctx, FAM_PSLSH, Q, nq, ix, batch, out);
+}
+culsh_status culsh_pslsh_fit_query_f32(culsh_ctx* ctx, const float* X, int n, int d, int T, int H, int w,
+                                       uint64_t seed, const float* P, const float* b, culsh_candidates** out) {
+    CULSH_REQUIRE(out, CULSH_ERR_INVALID, "null argument");
+    return dense_fit<float>(ctx, FAM_PSLSH, X, n, d, T, H, w, seed, P, b, nullptr, out);
+}
+culsh_status culsh_pslsh_fit_query_f64(culsh_ctx* ctx, const double* X, int n, int d, int T, int H, int w,
+                                       uint64_t seed, const double* P, const double* b, culsh_candidates** out) {
+    CULSH_REQUIRE(out, CULSH_ERR_INVALID, "null argument");
+    return dense_fit<double>(ctx, FAM_PSLSH, X, n, d, T, H, w, seed, P, b, nullptr, out);
+}
+
+// ---- MinHash
+culsh_status culsh_minhash_fit(culsh_ctx* ctx, const int32_t* indices, const int32_t* indptr, int n, int d, int T,
+                               int H, uint64_t seed, const uint32_t* A, const uint32_t* B, culsh_index** out) {
+    CULSH_REQUIRE(out, CULSH_ERR_INVALID, "null argument");
+    return minhash_fit_impl(ctx, indices, indptr, n, d, T, H, seed, A, B, out, nullptr);
+}
+culsh_status culsh_minhash_fit_query(culsh_ctx* ctx, const int32_t* indices, const int32_t* indptr, int n, int d,
+                                     int T, int H, uint64_t seed, const uint32_t* A, const uint32_t* B,
+                                     culsh_candidates** out) {
+    CULSH_REQUIRE(out, CULSH_ERR_INVALID, "null argument");
+    return minhash_fit_impl(ctx, indices, indptr, n, d, T, H, seed, A, B, nullptr, out);
+}
+culsh_status culsh_minhash_query(culsh_ctx* ctx, const int32_t* indices, const int32_t* indptr, int nq,
+                                 const culsh_index* ix, culsh_candidates** out) {
+    CULSH_REQUIRE(ctx && indptr && ix && out, CULSH_ERR_INVALID, "null argument");
+    CULSH_REQUIRE(nq > 0, CULSH_ERR_INVALID, "n_queries must be positive");
+    CULSH_REQUIRE(ix->kind == CULSH_KIND_MINHASH && ix->A && ix->B, CULSH_ERR_INVALID, "not a MinHash index");
+    ArenaScope scope(ctx);
+    CULSH_TRY(scope.begin_status);
+    const int T = ix->n_hash_tables, H = ix->n_hashes;
+    uint32_t* keys = nullptr;
+    CULSH_TRY(arena_alloc_t(ctx, static_cast<size_t>(nq) * T * H, &keys));
+    CULSH_TRY(launch_minhash(ctx, indices, indptr, ix->A, ix->B, nq, T, H, true, keys));
+    CandPtr c(new (std::nothrow) culsh_candidates());
+    CULSH_REQUIRE(c, CULSH_ERR_NOMEM, "host allocation failed");
+    c->device = ctx->device;
+    CULSH_TRY(query_keys(ctx, keys, nq, ix, c.get()));
+    CULSH_TRY(arena_end(ctx));
+    *out = c.release();
+    return CULSH_OK;
+}
+
+// ---- stage level
+#define STAGE_PROLOGUE()                                   \
+    CULSH_REQUIRE(ctx, CULSH_ERR_INVALID, "null argument"); \
+    ArenaScope scope(ctx);                                  \
+    CULSH_TRY(scope.begin_status)
+
+culsh_status culsh_rplsh_hash_f32(culsh_ctx* ctx, const float* X, const float* P, int n, int d, int T, int H,
+                                  uint8_t* sig) {
+    STAGE_PROLOGUE();
+    CULSH_TRY(launch_project_f32(ctx, X, P, nullptr, n, d, T, H, EPI_SIGN_BYTES, sig));
+    return arena_end(ctx);
+}
+culsh_status culsh_rplsh_hash_f64(culsh_ctx* ctx, const double* X, const double* P, int n, int d, int T, int H,
+                                  uint8_t* sig) {
+    STAGE_PROLOGUE();
+    CULSH_TRY(launch_project_f64(ctx, X, P, nullptr, n, d, T, H, EPI_SIGN_BYTES, sig));
+    return arena_end(ctx);
+}
+culsh_status culsh_pslsh_hash_f32(culsh_ctx* ctx, const float* X, const float* P, const float* b, int n, int d,
+                                  int T, int H, int32_t* sig) {
+    STAGE_PROLOGUE();
+    CULSH_TRY(launch_project_f32(ctx, X, P, b, n, d, T, H, EPI_FLOOR_I32, sig));
+    return arena_end(ctx);
+}
+culsh_status culsh_pslsh_hash_f64(culsh_ctx* ctx, const double* X, const double* P, const double* b, int n, int d,
+                                  int T, int H, int32_t* sig) {
+    STAGE_PROLOGUE();
+    CULSH_TRY(launch_project_f64(ctx, X, P, b, n, d, T, H, EPI_FLOOR_I32, sig));
+    return arena_end(ctx);
+}
+culsh_status culsh_minhash_compute(culsh_ctx* ctx, const int32_t* indices, const int32_t* indptr, const uint32_t* A,
+                                   const uint32_t* B, int n, int T, int H, uint32_t* sig) {
+    STAGE_PROLOGUE();
+    CULSH_TRY(launch_minhash(ctx, indices, indptr, A, B, n, T, H, false, sig));
+    return arena_end(ctx);
+}
+
+culsh_status culsh_core_fit_index(culsh_ctx* ctx, const void* X_sig, int n, int T, int H, int S,
+                                  int32_t* item_to_bucket, culsh_index** out) {
+    CULSH_TRY(check_fit_args(ctx, X_sig, n, 1, T, H, out));
+    CULSH_REQUIRE(S > 0, CULSH_ERR_INVALID, "sig_nbytes must be > 0");  // core/fit.cuh:224
+    CULSH_REQUIRE(S <= 256, CULSH_ERR_LIMIT, "sig_nbytes > 256 is not supported");
+    ArenaScope scope(ctx);
+    CULSH_TRY(scope.begin_status);
+    IndexPtr ix(new (std::nothrow) culsh_index());
+    CULSH_REQUIRE(ix, CULSH_ERR_NOMEM, "host allocation failed");
+    ix->device = ctx->device;
+    const int W = key_words(ENC_BE, S);
+    uint32_t* keys = nullptr;
+    CULSH_TRY(arena_alloc_t(ctx, static_cast<size_t>(n) * T * W, &keys));
+    CULSH_TRY(launch_sig_to_keys(ctx, static_cast<const uint8_t*>(X_sig), static_cast<size_t>(n) * T, S, ENC_BE, W, keys));
+    CULSH_TRY(fit_index_from_keys(ctx, keys, n, T, H, S, ENC_BE, W, item_to_bucket, ix.get()));
+    CULSH_TRY(arena_end(ctx));
+    *out = ix.release();
+    return CULSH_OK;
+}
+
+static culsh_status sig_query_keys(culsh_ctx* ctx, const void* Q_sig, int nq, int S, const culsh_index* ix,
+                                   uint32_t** keys) {
+    CULSH_REQUIRE(ctx && Q_sig && ix, CULSH_ERR_INVALID, "null argument");
+    CULSH_REQUIRE(nq > 0, CULSH_ERR_INVALID, "n_queries must be positive");
+    CULSH_REQUIRE(S == ix->sig_nbytes, CULSH_ERR_INVALID, "sig_nbytes (%d) != index sig_nbytes (%d)", S,
+                  ix->sig_nbytes);  // core/query.cuh:494
+    CULSH_TRY(arena_alloc_t(ctx, static_cast<size_t>(nq) * ix->n_hash_tables * ix->key_w, keys));
+    return launch_sig_to_keys(ctx, static_cast<const uint8_t*>(Q_sig), static_cast<size_t>(nq) * ix->n_hash_tables,
+                              S, ix->enc, ix->key_w, *keys);
+}
+
+culsh_status culsh_core_find_matching_buckets(culsh_ctx* ctx, const void* Q_sig, int nq, int S,
+                                              const culsh_index* ix, int32_t* matched) {
+    CULSH_REQUIRE(ctx && matched, CULSH_ERR_INVALID, "null argument");
+    ArenaScope scope(ctx);
+    CULSH_TRY(scope.begin_status);
+    uint32_t* keys = nullptr;
+    CULSH_TRY(sig_query_keys(ctx, Q_sig, nq, S, ix, &keys));
+    CULSH_TRY(launch_find_matching_buckets(ctx, keys, nq, ix, matched));
+    return arena_end(ctx);
+}
+
+culsh_status culsh_core_query_index(culsh_ctx* ctx, const void* Q_sig, int nq, int S, const culsh_index* ix,
+                                    culsh_candidates** out) {
+    CULSH_REQUIRE(ctx && out, CULSH_ERR_INVALID, "null argument");
+    ArenaScope scope(ctx);
+    CULSH_TRY(scope.begin_status);
+    uint32_t* keys = nullptr;
+    CULSH_TRY(sig_query_keys(ctx, Q_sig, nq, S, ix, &keys));
+    CandPtr c(new (std::nothrow) culsh_candidates());
+    CULSH_REQUIRE(c, CULSH_ERR_NOMEM, "host allocation failed");
+    c->device = ctx->device;
+    CULSH_TRY(query_keys(ctx, keys, nq, ix, c.get()));
+    CULSH_TRY(arena_end(ctx));
+    *out = c.release();
+    return CULSH_OK;
+}
+
+culsh_status culsh_core_query_from_matched_buckets(culsh_ctx* ctx, const int32_t* matched, int nq,
+                                                   const culsh_index* ix, culsh_candidates** out) {
+    CULSH_REQUIRE(ctx && matched && ix && out, CULSH_ERR_INVALID, "null argument");
+    ArenaScope scope(ctx);
+    CULSH_TRY(scope.begin_status);
+    CandPtr c(new (std::nothrow) culsh_candidates());
+    CULSH_REQUIRE(c, CULSH_ERR_NOMEM, "host allocation failed");
+    c->device = ctx->device;
+    CULSH_TRY(query_from_matched(ctx, matched, nq, ix, c.get()));
+    CULSH_TRY(arena_end(ctx));
+    *out = c.release();
+    return CULSH_OK;
+}
+
+culsh_status culsh_core_fit_query(culsh_ctx* ctx, const void* X_sig, int n, int T, int H, int S,
+                                  culsh_candidates** out) {
+    CULSH_TRY(check_fit_args(ctx, X_sig, n, 1, T, H, out));
+    CULSH_REQUIRE(S > 0 && S <= 256, CULSH_ERR_INVALID, "sig_nbytes must be in [1, 256]");
+    ArenaScope scope(ctx);
+    CULSH_TRY(scope.begin_status);
+    IndexPtr ix(new (std::nothrow) culsh_index());
+    CandPtr c(new (std::nothrow) culsh_candidates());
+    CULSH_REQUIRE(ix && c, CULSH_ERR_NOMEM, "host allocation failed");
+    ix->device = c->device = ctx->device;
+    const int W = key_words(ENC_BE, S);
+    uint32_t* keys = nullptr;
+    CULSH_TRY(arena_alloc_t(ctx, static_cast<size_t>(n) * T * W, &keys));
+    CULSH_TRY(launch_sig_to_keys(ctx, static_cast<const uint8_t*>(X_sig), static_cast<size_t>(n) * T, S, ENC_BE, W, keys));
+    CULSH_TRY(finish_fit(ctx, keys, n, T, H, S, ENC_BE, W, ix.get(), c.get()));
+    CULSH_TRY(arena_end(ctx));
+    *out = c.release();
+    return CULSH_OK;
+}
+
+// ---- index object
+culsh_status culsh_index_get_meta(const culsh_index* ix, culsh_index_meta* m) {
+    CULSH_REQUIRE(ix && m, CULSH_ERR_INVALID, "null argument");
+    m->kind = ix->kind;
+    m->n_total_candidates = ix->n_total_candidates;
+    m->n_total_buckets = ix->n_total_buckets;
+    m->n_hash_tables = ix->n_hash_tables;
+    m->n_hashes = ix->n_hashes;
+    m->sig_nbytes = ix->sig_nbytes;
+    m->n_features = ix->n_features;
+    m->is_double = ix->is_double ? 1 : 0;
+    m->window_size = ix->window_size;
+    m->seed = ix->seed;
+    // Index::size_bytes (core/index.cuh:148-165) + family arrays (rplsh/index.cuh:45-53 etc.)
+    uint64_t sz = 0;
+    const bool core_empty = !ix->all_candidate_indices && !ix->all_bucket_signatures &&
+                            !ix->bucket_candidate_offsets && !ix->table_bucket_offsets;
+    if (!core_empty) {
+        sz += (static_cast<uint64_t>(ix->n_total_buckets) + 1) * 4 + (static_cast<uint64_t>(ix->n_hash_tables) + 1) * 4;
+        sz += static_cast<uint64_t>(ix->n_total_buckets) * ix->sig_nbytes;
+        sz += static_cast<uint64_t>(ix->n_total_candidates) * 4;
+    }
+    const uint64_t TH = static_cast<uint64_t>(ix->n_hash_tables) * ix->n_hashes;
+    const uint64_t fsz = ix->is_double ? 8 : 4;
+    if (ix->P && ix->n_features > 0) sz += TH * ix->n_features * fsz;
+    if (ix->b) sz += TH * fsz;
+    if (ix->A) sz += TH * 4;
+    if (ix->B) sz += TH * 4;
+    m->size_bytes = sz;
+    return CULSH_OK;
+}
+
+culsh_status culsh_index_array_info(const culsh_index* ix, culsh_array which, uint64_t* n_elems, uint32_t* elem_size) {
+    CULSH_REQUIRE(ix && n_elems && elem_size, CULSH_ERR_INVALID, "null argument");
+    const void* p = nullptr;
+    CULSH_TRY(index_array(ix, which, &p, n_elems));
+    *elem_size = static_cast<uint32_t>(elem_size_of(ix, which));
+    return CULSH_OK;
+}
+
+culsh_status culsh_index_copy_array(culsh_ctx* ctx, const culsh_index* ix, culsh_array which, void* dst,
+                                    uint64_t dst_bytes, int dst_is_device) {
+    CULSH_REQUIRE(ctx && ix, CULSH_ERR_INVALID, "null argument");
+    const void* p = nullptr;
+    uint64_t count = 0;
+    CULSH_TRY(index_array(ix, which, &p, &count));
+    const uint64_t bytes = count * elem_size_of(ix, which);
+    CULSH_REQUIRE(dst_bytes >= bytes, CULSH_ERR_INVALID, "destination too small (%llu < %llu bytes)",
+                  static_cast<unsigned long long>(dst_bytes), static_cast<unsigned long long>(bytes));
+    if (bytes == 0) return CULSH_OK;
+    CULSH_REQUIRE(dst, CULSH_ERR_INVALID, "null destination");
+    CULSH_HIP(hipSetDevice(ctx->device));
+    CULSH_HIP(hipMemcpy(dst, p, bytes, dst_is_device ? hipMemcpyDeviceToDevice : hipMemcpyDeviceToHost));
+    return CULSH_OK;
+}
+
+culsh_status culsh_index_load(culsh_ctx* ctx, culsh_kind kind, int is_double, const int32_t* cand,
+                              const uint8_t* bsig, const int32_t* bco, const int32_t* tbo, const void* param0,
+                              const void* param1, int n_total_candidates, int n_total_buckets, int T, int H, int S,
+                              int d, uint64_t seed, culsh_index** out) {
+    CULSH_REQUIRE(ctx && out, CULSH_ERR_INVALID, "null argument");
+    CULSH_REQUIRE(kind == CULSH_KIND_RPLSH || kind == CULSH_KIND_PSLSH || kind == CULSH_KIND_MINHASH ||
+                      kind == CULSH_KIND_CORE, CULSH_ERR_INVALID, "unknown index kind");
+    CULSH_REQUIRE(n_total_candidates >= 0 && n_total_buckets >= 0 && T > 0 && H > 0 && S > 0 && d >= 0,
+                  CULSH_ERR_INVALID, "bad index metadata");
+    CULSH_REQUIRE(S <= 256, CULSH_ERR_LIMIT, "sig_nbytes > 256 is not supported");
+    CULSH_REQUIRE((n_total_candidates == 0 || cand) && (n_total_buckets == 0 || bsig) && bco && tbo,
+                  CULSH_ERR_INVALID, "missing index array");
+    KeyEnc enc = ENC_BE;
+    if (kind == CULSH_KIND_RPLSH) {
+        CULSH_REQUIRE(S == H, CULSH_ERR_INVALID, "RPLSH signatures hold one byte per hash (sig_nbytes == n_hashes)");
+        const size_t nb = static_cast<size_t>(n_total_buckets) * S;
+        for (size_t i = 0; i < nb; ++i)
+            CULSH_REQUIRE(bsig[i] <= 1, CULSH_ERR_INVALID, "RPLSH bucket signatures must hold 0/1 bytes");
+        enc = ENC_BITS;
+    } else if (kind != CULSH_KIND_CORE) {
+        CULSH_REQUIRE(S == 4 * H, CULSH_ERR_INVALID, "sig_nbytes must be 4 * n_hashes for this family");
+    }
+    ArenaScope scope(ctx);
+    CULSH_TRY(scope.begin_status);
+    IndexPtr ix(new (std::nothrow) culsh_index());
+    CULSH_REQUIRE(ix, CULSH_ERR_NOMEM, "host allocation failed");
+    ix->device = ctx->device;
+    ix->kind = kind;
+    ix->is_double = is_double != 0;
+    ix->n_total_candidates = n_total_candidates;
+    ix->n_total_buckets = n_total_buckets;
+    ix->n_hash_tables = T;
+    ix->n_hashes = H;
+    ix->sig_nbytes = S;
+    ix->n_features = d;
+    ix->seed = seed;
+    ix->enc = enc;
+    ix->key_w = key_words(enc, S);
+    CULSH_TRY(upload(cand, static_cast<size_t>(n_total_candidates), &ix->all_candidate_indices));
+    CULSH_TRY(upload(bsig, static_cast<size_t>(n_total_buckets) * S, &ix->all_bucket_signatures));
+    CULSH_TRY(upload(bco, static_cast<size_t>(n_total_buckets) + 1, &ix->bucket_candidate_offsets));
+    CULSH_TRY(upload(tbo, static_cast<size_t>(T) + 1, &ix->table_bucket_offsets));
+    const size_t TH = static_cast<size_t>(T) * H;
+    if (kind == CULSH_KIND_RPLSH || kind == CULSH_KIND_PSLSH) {
+        CULSH_REQUIRE(param0, CULSH_ERR_INVALID, "projection is required");
+        if (ix->is_double) {
+            double* p = nullptr;
+            CULSH_TRY(upload(static_cast<const double*>(param0), TH * d, &p));
+            ix->P = p;
+        } else {
+            float* p = nullptr;
+            CULSH_TRY(upload(static_cast<const float*>(param0), TH * d, &p));
+            ix->P = p;
+        }
+        if (kind == CULSH_KIND_PSLSH) {
+            CULSH_REQUIRE(param1, CULSH_ERR_INVALID, "bias is required");
+            if (ix->is_double) {
+                double* p = nullptr;
+                CULSH_TRY(upload(static_cast<const double*>(param1), TH, &p));
+                ix->b = p;
+            } else {
+                float* p = nullptr;
+                CULSH_TRY(upload(static_cast<const float*>(param1), TH, &p));
+                ix->b = p;
+            }
+        }
+    } else if (kind == CULSH_KIND_MINHASH) {
+        CULSH_REQUIRE(param0 && param1, CULSH_ERR_INVALID, "hash_a and hash_b are required");
+        CULSH_TRY(upload(static_cast<const uint32_t*>(param0), TH, &ix->A));
+        CULSH_TRY(upload(static_cast<const uint32_t*>(param1), TH, &ix->B));
+    }
+    CULSH_HIP(hipMalloc(&ix->bucket_keys, std::max<size_t>(1, static_cast<size_t>(n_total_buckets) * ix->key_w) * 4));
+    CULSH_TRY(launch_sig_to_keys(ctx, ix->all_bucket_signatures, n_total_buckets, S, enc, ix->key_w, ix->bucket_keys));
+    CULSH_TRY(arena_end(ctx));
+    *out = ix.release();
+    return CULSH_OK;
+}
+
+void culsh_index_free(culsh_index* ix) {
+    if (!ix) return;
+    (void)hipSetDevice(ix->device);
+    free_index_arrays(ix);
+    delete ix;
+}
+
+// ---- candidates object
+culsh_status culsh_candidates_get_meta(const culsh_candidates* c, culsh_candidates_meta* m) {
+    CULSH_REQUIRE(c && m, CULSH_ERR_INVALID, "null argument");
+    m->n_queries = c->n_queries;
+    m->n_total_candidates = c->n_total_candidates;
+    m->is_empty = (!c->query_candidate_indices && !c->query_candidate_counts && !c->query_candidate_offsets) ? 1 : 0;
+    return CULSH_OK;
+}
+
+static culsh_status cand_array(const culsh_candidates* c, culsh_array which, const void** p, uint64_t* bytes) {
+    switch (which) {
+        case CULSH_ARR_QUERY_INDICES: *p = c->query_candidate_indices; *bytes = c->n_total_candidates * 4; break;
+        case CULSH_ARR_QUERY_COUNTS: *p = c->query_candidate_counts; *bytes = static_cast<uint64_t>(c->n_queries) * 8; break;
+        case CULSH_ARR_QUERY_OFFSETS:
+            *p = c->query_candidate_offsets; *bytes = (static_cast<uint64_t>(c->n_queries) + 1) * 8; break;
+        default: set_error("not a candidates array: %d", static_cast<int>(which)); return CULSH_ERR_INVALID;
+    }
+    if (*p == nullptr) *bytes = 0;
+    return CULSH_OK;
+}
+
+culsh_status culsh_candidates_copy_array(culsh_ctx* ctx, const culsh_candidates* c, culsh_array which, void* dst,
+                                         uint64_t dst_bytes, int dst_is_device) {
+    CULSH_REQUIRE(ctx && c, CULSH_ERR_INVALID, "null argument");
+    const void* p = nullptr;
+    uint64_t bytes = 0;
+    CULSH_TRY(cand_array(c, which, &p, &bytes));
+    CULSH_REQUIRE(dst_bytes >= bytes, CULSH_ERR_INVALID, "destination too small");
+    if (bytes == 0) return CULSH_OK;
+    CULSH_REQUIRE(dst, CULSH_ERR_INVALID, "null destination");
+    CULSH_HIP(hipSetDevice(ctx->device));
+    CULSH_HIP(hipMemcpy(dst, p, bytes, dst_is_device ? hipMemcpyDeviceToDevice : hipMemcpyDeviceToHost));
+    return CULSH_OK;
+}
+
+const void* culsh_candidates_device_ptr(const culsh_candidates* c, culsh_array which) {
+    if (!c) return nullptr;
+    const void* p = nullptr;
+    uint64_t bytes = 0;
+    if (cand_array(c, which, &p, &bytes) != CULSH_OK) return nullptr;
+    return p;
+}
+
+culsh_status culsh_candidates_merge(culsh_ctx* ctx, culsh_candidates** acc, culsh_candidates* other) {
+    CULSH_REQUIRE(ctx && acc, CULSH_ERR_INVALID, "null argument");
+    if (!other) return CULSH_OK;
+    const bool other_empty = !other->query_candidate_indices && !other->query_candidate_counts &&
+                             !other->query_candidate_offsets;
+    if (other_empty) {  // candidates.cuh:140-142
+        culsh_candidates_free(other);
+        return CULSH_OK;
+    }
+    culsh_candidates* a = *acc;
+    const bool acc_empty = !a || (!a->query_candidate_indices && !a->query_candidate_counts &&
+                                  !a->query_candidate_offsets);
+    if (acc_empty) {  // candidates.cuh:144-148
+        if (a) culsh_candidates_free(a);
+        *acc = other;
+        return CULSH_OK;
+    }
+    ArenaScope scope(ctx);
+    CULSH_TRY(scope.begin_status);
+    CandPtr result(new (std::nothrow) culsh_candidates());
+    CULSH_REQUIRE(result, CULSH_ERR_NOMEM, "host allocation failed");
+    result->device = ctx->device;
+    CULSH_TRY(concat_candidates(ctx, {a, other}, result.get()));
+    CULSH_TRY(arena_end(ctx));
+    culsh_candidates_free(a);
+    culsh_candidates_free(other);
+    *acc = result.release();
+    return CULSH_OK;
+}
+
+void culsh_candidates_free(culsh_candidates* c) {
+    if (!c) return;
+    (void)hipSetDevice(c->device);
+    free_candidates_arrays(c);
+    delete c;
+}
+
+}  // extern "C"

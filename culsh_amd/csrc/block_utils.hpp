@@ -1,0 +1,53 @@
+// Wavefront (64 lanes) and workgroup scan / reduce helpers for gfx950 kernels.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+
+namespace culsh_amd {
+
+constexpr int WAVE = 64;
+
+template <typename T>
+__device__ __forceinline__ T wave_inclusive_sum(T v) {
+    const int lane = threadIdx.x & (WAVE - 1);
+#pragma unroll
+    for (int d = 1; d < WAVE; d <<= 1) {
+        const T o = __shfl_up(v, d, WAVE);
+        if (lane >= d) v += o;
+    }
+    return v;
+}
+
+template <typename T>
+__device__ __forceinline__ T wave_sum(T v) {
+#pragma unroll
+    for (int d = WAVE / 2; d > 0; d >>= 1) v += __shfl_xor(v, d, WAVE);
+    return v;
+}
+
+// Exclusive prefix sum over the workgroup (blockDim.x a multiple of 64, at most 1024).
+// `scratch` holds 17 words of type T in LDS.  Returns this thread's exclusive prefix and
+// stores the workgroup total in *total.  Contains three barriers; all threads must call it.
+template <typename T>
+__device__ __forceinline__ T block_exclusive_sum(T v, T* scratch, T* total) {
+    const int lane = threadIdx.x & (WAVE - 1), wave = threadIdx.x >> 6;
+    const int nwaves = (blockDim.x + WAVE - 1) >> 6;
+    const T incl = wave_inclusive_sum(v);
+    if (lane == WAVE - 1) scratch[wave] = incl;
+    __syncthreads();
+    if (wave == 0) {
+        T w = (lane < nwaves) ? scratch[lane] : T(0);
+        const T wi = wave_inclusive_sum(w);
+        if (lane < nwaves) scratch[lane] = wi - w;  // exclusive wave offsets
+        if (lane == nwaves - 1) scratch[16] = wi;   // total
+    }
+    __syncthreads();
+    const T res = scratch[wave] + incl - v;
+    *total = scratch[16];
+    __syncthreads();  // scratch may be reused by the next call
+    return res;
+}
+
+}  // namespace culsh_amd

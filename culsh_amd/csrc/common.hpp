@@ -1,0 +1,204 @@
+// Internal definitions shared by the HIP translation units of libculsh_amd.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdint>
+#include <cstdio>
+#include <string>
+#include <vector>
+
+#include "../../include/culsh_amd.h"
+
+namespace culsh_amd {
+
+// ---------------------------------------------------------------- errors
+void set_error(const char* fmt, ...);
+
+struct Status {
+    culsh_status code = CULSH_OK;
+    bool ok() const { return code == CULSH_OK; }
+};
+
+#define CULSH_HIP(call)                                                                   \
+    do {                                                                                  \
+        hipError_t e_ = (call);                                                           \
+        if (e_ != hipSuccess) {                                                           \
+            ::culsh_amd::set_error("%s failed: %s (%s:%d)", #call, hipGetErrorString(e_), \
+                                   __FILE__, __LINE__);                                   \
+            return (e_ == hipErrorOutOfMemory) ? CULSH_ERR_NOMEM : CULSH_ERR_HIP;         \
+        }                                                                                 \
+    } while (0)
+
+#define CULSH_TRY(expr)                    \
+    do {                                   \
+        culsh_status s_ = (expr);          \
+        if (s_ != CULSH_OK) return s_;     \
+    } while (0)
+
+#define CULSH_REQUIRE(cond, code, ...)         \
+    do {                                       \
+        if (!(cond)) {                         \
+            ::culsh_amd::set_error(__VA_ARGS__); \
+            return (code);                     \
+        }                                      \
+    } while (0)
+
+// Checks the launch itself (bad configuration); execution errors surface at the next sync.
+#define CULSH_LAUNCH_CHECK() CULSH_HIP(hipGetLastError())
+
+// ---------------------------------------------------------------- key encodings
+// Signatures are opaque byte strings ordered lexicographically (unsigned bytes, byte 0
+// most significant).  Internally every signature is held as `W` 32-bit key words whose
+// unsigned word-lexicographic order is that byte order:
+//   ENC_BE   word w = big-endian load of signature bytes [4w, 4w+4), zero padded
+//   ENC_BITS (signatures made of 0/1 bytes) hash h -> bit (31 - h%32) of word h/32
+enum KeyEnc : int { ENC_BE = 0, ENC_BITS = 1 };
+
+inline int key_words(KeyEnc enc, int sig_nbytes) {
+    return enc == ENC_BITS ? (sig_nbytes + 31) / 32 : (sig_nbytes + 3) / 4;
+}
+
+}  // namespace culsh_amd
+
+// ---------------------------------------------------------------- opaque objects
+struct culsh_ctx {
+    int device = 0;
+    hipStream_t stream = nullptr;
+    // scratch arena (bump allocated per call, grown between calls)
+    char* arena = nullptr;
+    size_t arena_cap = 0;
+    size_t arena_off = 0;
+    size_t arena_want = 0;               // high-water mark incl. overflow blocks
+    std::vector<void*> overflow;         // freed at the end of the call
+    uint64_t* pinned = nullptr;          // 64 x u64 pinned host words for D2H scalars
+    int lds_max = 0;                     // max LDS bytes per workgroup
+    int n_cus = 0;
+};
+
+struct culsh_index {
+    // core::Index (core/index.cuh:12-40)
+    int32_t* all_candidate_indices = nullptr;
+    uint8_t* all_bucket_signatures = nullptr;
+    int32_t* bucket_candidate_offsets = nullptr;
+    int32_t* table_bucket_offsets = nullptr;
+    int n_total_candidates = 0, n_total_buckets = 0, n_hash_tables = 0, n_hashes = 0;
+    int sig_nbytes = 0, n_features = 0;
+    uint64_t seed = 0;
+    // sort-order form of the bucket signatures: uint32 [n_total_buckets][key_w]
+    uint32_t* bucket_keys = nullptr;
+    culsh_amd::KeyEnc enc = culsh_amd::ENC_BE;
+    int key_w = 0;
+    // family parameters (device): rplsh/index.cuh, pslsh/index.cuh, minhash/index.cuh
+    culsh_kind kind = CULSH_KIND_CORE;
+    bool is_double = false;
+    int window_size = 0;
+    void* P = nullptr;    // [T*H][d] f32/f64
+    void* b = nullptr;    // [T*H] f32/f64
+    uint32_t* A = nullptr;
+    uint32_t* B = nullptr;
+    int device = 0;
+};
+
+struct culsh_candidates {
+    // core::Candidates (core/candidates.cuh:14-40)
+    int32_t* query_candidate_indices = nullptr;
+    uint64_t* query_candidate_counts = nullptr;
+    uint64_t* query_candidate_offsets = nullptr;
+    int n_queries = 0;
+    uint64_t n_total_candidates = 0;
+    int device = 0;
+};
+
+namespace culsh_amd {
+
+// ---------------------------------------------------------------- scratch arena
+culsh_status arena_begin(culsh_ctx* ctx);                 // start of an API call
+culsh_status arena_alloc(culsh_ctx* ctx, size_t bytes, void** out);
+culsh_status arena_end(culsh_ctx* ctx);                   // syncs the stream, frees overflow
+template <typename T>
+inline culsh_status arena_alloc_t(culsh_ctx* ctx, size_t count, T** out) {
+    void* p = nullptr;
+    culsh_status s = arena_alloc(ctx, count * sizeof(T), &p);
+    *out = static_cast<T*>(p);
+    return s;
+}
+// RAII: arena_begin at construction, arena_end at scope exit.
+struct ArenaScope {
+    culsh_ctx* ctx;
+    culsh_status begin_status;
+    explicit ArenaScope(culsh_ctx* c) : ctx(c), begin_status(arena_begin(c)) {}
+    ~ArenaScope() { arena_end(ctx); }
+};
+
+// Reads `count` (<= 64) device u64/u32 words into host memory; synchronises the stream.
+culsh_status read_back_u64(culsh_ctx* ctx, const uint64_t* dev, int count, uint64_t* host);
+culsh_status read_back_u32(culsh_ctx* ctx, const uint32_t* dev, int count, uint32_t* host);
+
+// ---------------------------------------------------------------- projection (project.hip)
+// Output modes of the projection kernels.
+enum ProjEpilogue : int {
+    EPI_SIGN_KEYS = 0,   // RPLSH, fused: packed sign bits -> key words [T][n][W] (ENC_BITS)
+    EPI_SIGN_BYTES = 1,  // RPLSH, reference layout: uint8 [T][n][H]
+    EPI_FLOOR_KEYS = 2,  // p-stable, fused: byte-swapped floor(x+b) -> key words [T][n][H] (ENC_BE)
+    EPI_FLOOR_I32 = 3    // p-stable, reference layout: int32 [T][n][H]
+};
+culsh_status launch_project_f32(culsh_ctx* ctx, const float* X, const float* P, const float* b,
+                                int n, int d, int T, int H, ProjEpilogue epi, void* out);
+culsh_status launch_project_f64(culsh_ctx* ctx, const double* X, const double* P, const double* b,
+                                int n, int d, int T, int H, ProjEpilogue epi, void* out);
+
+// ---------------------------------------------------------------- minhash (minhash.hip)
+// as_keys: write byte-swapped values (ENC_BE key words) instead of the raw uint32.
+culsh_status launch_minhash(culsh_ctx* ctx, const int32_t* indices, const int32_t* indptr,
+                            const uint32_t* A, const uint32_t* B, int n, int T, int H,
+                            bool as_keys, uint32_t* out);
+
+// ---------------------------------------------------------------- key codec (index.hip)
+// signature bytes [T][n][S] -> key words [T][n][W]
+culsh_status launch_sig_to_keys(culsh_ctx* ctx, const uint8_t* sig, size_t n_items, int S,
+                                KeyEnc enc, int W, uint32_t* keys);
+// key words [count][W] -> signature bytes [count][S]
+culsh_status launch_keys_to_sig(culsh_ctx* ctx, const uint32_t* keys, size_t count, int S,
+                                KeyEnc enc, int W, uint8_t* sig);
+
+// ---------------------------------------------------------------- sort (sort.hip)
+// Stable sort of each table's n items by key words (word 0 most significant), starting
+// from the identity permutation.  keys_in [T][n][W] is clobbered.  On return
+// *sorted_keys points at whichever of keys_in / keys_tmp holds the sorted keys and
+// rows_out [T][n] holds the row ids in sorted order.
+culsh_status sort_tables(culsh_ctx* ctx, uint32_t* keys_in, uint32_t* keys_tmp, int32_t* rows_tmp,
+                         int32_t* rows_out, int n, int T, int W, uint32_t** sorted_keys);
+size_t sort_scratch_bytes(int n, int T, int W);
+
+// ---------------------------------------------------------------- index build (index.hip)
+// From sorted keys + rows to the core::Index arrays (allocates them; one host sync).
+culsh_status build_index_from_sorted(culsh_ctx* ctx, const uint32_t* sorted_keys, int32_t* rows_sorted_owned,
+                                     int n, int T, int H, int S, KeyEnc enc, int W,
+                                     int32_t* item_to_bucket_opt, culsh_index* index);
+// Full pipeline from unsorted key words (arena-owned, clobbered).
+culsh_status fit_index_from_keys(culsh_ctx* ctx, uint32_t* keys, int n, int T, int H, int S,
+                                 KeyEnc enc, int W, int32_t* item_to_bucket_opt, culsh_index* index);
+
+// ---------------------------------------------------------------- query (query.hip)
+culsh_status launch_find_matching_buckets(culsh_ctx* ctx, const uint32_t* q_keys, int n_queries,
+                                          const culsh_index* index, int32_t* matched);
+culsh_status query_from_matched(culsh_ctx* ctx, const int32_t* matched, int n_queries,
+                                const culsh_index* index, culsh_candidates* out);
+
+// ---------------------------------------------------------------- scans (scan.hip)
+// Exclusive prefix sum of `n` u64 values; out[n] receives the total (out has n+1 slots).
+culsh_status exclusive_scan_u64(culsh_ctx* ctx, const uint64_t* in, uint64_t* out, size_t n);
+
+// ---------------------------------------------------------------- host-side generator (rng.cpp part of api)
+void gen_normals_f64(uint64_t seed, int stream, size_t n, double* out);
+void gen_raw_u64(uint64_t seed, int stream, size_t n, uint64_t* out);
+
+void free_index_arrays(culsh_index* ix);
+void free_candidates_arrays(culsh_candidates* c);
+
+inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
+inline unsigned div_up(size_t a, size_t b) { return static_cast<unsigned>((a + b - 1) / b); }
+
+}  // namespace culsh_amd

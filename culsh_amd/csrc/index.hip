@@ -1,0 +1,194 @@
+// Index build from sorted keys, and the signature <-> key-word codec.
+//
+// Role of mark_boundaries_kernel, the bucket-flag scan, the table-offset selection and
+// build_final_index_kernel of the reference (core/fit.cuh:97-208, 305-362), fused into
+// two passes over the sorted items: count bucket heads per tile, then (after a scan of
+// the tile counts) write bucket offsets, bucket keys, table offsets and, optionally, the
+// (row, table) -> bucket map.
+#include "block_utils.hpp"
+#include "common.hpp"
+
+namespace culsh_amd {
+namespace {
+
+constexpr int IB_THREADS = 256;
+constexpr int IB_ITEMS = 8;
+constexpr int IB_TILE = IB_THREADS * IB_ITEMS;
+
+// head(i): first item of its table, or key differs from the previous item
+// (mark_boundaries_kernel, core/fit.cuh:97-143)
+__device__ __forceinline__ uint32_t is_head(const uint32_t* __restrict__ keys, size_t i, int n, int W) {
+    if (i % n == 0) return 1u;
+    const uint32_t* a = keys + i * W;
+    const uint32_t* b = a - W;
+    uint32_t diff = 0;
+    for (int w = 0; w < W; ++w) diff |= a[w] ^ b[w];
+    return diff != 0u;
+}
+
+__global__ __launch_bounds__(IB_THREADS) void count_heads_kernel(const uint32_t* __restrict__ keys, size_t N,
+                                                                int n, int W, uint64_t* __restrict__ tile_counts) {
+    __shared__ uint64_t scratch[17];
+    const size_t base = static_cast<size_t>(blockIdx.x) * IB_TILE + threadIdx.x * IB_ITEMS;
+    uint64_t c = 0;
+#pragma unroll
+    for (int i = 0; i < IB_ITEMS; ++i)
+        if (base + i < N) c += is_head(keys, base + i, n, W);
+    uint64_t total;
+    block_exclusive_sum(c, scratch, &total);
+    if (threadIdx.x == 0) tile_counts[blockIdx.x] = total;
+}
+
+__global__ __launch_bounds__(IB_THREADS) void build_index_kernel(
+    const uint32_t* __restrict__ keys, const int32_t* __restrict__ rows, size_t N, int n, int T, int W,
+    const uint64_t* __restrict__ tile_base, int n_buckets, int32_t* __restrict__ bucket_candidate_offsets,
+    uint32_t* __restrict__ bucket_keys, int32_t* __restrict__ table_bucket_offsets,
+    int32_t* __restrict__ item_to_bucket) {
+    __shared__ uint64_t scratch[17];
+    const size_t base = static_cast<size_t>(blockIdx.x) * IB_TILE + threadIdx.x * IB_ITEMS;
+    uint32_t flag[IB_ITEMS];
+    uint64_t c = 0;
+#pragma unroll
+    for (int i = 0; i < IB_ITEMS; ++i) {
+        flag[i] = (base + i < N) ? is_head(keys, base + i, n, W) : 0u;
+        c += flag[i];
+    }
+    uint64_t total;
+    uint64_t run = tile_base[blockIdx.x] + block_exclusive_sum(c, scratch, &total);
+#pragma unroll
+    for (int i = 0; i < IB_ITEMS; ++i) {
+        const size_t pos = base + i;
+        if (pos >= N) break;
+        run += flag[i];
+        const int32_t bucket = static_cast<int32_t>(run) - 1;  // scan + flag - 1 (fit.cuh:183)
+        if (flag[i]) {
+            bucket_candidate_offsets[bucket] = static_cast<int32_t>(pos);  // fit.cuh:190-191
+            for (int w = 0; w < W; ++w) bucket_keys[static_cast<size_t>(bucket) * W + w] = keys[pos * W + w];
+            if (pos % n == 0) table_bucket_offsets[pos / n] = bucket;      // fit.cuh:317-326
+        }
+        if (item_to_bucket) {
+            const size_t t = pos / n;
+            item_to_bucket[static_cast<size_t>(rows[pos]) * T + t] = bucket;  // fit.cuh:180-185
+        }
+    }
+    if (blockIdx.x == 0 && threadIdx.x == 0) {  // terminators, fit.cuh:351-357
+        table_bucket_offsets[T] = n_buckets;
+        bucket_candidate_offsets[n_buckets] = static_cast<int32_t>(N);
+    }
+}
+
+__global__ __launch_bounds__(256) void sig_to_keys_kernel(const uint8_t* __restrict__ sig, size_t n_items,
+                                                         int S, int enc, int W, uint32_t* __restrict__ keys) {
+    const size_t idx = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (idx >= n_items * W) return;
+    const size_t item = idx / W;
+    const int w = static_cast<int>(idx - item * W);
+    const uint8_t* s = sig + item * S;
+    uint32_t k = 0;
+    if (enc == ENC_BE) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int byte = 4 * w + j;
+            if (byte < S) k |= static_cast<uint32_t>(s[byte]) << (24 - 8 * j);
+        }
+    } else {
+        for (int j = 0; j < 32; ++j) {
+            const int h = 32 * w + j;
+            if (h < S && s[h] != 0) k |= 1u << (31 - j);
+        }
+    }
+    keys[idx] = k;
+}
+
+__global__ __launch_bounds__(256) void keys_to_sig_kernel(const uint32_t* __restrict__ keys, size_t count,
+                                                         int S, int enc, int W, uint8_t* __restrict__ sig) {
+    const size_t idx = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (idx >= count * S) return;
+    const size_t item = idx / S;
+    const int byte = static_cast<int>(idx - item * S);
+    const uint32_t* k = keys + item * W;
+    if (enc == ENC_BE)
+        sig[idx] = static_cast<uint8_t>(k[byte >> 2] >> (24 - 8 * (byte & 3)));
+    else
+        sig[idx] = static_cast<uint8_t>((k[byte >> 5] >> (31 - (byte & 31))) & 1u);
+}
+
+}  // namespace
+
+culsh_status launch_sig_to_keys(culsh_ctx* ctx, const uint8_t* sig, size_t n_items, int S, KeyEnc enc, int W,
+                                uint32_t* keys) {
+    if (n_items == 0) return CULSH_OK;
+    const size_t total = n_items * W;
+    CULSH_REQUIRE(div_up(total, 256) < (1u << 31) && total / 256 < (1ull << 31), CULSH_ERR_LIMIT, "too many items");
+    hipLaunchKernelGGL(sig_to_keys_kernel, dim3(div_up(total, 256)), dim3(256), 0, ctx->stream, sig, n_items, S,
+                       static_cast<int>(enc), W, keys);
+    CULSH_LAUNCH_CHECK();
+    return CULSH_OK;
+}
+
+culsh_status launch_keys_to_sig(culsh_ctx* ctx, const uint32_t* keys, size_t count, int S, KeyEnc enc, int W,
+                                uint8_t* sig) {
+    if (count == 0) return CULSH_OK;
+    const size_t total = count * S;
+    CULSH_REQUIRE(total / 256 < (1ull << 31), CULSH_ERR_LIMIT, "too many buckets");
+    hipLaunchKernelGGL(keys_to_sig_kernel, dim3(div_up(total, 256)), dim3(256), 0, ctx->stream, keys, count, S,
+                       static_cast<int>(enc), W, sig);
+    CULSH_LAUNCH_CHECK();
+    return CULSH_OK;
+}
+
+culsh_status build_index_from_sorted(culsh_ctx* ctx, const uint32_t* sorted_keys, int32_t* rows_sorted_owned,
+                                     int n, int T, int H, int S, KeyEnc enc, int W,
+                                     int32_t* item_to_bucket_opt, culsh_index* index) {
+    const size_t N = static_cast<size_t>(n) * T;
+    const size_t tiles = (N + IB_TILE - 1) / IB_TILE;
+    uint64_t* tile_counts = nullptr;
+    uint64_t* tile_base = nullptr;
+    CULSH_TRY(arena_alloc_t(ctx, tiles, &tile_counts));
+    CULSH_TRY(arena_alloc_t(ctx, tiles + 1, &tile_base));
+    hipLaunchKernelGGL(count_heads_kernel, dim3(static_cast<unsigned>(tiles)), dim3(IB_THREADS), 0, ctx->stream,
+                       sorted_keys, N, n, W, tile_counts);
+    CULSH_LAUNCH_CHECK();
+    CULSH_TRY(exclusive_scan_u64(ctx, tile_counts, tile_base, tiles));
+    uint64_t n_buckets64 = 0;
+    CULSH_TRY(read_back_u64(ctx, tile_base + tiles, 1, &n_buckets64));  // the one host sync (fit.cuh:332-337)
+    const int B = static_cast<int>(n_buckets64);
+
+    index->all_candidate_indices = rows_sorted_owned;
+    index->n_total_candidates = static_cast<int>(N);
+    index->n_total_buckets = B;
+    index->n_hash_tables = T;
+    index->n_hashes = H;
+    index->sig_nbytes = S;
+    index->enc = enc;
+    index->key_w = W;
+    CULSH_HIP(hipMalloc(&index->bucket_candidate_offsets, (static_cast<size_t>(B) + 1) * sizeof(int32_t)));
+    CULSH_HIP(hipMalloc(&index->table_bucket_offsets, (static_cast<size_t>(T) + 1) * sizeof(int32_t)));
+    CULSH_HIP(hipMalloc(&index->bucket_keys, std::max<size_t>(1, static_cast<size_t>(B) * W) * sizeof(uint32_t)));
+    CULSH_HIP(hipMalloc(&index->all_bucket_signatures, std::max<size_t>(1, static_cast<size_t>(B) * S)));
+    hipLaunchKernelGGL(build_index_kernel, dim3(static_cast<unsigned>(tiles)), dim3(IB_THREADS), 0, ctx->stream,
+                       sorted_keys, rows_sorted_owned, N, n, T, W, tile_base, B, index->bucket_candidate_offsets,
+                       index->bucket_keys, index->table_bucket_offsets, item_to_bucket_opt);
+    CULSH_LAUNCH_CHECK();
+    CULSH_TRY(launch_keys_to_sig(ctx, index->bucket_keys, B, S, enc, W, index->all_bucket_signatures));
+    return CULSH_OK;
+}
+
+culsh_status fit_index_from_keys(culsh_ctx* ctx, uint32_t* keys, int n, int T, int H, int S, KeyEnc enc, int W,
+                                 int32_t* item_to_bucket_opt, culsh_index* index) {
+    const size_t N = static_cast<size_t>(n) * T;
+    CULSH_REQUIRE(N < (1ull << 31), CULSH_ERR_LIMIT,
+                  "n_samples * n_hash_tables must be below 2^31 (int32 candidate positions)");
+    uint32_t* keys_tmp = nullptr;
+    int32_t* rows_tmp = nullptr;
+    int32_t* rows_out = nullptr;
+    CULSH_TRY(arena_alloc_t(ctx, N * W, &keys_tmp));
+    CULSH_TRY(arena_alloc_t(ctx, N, &rows_tmp));
+    CULSH_HIP(hipMalloc(&rows_out, N * sizeof(int32_t)));
+    index->all_candidate_indices = rows_out;  // owned by the index from here on (freed with it)
+    uint32_t* sorted = nullptr;
+    CULSH_TRY(sort_tables(ctx, keys, keys_tmp, rows_tmp, rows_out, n, T, W, &sorted));
+    return build_index_from_sorted(ctx, sorted, rows_out, n, T, H, S, enc, W, item_to_bucket_opt, index);
+}
+
+}  // namespace culsh_amd

@@ -1,0 +1,353 @@
+// Projection hashing for RPLSH and p-stable LSH on gfx950.
+//
+// Replaces the reference's GEMM + elementwise pass (rplsh/hash.cuh:92-129,
+// pslsh/hash.cuh:104-142): X * P^T is computed with fp32 MFMA tiles and the sign /
+// floor epilogue is applied to the accumulators in registers, so the n x (T*H)
+// projection matrix is never written to memory.
+#include "common.hpp"
+
+namespace culsh_amd {
+
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+namespace {
+
+constexpr int BM = 128;        // rows of X per workgroup
+constexpr int BN = 128;        // (virtual) hash columns per workgroup
+constexpr int BK = 32;         // features per LDS stage
+constexpr int PITCH = BK + 4;  // LDS row pitch in floats (bank spread for 16-byte reads)
+constexpr int NTHREADS = 256;  // 4 wavefronts as 2 x 2, each 64 x 64 of the tile
+
+struct ProjArgs {
+    const float* X;
+    const float* P;
+    const float* b;
+    void* out;
+    int n, d, T, H;
+    int n_row_tiles, n_col_tiles;
+    int vec_x, vec_p;  // 16-byte vector loads allowed
+};
+
+// Column order of the sign-packing epilogue.  Columns are grouped in tiles of 32 so that
+// one wavefront ballot over a 32-column MFMA tile yields key bits directly:
+//   H <= 32: a tile holds floor(32/H) whole tables; table `sub` owns ballot bits
+//            [sub*H, sub*H + H) with hash 0 at the top of that field
+//   H  > 32: a tile is one 32-bit key word of one table, hash 32w + j at bit 31 - j
+// Returns the row of P feeding virtual column vc, or -1 for a padding column.
+__device__ __forceinline__ int sign_vcol_to_prow(int vc, int T, int H) {
+    const int tile = vc >> 5, c = vc & 31;
+    if (H <= 32) {
+        const int tpt = 32 / H;
+        const int sub = c / H;
+        const int table = tile * tpt + sub;
+        if (sub >= tpt || table >= T) return -1;
+        return table * H + (H - 1 - (c - sub * H));
+    }
+    const int wt = (H + 31) >> 5;
+    const int table = tile / wt, w = tile - table * wt;
+    const int h = 32 * w + (31 - c);
+    if (table >= T || h >= H) return -1;
+    return table * H + h;
+}
+
+__device__ __forceinline__ float4 load4(const float* __restrict__ base, size_t row_off, int k,
+                                        int d, bool row_ok, int vec_ok) {
+    float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (!row_ok) return v;
+    const float* p = base + row_off + k;
+    if (vec_ok && k + 3 < d) return *reinterpret_cast<const float4*>(p);
+    if (k + 0 < d) v.x = p[0];
+    if (k + 1 < d) v.y = p[1];
+    if (k + 2 < d) v.z = p[2];
+    if (k + 3 < d) v.w = p[3];
+    return v;
+}
+
+template <int EPI>
+__global__ __launch_bounds__(NTHREADS) void project_f32_kernel(ProjArgs a) {
+    __shared__ __attribute__((aligned(16))) float As[BM * PITCH];
+    __shared__ __attribute__((aligned(16))) float Bs[BN * PITCH];
+    __shared__ uint32_t tw[(EPI == EPI_SIGN_KEYS) ? BM * (BN / 32) : 1];
+
+    // Workgroup -> (row tile, column tile).  Consecutive workgroup ids are dealt round
+    // robin to the 8 XCDs; ids are arranged so that all column tiles of one row tile land
+    // on the same XCD (same id mod 8) and close in time, so the X tile is fetched from HBM
+    // once and served from that XCD's L2 afterwards.
+    const int nct = a.n_col_tiles;
+    const int per_group = 8 * nct;
+    const int g = blockIdx.x / per_group, rem = blockIdx.x - g * per_group;
+    const int ct = rem >> 3, slot = rem & 7;
+    const int rt = g * 8 + slot;
+    if (rt >= a.n_row_tiles) return;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int r32 = lane & 31, half = lane >> 5;
+    const int n = a.n, d = a.d, T = a.T, H = a.H;
+    const int TH = T * H;
+
+    // global -> LDS staging: thread loads float4 number (tid + 256*i), i < 4, of each tile
+    const int lrow = tid >> 3, c4 = (tid & 7) * 4;
+    size_t xoff[4], poff[4];
+    bool xok[4], pok[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int row = rt * BM + lrow + 32 * i;
+        xok[i] = row < n;
+        xoff[i] = static_cast<size_t>(row) * d;
+        const int vc = ct * BN + lrow + 32 * i;
+        const int prow = (EPI == EPI_SIGN_KEYS) ? sign_vcol_to_prow(vc, T, H) : (vc < TH ? vc : -1);
+        pok[i] = prow >= 0;
+        poff[i] = static_cast<size_t>(prow < 0 ? 0 : prow) * d;
+    }
+
+    f32x16 acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+
+    float4 ra[4], rb[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        ra[i] = load4(a.X, xoff[i], c4, d, xok[i], a.vec_x);
+        rb[i] = load4(a.P, poff[i], c4, d, pok[i], a.vec_p);
+    }
+
+    const int nk = (d + BK - 1) / BK;
+    for (int kt = 0; kt < nk; ++kt) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            *reinterpret_cast<float4*>(&As[(lrow + 32 * i) * PITCH + c4]) = ra[i];
+            *reinterpret_cast<float4*>(&Bs[(lrow + 32 * i) * PITCH + c4]) = rb[i];
+        }
+        __syncthreads();
+        if (kt + 1 < nk) {
+            const int k0 = (kt + 1) * BK + c4;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                ra[i] = load4(a.X, xoff[i], k0, d, xok[i], a.vec_x);
+                rb[i] = load4(a.P, poff[i], k0, d, pok[i], a.vec_p);
+            }
+        }
+        // The 32x32x2 MFMA takes, per lane, A[row = lane%32][k = lane/32] and
+        // B[k = lane/32][col = lane%32].  Any pairing of k between A and B that covers each
+        // feature once is a valid dot product, so lanes 0-31 walk features 0..15 of the
+        // stage and lanes 32-63 features 16..31: each lane reads 16 consecutive floats.
+        float af[2][16], bf[2][16];
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            const float* pa = &As[(wm * 64 + i * 32 + r32) * PITCH + half * 16];
+            const float* pb = &Bs[(wn * 64 + i * 32 + r32) * PITCH + half * 16];
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const float4 va = *reinterpret_cast<const float4*>(pa + 4 * q);
+                const float4 vb = *reinterpret_cast<const float4*>(pb + 4 * q);
+                af[i][4 * q + 0] = va.x; af[i][4 * q + 1] = va.y;
+                af[i][4 * q + 2] = va.z; af[i][4 * q + 3] = va.w;
+                bf[i][4 * q + 0] = vb.x; bf[i][4 * q + 1] = vb.y;
+                bf[i][4 * q + 2] = vb.z; bf[i][4 * q + 3] = vb.w;
+            }
+        }
+#pragma unroll
+        for (int k = 0; k < 16; ++k)
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+#pragma unroll
+                for (int j = 0; j < 2; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[i][k], bf[j][k], acc[i][j], 0, 0, 0);
+        __syncthreads();
+    }
+
+    // Accumulator layout of the 32x32 tile: register v of lane l holds
+    // row 8*(v/4) + 4*(l/32) + v%4, column l%32.
+    if (EPI == EPI_SIGN_KEYS) {
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                uint32_t mine = 0;
+#pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    // hash bit = 1 iff the sign bit is clear (rplsh/hash.cuh:47)
+                    const unsigned long long m =
+                        __builtin_amdgcn_ballot_w64((__float_as_uint(acc[i][j][v]) >> 31) == 0u);
+                    const int rlo = 8 * (v >> 2) + (v & 3);
+                    mine = (lane == rlo) ? static_cast<uint32_t>(m) : mine;
+                    mine = (lane == rlo + 4) ? static_cast<uint32_t>(m >> 32) : mine;
+                }
+                if (lane < 32) tw[(wm * 64 + i * 32 + lane) * (BN / 32) + (wn * 2 + j)] = mine;
+            }
+        __syncthreads();
+        uint32_t* keys = static_cast<uint32_t*>(a.out);
+        if (H <= 32) {
+            const int tpt = 32 / H;
+            const uint32_t mask = (H == 32) ? 0xFFFFFFFFu : ((1u << H) - 1u);
+            const int total = (BN / 32) * tpt * BM;
+            for (int idx = tid; idx < total; idx += NTHREADS) {
+                const int tl = idx / BM, row = idx - tl * BM;
+                const int tc = tl / tpt, sub = tl - tc * tpt;
+                const int table = (ct * (BN / 32) + tc) * tpt + sub;
+                const int grow = rt * BM + row;
+                if (table < T && grow < n) {
+                    const uint32_t field = (tw[row * (BN / 32) + tc] >> (sub * H)) & mask;
+                    keys[static_cast<size_t>(table) * n + grow] = field << (32 - H);
+                }
+            }
+        } else {
+            const int wt = (H + 31) >> 5;
+            for (int idx = tid; idx < (BN / 32) * BM; idx += NTHREADS) {
+                const int tc = idx / BM, row = idx - tc * BM;
+                const int tile = ct * (BN / 32) + tc;
+                const int table = tile / wt, w = tile - table * wt;
+                const int grow = rt * BM + row;
+                if (table < T && grow < n) {
+                    const int nbits = min(32, H - 32 * w);
+                    const uint32_t mask = (nbits == 32) ? 0xFFFFFFFFu : (0xFFFFFFFFu << (32 - nbits));
+                    keys[(static_cast<size_t>(table) * n + grow) * wt + w] = tw[row * (BN / 32) + tc] & mask;
+                }
+            }
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                const int col = ct * BN + wn * 64 + j * 32 + r32;
+                if (col >= TH) continue;
+                const int t = col / H, h = col - t * H;
+                const float bias = (EPI == EPI_FLOOR_KEYS || EPI == EPI_FLOOR_I32) ? a.b[col] : 0.f;
+#pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    const int row = rt * BM + wm * 64 + i * 32 + 8 * (v >> 2) + 4 * half + (v & 3);
+                    if (row >= n) continue;
+                    const size_t off = (static_cast<size_t>(t) * n + row) * H + h;
+                    const float x = acc[i][j][v];
+                    if (EPI == EPI_SIGN_BYTES) {
+                        static_cast<uint8_t*>(a.out)[off] =
+                            static_cast<uint8_t>((__float_as_uint(x) >> 31) ^ 1u);
+                    } else {
+                        const int32_t f = static_cast<int32_t>(floorf(x + bias));  // pslsh/hash.cuh:46
+                        if (EPI == EPI_FLOOR_I32)
+                            static_cast<int32_t*>(a.out)[off] = f;
+                        else
+                            static_cast<uint32_t*>(a.out)[off] = __builtin_bswap32(static_cast<uint32_t>(f));
+                    }
+                }
+            }
+    }
+}
+
+// ---------------------------------------------------------------- fp64 (plain FMA tiles)
+constexpr int DT = 64;   // tile edge
+constexpr int DK = 16;   // features per stage
+
+template <int EPI>
+__global__ __launch_bounds__(256) void project_f64_kernel(const double* __restrict__ X,
+                                                         const double* __restrict__ P,
+                                                         const double* __restrict__ b, void* out,
+                                                         int n, int d, int T, int H) {
+    __shared__ double Xs[DK][DT + 1];
+    __shared__ double Ps[DK][DT + 1];
+    const int tx = threadIdx.x & 15, ty = threadIdx.x >> 4;
+    const int row0 = blockIdx.x * DT, col0 = blockIdx.y * DT;
+    const int TH = T * H;
+    double acc[4][4] = {};
+    for (int k0 = 0; k0 < d; k0 += DK) {
+        for (int idx = threadIdx.x; idx < DT * DK; idx += 256) {
+            const int r = idx / DK, k = idx - r * DK;
+            const int gr = row0 + r, gc = col0 + r, gk = k0 + k;
+            Xs[k][r] = (gr < n && gk < d) ? X[static_cast<size_t>(gr) * d + gk] : 0.0;
+            Ps[k][r] = (gc < TH && gk < d) ? P[static_cast<size_t>(gc) * d + gk] : 0.0;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int k = 0; k < DK; ++k) {
+            double xa[4], pb[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) { xa[i] = Xs[k][ty + 16 * i]; pb[i] = Ps[k][tx + 16 * i]; }
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) acc[i][j] = fma(xa[i], pb[j], acc[i][j]);
+        }
+        __syncthreads();
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int row = row0 + ty + 16 * i, col = col0 + tx + 16 * j;
+            if (row >= n || col >= TH) continue;
+            const int t = col / H, h = col - t * H;
+            const size_t off = (static_cast<size_t>(t) * n + row) * H + h;
+            if (EPI == EPI_SIGN_BYTES) {
+                // narrowing to float keeps the sign (rplsh/hash.cuh:47)
+                static_cast<uint8_t*>(out)[off] = (__double_as_longlong(acc[i][j]) < 0) ? 0 : 1;
+            } else {
+                static_cast<int32_t*>(out)[off] = static_cast<int32_t>(floor(acc[i][j] + b[col]));
+            }
+        }
+}
+
+}  // namespace
+
+culsh_status launch_project_f32(culsh_ctx* ctx, const float* X, const float* P, const float* b,
+                                int n, int d, int T, int H, ProjEpilogue epi, void* out) {
+    CULSH_REQUIRE(X && P && out, CULSH_ERR_INVALID, "projection: null pointer");
+    CULSH_REQUIRE(n > 0 && d > 0 && T > 0 && H > 0, CULSH_ERR_INVALID, "projection: sizes must be positive");
+    const bool floor_epi = (epi == EPI_FLOOR_KEYS || epi == EPI_FLOOR_I32);
+    CULSH_REQUIRE(!floor_epi || b, CULSH_ERR_INVALID, "projection: bias is required");
+    CULSH_REQUIRE(static_cast<long long>(T) * H < (1ll << 30), CULSH_ERR_LIMIT, "T*H too large");
+    long long n_vcols;
+    if (epi == EPI_SIGN_KEYS) {
+        const long long tiles = (H <= 32) ? (T + (32 / H) - 1) / (32 / H)
+                                          : static_cast<long long>(T) * ((H + 31) / 32);
+        n_vcols = tiles * 32;
+    } else {
+        n_vcols = static_cast<long long>(T) * H;
+    }
+    ProjArgs a;
+    a.X = X; a.P = P; a.b = b; a.out = out;
+    a.n = n; a.d = d; a.T = T; a.H = H;
+    a.n_row_tiles = (n + BM - 1) / BM;
+    a.n_col_tiles = static_cast<int>((n_vcols + BN - 1) / BN);
+    a.vec_x = (d % 4 == 0) && (reinterpret_cast<uintptr_t>(X) % 16 == 0);
+    a.vec_p = (d % 4 == 0) && (reinterpret_cast<uintptr_t>(P) % 16 == 0);
+    const long long groups = (a.n_row_tiles + 7) / 8;
+    const long long blocks = groups * 8 * a.n_col_tiles;
+    CULSH_REQUIRE(blocks < (1ll << 31), CULSH_ERR_LIMIT, "projection grid too large");
+    dim3 grid(static_cast<unsigned>(blocks)), block(NTHREADS);
+    switch (epi) {
+        case EPI_SIGN_KEYS: hipLaunchKernelGGL(project_f32_kernel<EPI_SIGN_KEYS>, grid, block, 0, ctx->stream, a); break;
+        case EPI_SIGN_BYTES: hipLaunchKernelGGL(project_f32_kernel<EPI_SIGN_BYTES>, grid, block, 0, ctx->stream, a); break;
+        case EPI_FLOOR_KEYS: hipLaunchKernelGGL(project_f32_kernel<EPI_FLOOR_KEYS>, grid, block, 0, ctx->stream, a); break;
+        case EPI_FLOOR_I32: hipLaunchKernelGGL(project_f32_kernel<EPI_FLOOR_I32>, grid, block, 0, ctx->stream, a); break;
+    }
+    CULSH_LAUNCH_CHECK();
+    return CULSH_OK;
+}
+
+culsh_status launch_project_f64(culsh_ctx* ctx, const double* X, const double* P, const double* b,
+                                int n, int d, int T, int H, ProjEpilogue epi, void* out) {
+    CULSH_REQUIRE(X && P && out, CULSH_ERR_INVALID, "projection: null pointer");
+    CULSH_REQUIRE(n > 0 && d > 0 && T > 0 && H > 0, CULSH_ERR_INVALID, "projection: sizes must be positive");
+    CULSH_REQUIRE(epi == EPI_SIGN_BYTES || epi == EPI_FLOOR_I32, CULSH_ERR_INTERNAL,
+                  "fp64 projection writes the reference layout only");
+    CULSH_REQUIRE(epi != EPI_FLOOR_I32 || b, CULSH_ERR_INVALID, "projection: bias is required");
+    const long long TH = static_cast<long long>(T) * H;
+    const long long gy = (TH + DT - 1) / DT;
+    CULSH_REQUIRE(gy <= 65535, CULSH_ERR_LIMIT, "T*H too large for the fp64 projection grid");
+    dim3 grid((n + DT - 1) / DT, static_cast<unsigned>(gy)), block(256);
+    if (epi == EPI_SIGN_BYTES)
+        hipLaunchKernelGGL(project_f64_kernel<EPI_SIGN_BYTES>, grid, block, 0, ctx->stream, X, P, b, out, n, d, T, H);
+    else
+        hipLaunchKernelGGL(project_f64_kernel<EPI_FLOOR_I32>, grid, block, 0, ctx->stream, X, P, b, out, n, d, T, H);
+    CULSH_LAUNCH_CHECK();
+    return CULSH_OK;
+}
+
+}  // namespace culsh_amd

@@ -1,0 +1,406 @@
+"""
+GPU parity tests: the HIP path, called through the C ABI, against the CPU oracle on the
+same seeded inputs.
+
+Bar: bucket tables, matched buckets and candidate lists are bit-exact given identical
+signatures; MinHash signatures are bit-exact; RPLSH / p-stable hash values may differ
+from the float64 oracle only where the projection lies within 1e-5 (relative to
+sum |x_i p_i|) of the decision boundary - the band left open by the unspecified
+summation order of the reference's GEMM.
+"""
+
+import numpy as np
+import pytest
+
+from oracle import culsh_oracle as o
+
+pytestmark = pytest.mark.gpu
+
+TOL = 1e-5  # relative width of the implementation-defined band around a hash boundary
+
+
+@pytest.fixture(scope="module")
+def ctx():
+    from abi import Ctx
+
+    c = Ctx(0)
+    yield c
+    c.close()
+
+
+def _announce(*a):
+    print("[case]", *a, flush=True)
+
+
+def random_sigs(rng, T, n, H, kind):
+    if kind == "rplsh":
+        return rng.integers(0, 2, size=(T, n, H), dtype=np.uint8)
+    if kind == "pslsh":
+        return rng.integers(-3, 4, size=(T, n, H)).astype(np.int32)
+    if kind == "minhash":
+        v = rng.integers(0, 6, size=(T, n, H)).astype(np.uint32)
+        return (v * np.uint32(0x01000193)) ^ np.uint32(0x80000001)
+    if kind == "bytes3":  # generic opaque signatures whose width is not a multiple of 4
+        return rng.integers(0, 3, size=(T, n, 3), dtype=np.uint8) * np.uint8(100)
+    raise ValueError(kind)
+
+
+# ---------------------------------------------------------------- hashing
+@pytest.mark.parametrize("n,d,T,H", [
+    (1, 8, 1, 1), (257, 100, 8, 8), (1000, 128, 16, 8), (333, 33, 5, 16), (129, 64, 3, 32),
+    (200, 40, 4, 20), (150, 128, 2, 40), (300, 36, 3, 64), (4100, 128, 32, 16), (100, 768, 4, 16),
+])
+def test_rplsh_hash_f32(ctx, n, d, T, H):
+    _announce("rplsh_hash_f32", n, d, T, H)
+    rng = np.random.default_rng(n * 7 + d)
+    X = rng.standard_normal((n, d)).astype(np.float32)
+    P = rng.standard_normal((T * H, d)).astype(np.float32)
+    got = ctx.rplsh_hash(X, P, T, H)
+    exp = o.rplsh_hash(X, P, T, H)
+    safe = o.rplsh_margin(X, P, T, H) > TOL
+    assert got.shape == exp.shape and safe.mean() > 0.999
+    np.testing.assert_array_equal(got[safe], exp[safe])
+    assert set(np.unique(got)) <= {0, 1}
+
+
+def test_rplsh_hash_zero_rule(ctx):
+    """+0.0 -> 1 (rplsh/hash.cuh:47): zero rows and zero projections hash to 1; integer
+    data with small-integer projections is exact in fp32, so every bit must match."""
+    rng = np.random.default_rng(1)
+    n, d, T, H = 300, 64, 4, 8
+    X = rng.integers(0, 4, size=(n, d)).astype(np.float32)
+    X[::7] = 0.0
+    P = rng.integers(-2, 3, size=(T * H, d)).astype(np.float32)
+    P[5] = 0.0
+    got = ctx.rplsh_hash(X, P, T, H)
+    proj = X.astype(np.float64) @ P.astype(np.float64).T
+    exp = o.rplsh_hash(X, P, T, H)
+    np.testing.assert_array_equal(got, exp)
+    assert (proj == 0).sum() > n            # exact zeros are exercised
+    assert np.all(got[:, ::7, :] == 1)
+
+
+@pytest.mark.parametrize("n,d,T,H", [(257, 100, 8, 8), (130, 33, 3, 5)])
+def test_rplsh_hash_f64(ctx, n, d, T, H):
+    _announce("rplsh_hash_f64", n, d, T, H)
+    rng = np.random.default_rng(n)
+    X = rng.standard_normal((n, d))
+    P = rng.standard_normal((T * H, d))
+    got = ctx.rplsh_hash(X, P, T, H)
+    safe = o.rplsh_margin(X, P, T, H) > 1e-12
+    np.testing.assert_array_equal(got[safe], o.rplsh_hash(X, P, T, H)[safe])
+
+
+@pytest.mark.parametrize("dtype,tol", [(np.float32, TOL), (np.float64, 1e-12)])
+@pytest.mark.parametrize("n,d,T,H,w", [(300, 128, 16, 8, 4), (129, 30, 3, 5, 2)])
+def test_pslsh_hash(ctx, dtype, tol, n, d, T, H, w):
+    _announce("pslsh_hash", dtype.__name__, n, d, T, H, w)
+    rng = np.random.default_rng(d)
+    X = rng.standard_normal((n, d)).astype(dtype)
+    P, b = o.generate_random_projections_biases(5, T * H, d, w, dtype)
+    got = ctx.pslsh_hash(X, P, b, T, H)
+    exp = o.pslsh_hash(X, P, b, T, H)
+    safe = o.pslsh_margin(X, P, b, T, H) > tol
+    assert safe.mean() > 0.99 and exp.min() < 0 < exp.max()
+    np.testing.assert_array_equal(got[safe], exp[safe])
+
+
+def make_csr(rng, n, d, mean_nnz, empty_rows=()):
+    rows = [np.sort(rng.choice(d, size=min(d, rng.poisson(mean_nnz)), replace=False)) for _ in range(n)]
+    for r in empty_rows:
+        rows[r] = np.array([], dtype=np.int64)
+    indptr = np.concatenate([[0], np.cumsum([len(r) for r in rows])]).astype(np.int32)
+    indices = (np.concatenate(rows) if indptr[-1] else np.zeros(0)).astype(np.int32)
+    return indices, indptr
+
+
+@pytest.mark.parametrize("n,d,T,H,nnz", [(1, 10, 1, 1, 3), (500, 5000, 32, 4, 50), (77, 300, 5, 3, 8), (64, 100000, 2, 130, 20)])
+def test_minhash_compute_exact(ctx, n, d, T, H, nnz):
+    _announce("minhash", n, d, T, H, nnz)
+    rng = np.random.default_rng(n + H)
+    indices, indptr = make_csr(rng, n, d, nnz, empty_rows=(0,) if n > 1 else ())
+    A, B = o.generate_hash_integers(9, T * H)
+    A[0], B[0] = o.MINHASH_PRIME - 1, o.MINHASH_PRIME - 1
+    got = ctx.minhash_compute(indices, indptr, A, B, T, H)
+    np.testing.assert_array_equal(got, o.minhash_hash(indices, indptr, A, B, T, H))
+
+
+# ---------------------------------------------------------------- index build
+@pytest.mark.parametrize("kind", ["rplsh", "pslsh", "minhash", "bytes3"])
+@pytest.mark.parametrize("T,n,H", [(1, 1, 1), (3, 50, 2), (4, 5000, 3), (2, 9000, 8), (33, 300, 16)])
+def test_core_fit_index(ctx, kind, T, n, H):
+    _announce("core_fit_index", kind, T, n, H)
+    rng = np.random.default_rng(7 + T * 1000 + n)
+    sig = random_sigs(rng, T, n, H, kind)
+    ih, itb = ctx.core_fit_index(sig, H, want_item_to_bucket=True)
+    from abi import assert_index_matches
+
+    exp = o.fit_index(sig, H, with_item_to_bucket=True)
+    assert_index_matches(ctx.index_arrays(ih), exp)
+    np.testing.assert_array_equal(itb, exp.item_to_bucket)
+    ctx.free_index(ih)
+
+
+def test_core_fit_index_single_bucket_per_table(ctx):
+    """All signatures equal: no radix pass runs and rows stay in identity order."""
+    sig = np.full((3, 1000, 4), 1, dtype=np.uint8)
+    ih, _ = ctx.core_fit_index(sig, 4)
+    from abi import assert_index_matches
+
+    assert_index_matches(ctx.index_arrays(ih), o.fit_index(sig, 4))
+    ctx.free_index(ih)
+
+
+def test_core_fit_index_against_c_oracle_larger(ctx, c_oracle):
+    rng = np.random.default_rng(99)
+    T, n, H = 8, 60000, 12
+    sig = rng.integers(0, 2, size=(T, n, H), dtype=np.uint8)
+    sig[:, :, :4] = 1       # constant leading bytes
+    ih, _ = ctx.core_fit_index(sig, H)
+    from abi import assert_index_matches
+
+    assert_index_matches(ctx.index_arrays(ih), c_oracle.fit_index(sig, H))
+    ctx.free_index(ih)
+
+
+# ---------------------------------------------------------------- query
+@pytest.mark.parametrize("kind", ["rplsh", "pslsh", "minhash", "bytes3"])
+def test_core_query(ctx, kind):
+    _announce("core_query", kind)
+    rng = np.random.default_rng(23)
+    T, n, nq, H = 6, 3000, 200, 3
+    sig = random_sigs(rng, T, n, H, kind)
+    qsig = random_sigs(rng, T, nq, H, kind)
+    qsig[:, :20] = sig[:, :20]
+    if kind != "rplsh":
+        qsig[:, 20:25] = 77
+    ih, _ = ctx.core_fit_index(sig, H)
+    exp_ix = o.fit_index(sig, H)
+    np.testing.assert_array_equal(ctx.core_find_matching_buckets(qsig, ih),
+                                  o.find_matching_buckets_fast(qsig, exp_ix))
+    from abi import assert_candidates_match
+
+    got = ctx.core_query_index(qsig, ih)
+    assert_candidates_match(got, o.query_index(qsig, exp_ix))
+    assert got["counts"].dtype == np.uint64 and got["indices"].dtype == np.int32
+    ctx.free_index(ih)
+
+
+def test_core_query_no_candidates(ctx):
+    sig = np.zeros((2, 100, 2), dtype=np.uint8)
+    qsig = np.ones((2, 7, 2), dtype=np.uint8)
+    ih, _ = ctx.core_fit_index(sig, 2)
+    got = ctx.core_query_index(qsig, ih)
+    assert got["n_total_candidates"] == 0 and len(got["indices"]) == 0
+    np.testing.assert_array_equal(got["offsets"], np.zeros(8, np.uint64))
+    np.testing.assert_array_equal(got["counts"], np.zeros(7, np.uint64))
+    ctx.free_index(ih)
+
+
+def test_core_query_from_matched_with_misses(ctx):
+    rng = np.random.default_rng(4)
+    T, n, H = 5, 2000, 2
+    sig = random_sigs(rng, T, n, H, "pslsh")
+    ih, _ = ctx.core_fit_index(sig, H)
+    exp_ix = o.fit_index(sig, H)
+    nq = 64
+    matched = rng.integers(-1, exp_ix.n_total_buckets, size=nq * T).astype(np.int32)
+    for t in range(T):  # keep each entry inside its table (or -1)
+        col = matched[t::T]
+        lo, hi = exp_ix.table_bucket_offsets[t], exp_ix.table_bucket_offsets[t + 1]
+        col[col >= 0] = lo + col[col >= 0] % (hi - lo)
+    from abi import assert_candidates_match
+
+    assert_candidates_match(ctx.core_query_from_matched(matched, nq, ih),
+                            o.query_from_matched_buckets(matched, nq, exp_ix))
+    ctx.free_index(ih)
+
+
+@pytest.mark.parametrize("n", [40000, 1200000])
+def test_core_query_wide_row_range(ctx, c_oracle, n):
+    """Row ranges beyond one LDS bitmap pass (2^20 rows) and beyond one word per thread."""
+    _announce("wide_row_range", n)
+    rng = np.random.default_rng(n)
+    T, H, nq = 3, 2, 20
+    sig = rng.integers(0, 2, size=(T, n, H), dtype=np.uint8)
+    qsig = rng.integers(0, 2, size=(T, nq, H), dtype=np.uint8)
+    ih, _ = ctx.core_fit_index(sig, H)
+    from abi import assert_candidates_match, assert_index_matches
+
+    cix = c_oracle.fit_index_c(sig, H)
+    assert_index_matches(ctx.index_arrays(ih), cix.to_numpy(n))
+    assert_candidates_match(ctx.core_query_index(qsig, ih), c_oracle.query_index_c(qsig, cix))
+    ctx.free_index(ih)
+
+
+@pytest.mark.parametrize("kind", ["rplsh", "pslsh", "minhash"])
+def test_core_fit_query(ctx, kind):
+    """fit_query == fit + query on the same signatures (python/tests/test_rplsh.py:145-174)."""
+    rng = np.random.default_rng(5)
+    T, n, H = 4, 3000, 3
+    sig = random_sigs(rng, T, n, H, kind)
+    from abi import assert_candidates_match
+
+    got = ctx.core_fit_query(sig, H)
+    assert_candidates_match(got, o.fit_query(sig, H))
+    ih, _ = ctx.core_fit_index(sig, H)
+    again = ctx.core_query_index(sig, ih)
+    for k in ("indices", "offsets", "counts"):
+        np.testing.assert_array_equal(got[k], again[k])
+    ctx.free_index(ih)
+
+
+# ---------------------------------------------------------------- whole path per family
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("n,d,T,H,nq", [(10000, 128, 16, 8, 100), (3000, 100, 8, 16, 64), (2000, 64, 3, 40, 50)])
+def test_rplsh_fit_query_path(ctx, dtype, n, d, T, H, nq):
+    """Config-1 shape (10000x128, 100 queries, 16 tables x 8 hashes, P from seed 42) and
+    variants.  The bucket table must equal the oracle's table built from the GPU's own
+    signatures (bit-exact given identical signatures); the GPU signatures must equal the
+    float64 oracle's outside the band; candidate sets must have Jaccard >= 0.999."""
+    _announce("rplsh_path", dtype.__name__, n, d, T, H, nq)
+    rng = np.random.default_rng(1234)
+    X = rng.standard_normal((n, d)).astype(dtype)
+    Q = np.random.default_rng(4321).standard_normal((nq, d)).astype(dtype)
+    P = np.random.default_rng(42).standard_normal((T * H, d)).astype(dtype)
+    from abi import assert_candidates_match, assert_index_matches
+
+    sig = ctx.rplsh_hash(X, P, T, H)
+    qsig = ctx.rplsh_hash(Q, P, T, H)
+    tol = TOL if dtype == np.float32 else 1e-12
+    safe = o.rplsh_margin(X, P, T, H) > tol
+    np.testing.assert_array_equal(sig[safe], o.rplsh_hash(X, P, T, H)[safe])
+
+    ih = ctx.rplsh_fit(X, T, H, seed=42, P=P)
+    exp_ix = o.fit_index(sig, H)
+    got_ix = ctx.index_arrays(ih)
+    assert_index_matches(got_ix, exp_ix)
+    assert got_ix["n_features"] == d and got_ix["is_double"] == (dtype == np.float64)
+    assert got_ix["sig_nbytes"] == H and got_ix["seed"] == 42
+    np.testing.assert_array_equal(ctx.index_param(ih, 4, dtype), P.reshape(-1))
+
+    got = ctx.rplsh_query(Q, ih)
+    assert_candidates_match(got, o.query_index(qsig, exp_ix))
+    # against the all-float64 oracle: per-query Jaccard
+    ref = o.query_index(o.rplsh_hash(Q, P, T, H), o.fit_index(o.rplsh_hash(X, P, T, H), H))
+    jac = []
+    for q in range(nq):
+        a = got["indices"][int(got["offsets"][q]):int(got["offsets"][q + 1])]
+        b = ref.query_candidate_indices[int(ref.query_candidate_offsets[q]):int(ref.query_candidate_offsets[q + 1])]
+        u = len(np.union1d(a, b))
+        jac.append(1.0 if u == 0 else len(np.intersect1d(a, b)) / u)
+    assert np.mean(jac) >= 0.999
+
+    # batched == unbatched (python/tests/test_rplsh.py:177-209)
+    for bs in (10, 50, nq, 7):
+        bat = ctx.rplsh_query(Q, ih, batch_size=bs)
+        for k in ("indices", "offsets", "counts"):
+            np.testing.assert_array_equal(bat[k], got[k])
+
+    # fit_query == fit + query(X) (python/tests/test_rplsh.py:145-174)
+    m = min(n, 1500)
+    fq = ctx.rplsh_fit_query(X[:m], T, H, seed=42, P=P)
+    ih2 = ctx.rplsh_fit(X[:m], T, H, seed=42, P=P)
+    qq = ctx.rplsh_query(X[:m], ih2)
+    for k in ("indices", "offsets", "counts"):
+        np.testing.assert_array_equal(fq[k], qq[k])
+    ctx.free_index(ih)
+    ctx.free_index(ih2)
+
+
+def test_rplsh_seeded_projection_matches_generator(ctx):
+    """fit without an injected P draws it from the seed with the documented generator."""
+    rng = np.random.default_rng(2)
+    X = rng.standard_normal((500, 32)).astype(np.float32)
+    ih = ctx.rplsh_fit(X, 4, 8, seed=7)
+    P = ctx.index_param(ih, 4, np.float32).reshape(32, 32)
+    np.testing.assert_allclose(P, o.generate_random_projections(7, 32, 32), rtol=2e-7, atol=0)
+    from abi import assert_index_matches
+
+    assert_index_matches(ctx.index_arrays(ih), o.fit_index(ctx.rplsh_hash(X, P, 4, 8), 8))
+    ctx.free_index(ih)
+
+
+def test_dtype_mismatch_is_an_error(ctx):
+    """bindings.cu:58-60, 75-77"""
+    X = np.random.default_rng(0).standard_normal((200, 16))
+    ih32 = ctx.rplsh_fit(X.astype(np.float32), 2, 4)
+    ih64 = ctx.rplsh_fit(X, 2, 4)
+    with pytest.raises(RuntimeError, match="fitted with float32, but query is float64"):
+        ctx.rplsh_query(X, ih32)
+    with pytest.raises(RuntimeError, match="fitted with float64, but query is float32"):
+        ctx.rplsh_query(X.astype(np.float32), ih64)
+    ctx.free_index(ih32)
+    ctx.free_index(ih64)
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_pslsh_fit_query_path(ctx, dtype):
+    _announce("pslsh_path", dtype.__name__)
+    n, d, T, H, nq, w = 5000, 128, 16, 8, 100, 4
+    X = np.random.default_rng(1234).standard_normal((n, d)).astype(dtype)
+    Q = (X[:nq] + 0.05 * np.random.default_rng(4321).standard_normal((nq, d))).astype(dtype)
+    P, b = o.generate_random_projections_biases(42, T * H, d, w, dtype)
+    from abi import assert_candidates_match, assert_index_matches
+
+    sig = ctx.pslsh_hash(X, P, b, T, H)
+    qsig = ctx.pslsh_hash(Q, P, b, T, H)
+    ih = ctx.pslsh_fit(X, T, H, w, seed=42, P=P, b=b)
+    exp_ix = o.fit_index(sig, H)
+    got_ix = ctx.index_arrays(ih)
+    assert_index_matches(got_ix, exp_ix)
+    assert got_ix["sig_nbytes"] == 4 * H and got_ix["window_size"] == w
+    got = ctx.pslsh_query(Q, ih)
+    assert_candidates_match(got, o.query_index(qsig, exp_ix))
+    assert got["n_total_candidates"] > 0
+    for bs in (10, 50):
+        bat = ctx.pslsh_query(Q, ih, batch_size=bs)
+        for k in ("indices", "offsets", "counts"):
+            np.testing.assert_array_equal(bat[k], got[k])
+    fq = ctx.pslsh_fit_query(X[:1000], T, H, w, seed=42, P=P, b=b)
+    ih2 = ctx.pslsh_fit(X[:1000], T, H, w, seed=42, P=P, b=b)
+    qq = ctx.pslsh_query(X[:1000], ih2)
+    for k in ("indices", "offsets", "counts"):
+        np.testing.assert_array_equal(fq[k], qq[k])
+    # seeded parameters follow the documented generator
+    ih3 = ctx.pslsh_fit(X[:100], T, H, w, seed=42)
+    np.testing.assert_allclose(ctx.index_param(ih3, 4, dtype), P.reshape(-1), rtol=3e-7)
+    np.testing.assert_allclose(ctx.index_param(ih3, 5, dtype), b, rtol=3e-7)
+    for h in (ih, ih2, ih3):
+        ctx.free_index(h)
+
+
+def test_minhash_fit_query_path(ctx):
+    _announce("minhash_path")
+    rng = np.random.default_rng(77)
+    n, d, T, H, nq = 4000, 2000, 32, 4, 100
+    indices, indptr = make_csr(rng, n, d, 30, empty_rows=(3, 9))
+    # queries: perturbed copies of rows so that buckets are hit
+    qrows = []
+    for i in range(nq):
+        r = indices[indptr[i]:indptr[i + 1]]
+        keep = r[rng.random(len(r)) > 0.1]
+        qrows.append(np.unique(np.concatenate([keep, rng.choice(d, 2)])))
+    qindptr = np.concatenate([[0], np.cumsum([len(r) for r in qrows])]).astype(np.int32)
+    qindices = np.concatenate(qrows).astype(np.int32)
+    A, B = o.generate_hash_integers(42, T * H)
+    from abi import assert_candidates_match, assert_index_matches
+
+    sig = o.minhash_hash(indices, indptr, A, B, T, H)       # exact integers: oracle signatures
+    qsig = o.minhash_hash(qindices, qindptr, A, B, T, H)
+    ih = ctx.minhash_fit(indices, indptr, d, T, H, seed=42, A=A, B=B)
+    exp_ix = o.fit_index(sig, H)
+    got_ix = ctx.index_arrays(ih)
+    assert_index_matches(got_ix, exp_ix)
+    assert got_ix["sig_nbytes"] == 4 * H
+    got = ctx.minhash_query(qindices, qindptr, ih)
+    assert_candidates_match(got, o.query_index(qsig, exp_ix))
+    assert got["n_total_candidates"] > nq // 2
+    fq = ctx.minhash_fit_query(indices, indptr, d, T, H, seed=42, A=A, B=B)
+    assert_candidates_match(fq, o.fit_query(sig, H))
+    # seeded coefficients follow the documented generator, bit for bit
+    ih2 = ctx.minhash_fit(indices, indptr, d, T, H, seed=42)
+    np.testing.assert_array_equal(ctx.index_param(ih2, 6, np.uint32), A)
+    np.testing.assert_array_equal(ctx.index_param(ih2, 7, np.uint32), B)
+    ctx.free_index(ih)
+    ctx.free_index(ih2)
