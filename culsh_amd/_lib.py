@@ -121,6 +121,14 @@ def load() -> C.CDLL:
         raise ImportError(
             f"{LIB_PATH} not found: build it with `make -C {os.path.join(_HERE, 'csrc')}` "
             "(hipcc, --offload-arch=gfx950). There is no CPU fallback.")
+    # A process can hold one HIP runtime.  PyTorch-ROCm ships its own libamdhip64 (same
+    # soname as the system one): importing torch first makes the loader resolve this
+    # library's dependency to that already-loaded runtime instead of opening a second one,
+    # which would leave whichever runtime initialises last without any visible GPU.
+    try:
+        import torch  # noqa: F401
+    except ImportError:
+        pass
     lib = C.CDLL(LIB_PATH)
     for name, argtypes in PROTOTYPES.items():
         fn = getattr(lib, name)
