@@ -59,6 +59,9 @@ _PP = C.POINTER(C.c_void_p)
 PROTOTYPES = {
     "culsh_ctx_create": [_I, _PP],
     "culsh_ctx_synchronize": [_P],
+    "culsh_profile_enable": [_P, _I],
+    "culsh_profile_reset": [_P],
+    "culsh_profile_get": [_P, _I, C.POINTER(C.c_char_p), C.POINTER(C.c_double), C.POINTER(C.c_int64)],
     "culsh_generate_projection_f32": [_U64, _I, _I, _P],
     "culsh_generate_projection_f64": [_U64, _I, _I, _P],
     "culsh_generate_pslsh_params_f32": [_U64, _I, _I, _I, _P, _P],
@@ -103,6 +106,7 @@ _SPECIAL = {
     "culsh_version": (C.c_char_p, []),
     "culsh_ctx_destroy": (None, [_P]),
     "culsh_ctx_stream": (_P, [_P]),
+    "culsh_profile_count": (C.c_int, [_P]),
     "culsh_index_free": (None, [_P]),
     "culsh_candidates_free": (None, [_P]),
     "culsh_candidates_device_ptr": (_P, [_P, _I]),

@@ -62,8 +62,52 @@ culsh_status arena_alloc(culsh_ctx* ctx, size_t bytes, void** out) {
     return CULSH_OK;
 }
 
+StageTimer::StageTimer(culsh_ctx* c, const char* name) : ctx(c) {
+    if (!c->profiling) return;
+    int stage = -1;
+    for (size_t i = 0; i < c->prof_stages.size(); ++i)
+        if (c->prof_stages[i].name == name) { stage = static_cast<int>(i); break; }
+    if (stage < 0) {
+        c->prof_stages.push_back({name, 0.0, 0});
+        stage = static_cast<int>(c->prof_stages.size()) - 1;
+    }
+    hipEvent_t ev[2];
+    for (auto& e : ev) {
+        if (!c->prof_pool.empty()) {
+            e = c->prof_pool.back();
+            c->prof_pool.pop_back();
+        } else if (hipEventCreate(&e) != hipSuccess) {
+            (void)hipGetLastError();
+            return;
+        }
+    }
+    (void)hipEventRecord(ev[0], c->stream);
+    c->prof_pending.push_back({stage, ev[0], ev[1]});
+    pending = static_cast<int>(c->prof_pending.size()) - 1;
+}
+
+StageTimer::~StageTimer() {
+    if (pending >= 0) (void)hipEventRecord(ctx->prof_pending[pending].stop, ctx->stream);
+}
+
+void profile_collect(culsh_ctx* ctx) {
+    for (auto& p : ctx->prof_pending) {
+        float ms = 0.f;
+        if (hipEventElapsedTime(&ms, p.start, p.stop) == hipSuccess) {
+            ctx->prof_stages[p.stage].total_ms += ms;
+            ctx->prof_stages[p.stage].launches += 1;
+        } else {
+            (void)hipGetLastError();
+        }
+        ctx->prof_pool.push_back(p.start);
+        ctx->prof_pool.push_back(p.stop);
+    }
+    ctx->prof_pending.clear();
+}
+
 culsh_status arena_end(culsh_ctx* ctx) {
     hipError_t e = hipStreamSynchronize(ctx->stream);
+    if (e == hipSuccess) profile_collect(ctx);
     for (void* p : ctx->overflow) (void)hipFree(p);
     ctx->overflow.clear();
     if (e != hipSuccess) {
@@ -262,7 +306,7 @@ static culsh_status concat_candidates(culsh_ctx* ctx, const std::vector<culsh_ca
             CULSH_HIP(hipMemcpyAsync(out->query_candidate_counts + q0, p->query_candidate_counts,
                                      p->n_queries * sizeof(uint64_t), hipMemcpyDeviceToDevice, ctx->stream));
             // offsets[1..] of the part, shifted by the running total (candidates.cuh:178-183)
-            hipLaunchKernelGGL(shift_offsets_kernel, dim3(div_up(p->n_queries, 256)), dim3(256), 0, ctx->stream,
+            CULSH_LAUNCH(ctx, shift_offsets_kernel, dim3(div_up(p->n_queries, 256)), dim3(256), 0, ctx->stream,
                                p->query_candidate_offsets + 1, out->query_candidate_offsets + q0 + 1,
                                static_cast<size_t>(p->n_queries), c0);
             CULSH_LAUNCH_CHECK();
@@ -530,6 +574,8 @@ void culsh_ctx_destroy(culsh_ctx* ctx) {
         (void)hipStreamSynchronize(ctx->stream);
         (void)hipStreamDestroy(ctx->stream);
     }
+    profile_collect(ctx);
+    for (hipEvent_t e : ctx->prof_pool) (void)hipEventDestroy(e);
     for (void* p : ctx->overflow) (void)hipFree(p);
     if (ctx->arena) (void)hipFree(ctx->arena);
     if (ctx->pinned) (void)hipHostFree(ctx->pinned);
@@ -543,6 +589,30 @@ culsh_status culsh_ctx_synchronize(culsh_ctx* ctx) {
 }
 
 void* culsh_ctx_stream(culsh_ctx* ctx) { return ctx ? static_cast<void*>(ctx->stream) : nullptr; }
+
+culsh_status culsh_profile_enable(culsh_ctx* ctx, int on) {
+    CULSH_REQUIRE(ctx, CULSH_ERR_INVALID, "null argument");
+    CULSH_HIP(hipStreamSynchronize(ctx->stream));
+    profile_collect(ctx);
+    ctx->profiling = on != 0;
+    return CULSH_OK;
+}
+culsh_status culsh_profile_reset(culsh_ctx* ctx) {
+    CULSH_REQUIRE(ctx, CULSH_ERR_INVALID, "null argument");
+    CULSH_HIP(hipStreamSynchronize(ctx->stream));
+    profile_collect(ctx);
+    ctx->prof_stages.clear();
+    return CULSH_OK;
+}
+int culsh_profile_count(const culsh_ctx* ctx) { return ctx ? static_cast<int>(ctx->prof_stages.size()) : 0; }
+culsh_status culsh_profile_get(const culsh_ctx* ctx, int i, const char** name, double* total_ms, int64_t* launches) {
+    CULSH_REQUIRE(ctx && name && total_ms && launches, CULSH_ERR_INVALID, "null argument");
+    CULSH_REQUIRE(i >= 0 && i < static_cast<int>(ctx->prof_stages.size()), CULSH_ERR_INVALID, "stage index out of range");
+    *name = ctx->prof_stages[i].name.c_str();
+    *total_ms = ctx->prof_stages[i].total_ms;
+    *launches = ctx->prof_stages[i].launches;
+    return CULSH_OK;
+}
 
 // ---- generators
 culsh_status culsh_generate_projection_f32(uint64_t seed, int n_rows, int d, float* P) {

@@ -75,6 +75,13 @@ struct culsh_ctx {
     uint64_t* pinned = nullptr;          // 64 x u64 pinned host words for D2H scalars
     int lds_max = 0;                     // max LDS bytes per workgroup
     int n_cus = 0;
+    // per-kernel timing with HIP events on `stream` (off unless enabled)
+    bool profiling = false;
+    struct ProfPending { int stage; hipEvent_t start, stop; };
+    struct ProfStage { std::string name; double total_ms = 0.0; long launches = 0; };
+    std::vector<ProfPending> prof_pending;
+    std::vector<hipEvent_t> prof_pool;
+    std::vector<ProfStage> prof_stages;
 };
 
 struct culsh_index {
@@ -131,6 +138,24 @@ struct ArenaScope {
     explicit ArenaScope(culsh_ctx* c) : ctx(c), begin_status(arena_begin(c)) {}
     ~ArenaScope() { arena_end(ctx); }
 };
+
+// Brackets the launches issued during its lifetime with two events on the context's stream
+// when profiling is enabled; elapsed times are folded into per-name totals at the next
+// end-of-call synchronisation.
+struct StageTimer {
+    culsh_ctx* ctx;
+    int pending = -1;
+    StageTimer(culsh_ctx* c, const char* name);
+    ~StageTimer();
+};
+void profile_collect(culsh_ctx* ctx);  // call with the stream idle
+
+// Kernel launch on the context's stream, timed under the kernel's name when profiling is on.
+#define CULSH_LAUNCH(ctx, kernel, ...)                    \
+    do {                                                  \
+        ::culsh_amd::StageTimer st_(ctx, #kernel);        \
+        hipLaunchKernelGGL(kernel, __VA_ARGS__);          \
+    } while (0)
 
 // Reads `count` (<= 64) device u64/u32 words into host memory; synchronises the stream.
 culsh_status read_back_u64(culsh_ctx* ctx, const uint64_t* dev, int count, uint64_t* host);

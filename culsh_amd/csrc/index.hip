@@ -120,7 +120,7 @@ culsh_status launch_sig_to_keys(culsh_ctx* ctx, const uint8_t* sig, size_t n_ite
     if (n_items == 0) return CULSH_OK;
     const size_t total = n_items * W;
     CULSH_REQUIRE(div_up(total, 256) < (1u << 31) && total / 256 < (1ull << 31), CULSH_ERR_LIMIT, "too many items");
-    hipLaunchKernelGGL(sig_to_keys_kernel, dim3(div_up(total, 256)), dim3(256), 0, ctx->stream, sig, n_items, S,
+    CULSH_LAUNCH(ctx, sig_to_keys_kernel, dim3(div_up(total, 256)), dim3(256), 0, ctx->stream, sig, n_items, S,
                        static_cast<int>(enc), W, keys);
     CULSH_LAUNCH_CHECK();
     return CULSH_OK;
@@ -131,7 +131,7 @@ culsh_status launch_keys_to_sig(culsh_ctx* ctx, const uint32_t* keys, size_t cou
     if (count == 0) return CULSH_OK;
     const size_t total = count * S;
     CULSH_REQUIRE(total / 256 < (1ull << 31), CULSH_ERR_LIMIT, "too many buckets");
-    hipLaunchKernelGGL(keys_to_sig_kernel, dim3(div_up(total, 256)), dim3(256), 0, ctx->stream, keys, count, S,
+    CULSH_LAUNCH(ctx, keys_to_sig_kernel, dim3(div_up(total, 256)), dim3(256), 0, ctx->stream, keys, count, S,
                        static_cast<int>(enc), W, sig);
     CULSH_LAUNCH_CHECK();
     return CULSH_OK;
@@ -146,7 +146,7 @@ culsh_status build_index_from_sorted(culsh_ctx* ctx, const uint32_t* sorted_keys
     uint64_t* tile_base = nullptr;
     CULSH_TRY(arena_alloc_t(ctx, tiles, &tile_counts));
     CULSH_TRY(arena_alloc_t(ctx, tiles + 1, &tile_base));
-    hipLaunchKernelGGL(count_heads_kernel, dim3(static_cast<unsigned>(tiles)), dim3(IB_THREADS), 0, ctx->stream,
+    CULSH_LAUNCH(ctx, count_heads_kernel, dim3(static_cast<unsigned>(tiles)), dim3(IB_THREADS), 0, ctx->stream,
                        sorted_keys, N, n, W, tile_counts);
     CULSH_LAUNCH_CHECK();
     CULSH_TRY(exclusive_scan_u64(ctx, tile_counts, tile_base, tiles));
@@ -166,7 +166,7 @@ culsh_status build_index_from_sorted(culsh_ctx* ctx, const uint32_t* sorted_keys
     CULSH_HIP(hipMalloc(&index->table_bucket_offsets, (static_cast<size_t>(T) + 1) * sizeof(int32_t)));
     CULSH_HIP(hipMalloc(&index->bucket_keys, std::max<size_t>(1, static_cast<size_t>(B) * W) * sizeof(uint32_t)));
     CULSH_HIP(hipMalloc(&index->all_bucket_signatures, std::max<size_t>(1, static_cast<size_t>(B) * S)));
-    hipLaunchKernelGGL(build_index_kernel, dim3(static_cast<unsigned>(tiles)), dim3(IB_THREADS), 0, ctx->stream,
+    CULSH_LAUNCH(ctx, build_index_kernel, dim3(static_cast<unsigned>(tiles)), dim3(IB_THREADS), 0, ctx->stream,
                        sorted_keys, rows_sorted_owned, N, n, T, W, tile_base, B, index->bucket_candidate_offsets,
                        index->bucket_keys, index->table_bucket_offsets, item_to_bucket_opt);
     CULSH_LAUNCH_CHECK();

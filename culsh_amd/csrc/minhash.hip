@@ -69,7 +69,7 @@ culsh_status launch_minhash(culsh_ctx* ctx, const int32_t* indices, const int32_
                             uint32_t* out) {
     CULSH_REQUIRE(indptr && A && B && out, CULSH_ERR_INVALID, "minhash: null pointer");
     CULSH_REQUIRE(n > 0 && T > 0 && H > 0, CULSH_ERR_INVALID, "minhash: sizes must be positive");
-    CULSH_REQUIRE(H <= 4096, CULSH_ERR_LIMIT, "minhash: n_hashes > 4096 is not supported");
+    CULSH_REQUIRE(H <= 384, CULSH_ERR_LIMIT, "minhash: n_hashes > 384 is not supported");
     const long long TH = static_cast<long long>(T) * H;
     CULSH_REQUIRE(TH < (1ll << 30), CULSH_ERR_LIMIT, "T*H too large");
     // hashes per LDS stage: whole tables, at most 12288 words (48 KiB) of staging
@@ -78,9 +78,9 @@ culsh_status launch_minhash(culsh_ctx* ctx, const int32_t* indices, const int32_
     const size_t lds = static_cast<size_t>(th_chunk) * RB * sizeof(uint32_t);
     dim3 grid((n + RB - 1) / RB), block(NTHREADS);
     if (as_keys)
-        hipLaunchKernelGGL(minhash_kernel<true>, grid, block, lds, ctx->stream, indices, indptr, A, B, n, T, H, th_chunk, out);
+        CULSH_LAUNCH(ctx, minhash_kernel<true>, grid, block, lds, ctx->stream, indices, indptr, A, B, n, T, H, th_chunk, out);
     else
-        hipLaunchKernelGGL(minhash_kernel<false>, grid, block, lds, ctx->stream, indices, indptr, A, B, n, T, H, th_chunk, out);
+        CULSH_LAUNCH(ctx, minhash_kernel<false>, grid, block, lds, ctx->stream, indices, indptr, A, B, n, T, H, th_chunk, out);
     CULSH_LAUNCH_CHECK();
     return CULSH_OK;
 }

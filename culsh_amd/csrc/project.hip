@@ -322,10 +322,10 @@ culsh_status launch_project_f32(culsh_ctx* ctx, const float* X, const float* P, 
     CULSH_REQUIRE(blocks < (1ll << 31), CULSH_ERR_LIMIT, "projection grid too large");
     dim3 grid(static_cast<unsigned>(blocks)), block(NTHREADS);
     switch (epi) {
-        case EPI_SIGN_KEYS: hipLaunchKernelGGL(project_f32_kernel<EPI_SIGN_KEYS>, grid, block, 0, ctx->stream, a); break;
-        case EPI_SIGN_BYTES: hipLaunchKernelGGL(project_f32_kernel<EPI_SIGN_BYTES>, grid, block, 0, ctx->stream, a); break;
-        case EPI_FLOOR_KEYS: hipLaunchKernelGGL(project_f32_kernel<EPI_FLOOR_KEYS>, grid, block, 0, ctx->stream, a); break;
-        case EPI_FLOOR_I32: hipLaunchKernelGGL(project_f32_kernel<EPI_FLOOR_I32>, grid, block, 0, ctx->stream, a); break;
+        case EPI_SIGN_KEYS: CULSH_LAUNCH(ctx, project_f32_kernel<EPI_SIGN_KEYS>, grid, block, 0, ctx->stream, a); break;
+        case EPI_SIGN_BYTES: CULSH_LAUNCH(ctx, project_f32_kernel<EPI_SIGN_BYTES>, grid, block, 0, ctx->stream, a); break;
+        case EPI_FLOOR_KEYS: CULSH_LAUNCH(ctx, project_f32_kernel<EPI_FLOOR_KEYS>, grid, block, 0, ctx->stream, a); break;
+        case EPI_FLOOR_I32: CULSH_LAUNCH(ctx, project_f32_kernel<EPI_FLOOR_I32>, grid, block, 0, ctx->stream, a); break;
     }
     CULSH_LAUNCH_CHECK();
     return CULSH_OK;
@@ -343,9 +343,9 @@ culsh_status launch_project_f64(culsh_ctx* ctx, const double* X, const double* P
     CULSH_REQUIRE(gy <= 65535, CULSH_ERR_LIMIT, "T*H too large for the fp64 projection grid");
     dim3 grid((n + DT - 1) / DT, static_cast<unsigned>(gy)), block(256);
     if (epi == EPI_SIGN_BYTES)
-        hipLaunchKernelGGL(project_f64_kernel<EPI_SIGN_BYTES>, grid, block, 0, ctx->stream, X, P, b, out, n, d, T, H);
+        CULSH_LAUNCH(ctx, project_f64_kernel<EPI_SIGN_BYTES>, grid, block, 0, ctx->stream, X, P, b, out, n, d, T, H);
     else
-        hipLaunchKernelGGL(project_f64_kernel<EPI_FLOOR_I32>, grid, block, 0, ctx->stream, X, P, b, out, n, d, T, H);
+        CULSH_LAUNCH(ctx, project_f64_kernel<EPI_FLOOR_I32>, grid, block, 0, ctx->stream, X, P, b, out, n, d, T, H);
     CULSH_LAUNCH_CHECK();
     return CULSH_OK;
 }

@@ -150,7 +150,7 @@ culsh_status launch_find_matching_buckets(culsh_ctx* ctx, const uint32_t* q_keys
                                           const culsh_index* index, int32_t* matched) {
     const size_t pairs = static_cast<size_t>(n_queries) * index->n_hash_tables;
     CULSH_REQUIRE(pairs / 256 < (1ull << 31), CULSH_ERR_LIMIT, "too many (query, table) pairs");
-    hipLaunchKernelGGL(lookup_kernel, dim3(div_up(pairs, 256)), dim3(256), 0, ctx->stream, q_keys,
+    CULSH_LAUNCH(ctx, lookup_kernel, dim3(div_up(pairs, 256)), dim3(256), 0, ctx->stream, q_keys,
                        index->bucket_keys, index->table_bucket_offsets, n_queries, index->n_hash_tables,
                        index->key_w, matched);
     CULSH_LAUNCH_CHECK();
@@ -203,7 +203,7 @@ culsh_status query_from_matched(culsh_ctx* ctx, const int32_t* matched, int n_qu
     a.counts = out->query_candidate_counts;
     a.offsets = nullptr;
     a.out = nullptr;
-    hipLaunchKernelGGL(dedup_kernel<false>, dim3(n_queries), dim3(DD_THREADS), lds_bytes, ctx->stream, a);
+    CULSH_LAUNCH(ctx, dedup_kernel<false>, dim3(n_queries), dim3(DD_THREADS), lds_bytes, ctx->stream, a);
     CULSH_LAUNCH_CHECK();
     CULSH_TRY(exclusive_scan_u64(ctx, out->query_candidate_counts, out->query_candidate_offsets, n_queries));
     uint64_t U = 0;
@@ -216,7 +216,7 @@ culsh_status query_from_matched(culsh_ctx* ctx, const int32_t* matched, int n_qu
     CULSH_HIP(hipMalloc(&out->query_candidate_indices, U * sizeof(int32_t)));
     a.offsets = out->query_candidate_offsets;
     a.out = out->query_candidate_indices;
-    hipLaunchKernelGGL(dedup_kernel<true>, dim3(n_queries), dim3(DD_THREADS), lds_bytes, ctx->stream, a);
+    CULSH_LAUNCH(ctx, dedup_kernel<true>, dim3(n_queries), dim3(DD_THREADS), lds_bytes, ctx->stream, a);
     CULSH_LAUNCH_CHECK();
     return CULSH_OK;
 }

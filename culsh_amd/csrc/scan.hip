@@ -76,12 +76,12 @@ culsh_status exclusive_scan_u64(culsh_ctx* ctx, const uint64_t* in, uint64_t* ou
     CULSH_REQUIRE(tiles < (1ull << 31), CULSH_ERR_LIMIT, "scan: input too large");
     uint64_t* sums = nullptr;
     CULSH_TRY(arena_alloc_t(ctx, tiles, &sums));
-    hipLaunchKernelGGL(tile_sums_kernel, dim3(static_cast<unsigned>(tiles)), dim3(SCAN_THREADS), 0,
+    CULSH_LAUNCH(ctx, tile_sums_kernel, dim3(static_cast<unsigned>(tiles)), dim3(SCAN_THREADS), 0,
                        ctx->stream, in, n, sums);
     CULSH_LAUNCH_CHECK();
-    hipLaunchKernelGGL(spine_scan_kernel, dim3(1), dim3(1024), 0, ctx->stream, sums, tiles, out + n);
+    CULSH_LAUNCH(ctx, spine_scan_kernel, dim3(1), dim3(1024), 0, ctx->stream, sums, tiles, out + n);
     CULSH_LAUNCH_CHECK();
-    hipLaunchKernelGGL(tile_scan_kernel, dim3(static_cast<unsigned>(tiles)), dim3(SCAN_THREADS), 0,
+    CULSH_LAUNCH(ctx, tile_scan_kernel, dim3(static_cast<unsigned>(tiles)), dim3(SCAN_THREADS), 0,
                        ctx->stream, in, n, sums, out);
     CULSH_LAUNCH_CHECK();
     return CULSH_OK;

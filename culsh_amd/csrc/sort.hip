@@ -168,7 +168,7 @@ culsh_status sort_tables(culsh_ctx* ctx, uint32_t* keys_in, uint32_t* keys_tmp, 
     CULSH_HIP(hipMemsetAsync(vary_dev, 0, W * sizeof(uint32_t), ctx->stream));
     {
         const unsigned bx = std::max(1u, std::min(64u, div_up(n, 256 * 8)));
-        hipLaunchKernelGGL(varying_bits_kernel, dim3(bx, T), dim3(256), 0, ctx->stream, keys_in, n, W, vary_dev);
+        CULSH_LAUNCH(ctx, varying_bits_kernel, dim3(bx, T), dim3(256), 0, ctx->stream, keys_in, n, W, vary_dev);
         CULSH_LAUNCH_CHECK();
     }
     uint32_t vary[64];
@@ -182,7 +182,7 @@ culsh_status sort_tables(culsh_ctx* ctx, uint32_t* keys_in, uint32_t* keys_tmp, 
             if ((vary[w] >> (8 * byte)) & 0xFFu) passes.push_back({w, 8 * byte});
 
     if (passes.empty()) {  // every table holds one distinct key: identity order
-        hipLaunchKernelGGL(iota_rows_kernel, dim3(div_up(N, 256)), dim3(256), 0, ctx->stream, rows_out, n, N);
+        CULSH_LAUNCH(ctx, iota_rows_kernel, dim3(div_up(N, 256)), dim3(256), 0, ctx->stream, rows_out, n, N);
         CULSH_LAUNCH_CHECK();
         *sorted_keys = keys_in;
         return CULSH_OK;
@@ -198,16 +198,16 @@ culsh_status sort_tables(culsh_ctx* ctx, uint32_t* keys_in, uint32_t* keys_tmp, 
         // the last pass must land in rows_out
         int32_t* rout = ((np - 1 - p) % 2 == 0) ? rows_out : rows_tmp;
         const dim3 grid(tiles, T);
-        hipLaunchKernelGGL(radix_hist_kernel, grid, dim3(SORT_THREADS), 0, ctx->stream, kin, n, W,
+        CULSH_LAUNCH(ctx, radix_hist_kernel, grid, dim3(SORT_THREADS), 0, ctx->stream, kin, n, W,
                            passes[p].word, passes[p].shift, tiles, hist);
         CULSH_LAUNCH_CHECK();
-        hipLaunchKernelGGL(radix_scan_kernel, dim3(T), dim3(1024), 0, ctx->stream, hist, tiles);
+        CULSH_LAUNCH(ctx, radix_scan_kernel, dim3(T), dim3(1024), 0, ctx->stream, hist, tiles);
         CULSH_LAUNCH_CHECK();
         if (W == 1)
-            hipLaunchKernelGGL(radix_scatter_kernel<true>, grid, dim3(SORT_THREADS), 0, ctx->stream, kin, rin,
+            CULSH_LAUNCH(ctx, radix_scatter_kernel<true>, grid, dim3(SORT_THREADS), 0, ctx->stream, kin, rin,
                                kout, rout, hist, n, W, passes[p].word, passes[p].shift, tiles);
         else
-            hipLaunchKernelGGL(radix_scatter_kernel<false>, grid, dim3(SORT_THREADS), 0, ctx->stream, kin, rin,
+            CULSH_LAUNCH(ctx, radix_scatter_kernel<false>, grid, dim3(SORT_THREADS), 0, ctx->stream, kin, rin,
                                kout, rout, hist, n, W, passes[p].word, passes[p].shift, tiles);
         CULSH_LAUNCH_CHECK();
         std::swap(kin, kout);

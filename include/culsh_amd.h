@@ -94,6 +94,15 @@ culsh_status culsh_ctx_synchronize(culsh_ctx* ctx);
 /* The context's hipStream_t, for callers that want to order their own work after it. */
 void* culsh_ctx_stream(culsh_ctx* ctx);
 
+/* ---- per-kernel timing ------------------------------------------------------------------
+ * No counterpart in the reference (it has wall-clock timing only, cuda/benchmark/bench.cu:144-163).
+ * When enabled, every kernel launch is bracketed by two HIP events on the context's stream;
+ * totals per kernel name are available after the call that launched them has returned. */
+culsh_status culsh_profile_enable(culsh_ctx* ctx, int on);
+culsh_status culsh_profile_reset(culsh_ctx* ctx);
+int culsh_profile_count(const culsh_ctx* ctx);
+culsh_status culsh_profile_get(const culsh_ctx* ctx, int i, const char** name, double* total_ms, int64_t* launches);
+
 /* ---- seeded hash parameters (host side) -------------------------------------------------
  * Role of generate_random_projections (rplsh/hash.cuh:58-78),
  * generate_random_projections_biases (pslsh/hash.cuh:59-89) and generate_hash_integers
