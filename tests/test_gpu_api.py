@@ -1,0 +1,275 @@
+"""
+GPU tests of the public Python API (culsh_amd.RPLSH / PStableLSH / MinHashLSH), written
+after the reference's own test-suite (python/tests/test_rplsh.py, test_pslsh.py,
+test_minhash.py): recall against a CPU LSH with independent random parameters, save/load
+round trips, fit_query == fit + query, batched == unbatched, auto window size.
+"""
+
+import os
+
+import numpy as np
+import pytest
+import scipy.sparse
+
+from oracle import culsh_oracle as o
+
+pytestmark = pytest.mark.gpu
+
+
+def dense(n, d, dtype, seed=42):
+    return np.random.default_rng(seed).standard_normal((n, d)).astype(dtype)
+
+
+def sparse(n, d, density, seed=42):
+    rs = np.random.RandomState(seed)
+    X = scipy.sparse.random(n, d, density=density, format="csr", dtype=np.float32, random_state=rs)
+    X.data[:] = 1.0
+    X.indices = X.indices.astype(np.int32)
+    X.indptr = X.indptr.astype(np.int32)
+    return X
+
+
+def recall_at_k(X, n_eval, k, indices, offsets, topk):
+    rec = []
+    for q in range(n_eval):
+        got = indices[int(offsets[q]):int(offsets[q + 1])]
+        rec.append(len(np.intersect1d(got, topk(q))) / k)
+    return float(np.mean(rec))
+
+
+def oracle_recall(sig, n_eval, k, H, topk):
+    c = o.query_index(sig[:, :n_eval], o.fit_index(sig, H))
+    return recall_at_k(None, n_eval, k, c.query_candidate_indices, c.query_candidate_offsets, topk)
+
+
+# ---------------------------------------------------------------- RPLSH
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("n_hash_tables", [8, 32, 64])
+@pytest.mark.parametrize("n_hashes", [8, 16])
+def test_rplsh_recall_vs_cpu_lsh(dtype, n_hash_tables, n_hashes):
+    """python/tests/test_rplsh.py:27-73: mean recall@20 of 50 self-queries within 0.05 of a
+    CPU LSH that draws its own projections."""
+    from culsh_amd import RPLSH
+
+    n, d, n_eval, k = 1000, 100, 50, 20
+    X = dense(n, d, dtype)
+    Xn = X / np.linalg.norm(X, axis=1, keepdims=True)
+
+    def topk(q):
+        return np.argsort(Xn @ Xn[q])[-k:]
+
+    P = np.random.default_rng(7).standard_normal((n_hash_tables * n_hashes, d)).astype(dtype)
+    ref = oracle_recall(o.rplsh_hash(X, P, n_hash_tables, n_hashes), n_eval, k, n_hashes, topk)
+    cand = RPLSH(n_hash_tables=n_hash_tables, n_hashes=n_hashes, seed=42).fit_query(X)
+    got = recall_at_k(X, n_eval, k, cand.get_indices(), cand.get_offsets(), topk)
+    assert abs(got - ref) < 0.05 and got <= 1.0
+    assert cand.n_queries == n and cand.get_counts().dtype == np.uint64
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("as_torch", [False, True])
+def test_rplsh_save_load(tmp_path, dtype, as_torch):
+    """python/tests/test_rplsh.py:76-142"""
+    import torch
+
+    from culsh_amd import RPLSH, RPLSHModel
+
+    X = dense(1000, 64, dtype)
+    Xin = torch.from_numpy(X).cuda() if as_torch else X
+    model = RPLSH(n_hash_tables=16, n_hashes=8, seed=42).fit(Xin)
+    path = os.path.join(tmp_path, "rplsh_model.npz")
+    model.save(path)
+    loaded = RPLSHModel.load(path)
+    assert (loaded.n_hash_tables, loaded.n_hashes, loaded.n_features) == (16, 8, 64)
+    for attr in ("n_total_candidates", "n_total_buckets", "n_hash_tables", "n_hashes", "sig_nbytes", "n_features",
+                 "seed", "is_double"):
+        assert getattr(loaded.index, attr) == getattr(model.index, attr), attr
+    assert model.index.sig_nbytes == 8 and model.index.is_double == (dtype == np.float64)
+    for getter in ("get_candidate_indices", "get_bucket_signatures", "get_bucket_candidate_offsets",
+                   "get_table_bucket_offsets", "get_projection_matrix"):
+        np.testing.assert_array_equal(getattr(loaded.index, getter)(), getattr(model.index, getter)())
+    assert set(np.unique(model.index.get_bucket_signatures())) <= {0, 1}
+    assert model.index.size_bytes() == loaded.index.size_bytes() > 0
+    a, b = model.query(Xin[:100]), loaded.query(Xin[:100])
+    np.testing.assert_array_equal(a.get_indices(), b.get_indices())
+    np.testing.assert_array_equal(a.get_offsets(), b.get_offsets())
+    data = np.load(path)
+    assert sorted(data.files) == sorted([
+        "n_hash_tables", "n_hashes", "n_features", "n_total_candidates", "n_total_buckets", "seed", "sig_nbytes",
+        "is_double", "candidate_indices", "bucket_signatures", "bucket_candidate_offsets", "table_bucket_offsets",
+        "projection"])
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_rplsh_fit_query_equals_fit_then_query(dtype):
+    """python/tests/test_rplsh.py:145-174"""
+    from culsh_amd import RPLSH
+
+    X = dense(1000, 64, dtype)
+    lsh = RPLSH(n_hash_tables=16, n_hashes=8, seed=42)
+    a = lsh.fit_query(X)
+    b = lsh.fit(X).query(X)
+    np.testing.assert_array_equal(a.get_indices(), b.get_indices())
+    np.testing.assert_array_equal(a.get_offsets(), b.get_offsets())
+    c = lsh.fit_query(X, batch_size=300)      # falls back to fit + batched query
+    np.testing.assert_array_equal(a.get_indices(), c.get_indices())
+
+
+@pytest.mark.parametrize("batch_size", [10, 50, 100])
+def test_rplsh_batched_query(batch_size):
+    """python/tests/test_rplsh.py:177-209"""
+    from culsh_amd import RPLSH
+
+    X, Q = dense(1000, 64, np.float32), dense(100, 64, np.float32, seed=1)
+    model = RPLSH(n_hash_tables=16, n_hashes=8, seed=42).fit(X)
+    a, b = model.query(Q), model.query(Q, batch_size=batch_size)
+    np.testing.assert_array_equal(a.get_indices(), b.get_indices())
+    np.testing.assert_array_equal(a.get_offsets(), b.get_offsets())
+    np.testing.assert_array_equal(a.get_counts(), b.get_counts())
+
+
+def test_rplsh_errors_and_device_getters():
+    import torch
+
+    from culsh_amd import RPLSH
+
+    X = dense(500, 32, np.float32)
+    model = RPLSH(4, 4, seed=1).fit(X)
+    with pytest.raises(ValueError, match=r"Query features \(16\) != fitted features \(32\)"):
+        model.query(dense(10, 16, np.float32))
+    with pytest.raises(TypeError, match="Unsupported dtype"):
+        model.query(X.astype(np.float16))
+    with pytest.raises(TypeError, match="Unsupported dtype"):
+        RPLSH(4, 4).fit(X.astype(np.int32))
+    with pytest.raises(RuntimeError, match="fitted with float32, but query is float64"):
+        model.query(X.astype(np.float64))
+    with pytest.raises(ValueError, match="Expected 2D array"):
+        model.query(X[0])
+    c = model.query(X[:20])
+    t = c.get_indices(as_torch=True)
+    assert t.is_cuda and t.dtype == torch.int32
+    np.testing.assert_array_equal(t.cpu().numpy(), c.get_indices())
+    np.testing.assert_array_equal(c.get_offsets(as_torch=True).cpu().numpy().view(np.uint64), c.get_offsets())
+    assert not c.empty() and c.n_total_candidates == len(c.get_indices())
+    # non-contiguous input is made contiguous
+    Xt = torch.from_numpy(np.ascontiguousarray(X.T)).cuda().T
+    assert not Xt.is_contiguous()
+    np.testing.assert_array_equal(RPLSH(4, 4, seed=1).fit(Xt).index.get_candidate_indices(),
+                                  model.index.get_candidate_indices())
+
+
+# ---------------------------------------------------------------- p-stable
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("window_size", [4, 8])
+def test_pslsh_recall_vs_cpu_lsh(dtype, window_size):
+    """python/tests/test_pslsh.py:26-85"""
+    from culsh_amd import PStableLSH
+
+    n, d, n_eval, k, T, H = 1000, 100, 50, 20, 32, 4
+    X = dense(n, d, dtype)
+
+    def topk(q):
+        return np.argsort(np.linalg.norm(X - X[q], axis=1))[:k]
+
+    rng = np.random.default_rng(7)
+    P = (rng.standard_normal((T * H, d)) / window_size).astype(dtype)
+    b = rng.uniform(0, 1, size=T * H).astype(dtype)
+    ref = oracle_recall(o.pslsh_hash(X, P, b, T, H), n_eval, k, H, topk)
+    cand = PStableLSH(n_hash_tables=T, n_hashes=H, window_size=window_size, seed=42).fit_query(X)
+    got = recall_at_k(X, n_eval, k, cand.get_indices(), cand.get_offsets(), topk)
+    assert abs(got - ref) < 0.05 and got <= 1.0
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_pslsh_save_load_fit_query_batched(tmp_path, dtype):
+    """python/tests/test_pslsh.py:88-240"""
+    from culsh_amd import PStableLSH, PStableLSHModel
+
+    X = dense(1000, 64, dtype)
+    lsh = PStableLSH(n_hash_tables=16, n_hashes=4, window_size=4, seed=42)
+    model = lsh.fit(X)
+    path = os.path.join(tmp_path, "pslsh_model.npz")
+    model.save(path)
+    loaded = PStableLSHModel.load(path)
+    assert loaded.window_size == 4 and model.index.sig_nbytes == 16
+    for getter in ("get_candidate_indices", "get_bucket_signatures", "get_bucket_candidate_offsets",
+                   "get_table_bucket_offsets", "get_projection_matrix", "get_bias"):
+        np.testing.assert_array_equal(getattr(loaded.index, getter)(), getattr(model.index, getter)())
+    bias = model.index.get_bias()
+    assert bias.dtype == dtype and bias.min() > 0 and bias.max() <= 1
+    a, b = model.query(X[:100]), loaded.query(X[:100])
+    np.testing.assert_array_equal(a.get_indices(), b.get_indices())
+    fq = lsh.fit_query(X)
+    full = model.query(X)
+    np.testing.assert_array_equal(fq.get_indices(), full.get_indices())
+    np.testing.assert_array_equal(fq.get_offsets(), full.get_offsets())
+    for bs in (10, 50, 100):
+        c = model.query(X[:100], batch_size=bs)
+        np.testing.assert_array_equal(a.get_indices(), c.get_indices())
+        np.testing.assert_array_equal(a.get_offsets(), c.get_offsets())
+    assert "window_size" in np.load(path).files and "bias" in np.load(path).files
+
+
+def test_pslsh_auto_window_size():
+    """python/tests/test_pslsh.py:243-255"""
+    import torch
+
+    from culsh_amd import PStableLSH
+
+    X = dense(1000, 32, np.float32)
+    X = (100.0 * X / np.linalg.norm(X, axis=1, keepdims=True)).astype(np.float32)
+    assert PStableLSH._estimate_window_size(torch.from_numpy(X).cuda()) in (99, 100)
+    model = PStableLSH(n_hash_tables=4, n_hashes=2, window_size="auto", seed=3).fit(X)
+    assert model.window_size in (99, 100)
+
+
+# ---------------------------------------------------------------- MinHash
+@pytest.mark.parametrize("density", [0.1, 0.5])
+def test_minhash_recall_vs_cpu_lsh(density):
+    """python/tests/test_minhash.py:36-82"""
+    from culsh_amd import MinHashLSH
+
+    n, d, n_eval, k, T, H = 1000, 100, 50, 20, 32, 2
+    X = sparse(n, d, density)
+    Xd = (X.toarray() > 0)
+
+    def topk(q):
+        inter = (Xd & Xd[q]).sum(1)
+        union = (Xd | Xd[q]).sum(1)
+        return np.argsort(inter / np.maximum(union, 1))[-k:]
+
+    A, B = o.generate_hash_integers(7, T * H)
+    ref = oracle_recall(o.minhash_hash(X.indices, X.indptr, A, B, T, H), n_eval, k, H, topk)
+    cand = MinHashLSH(n_hash_tables=T, n_hashes=H, seed=42).fit_query(X)
+    got = recall_at_k(X, n_eval, k, cand.get_indices(), cand.get_offsets(), topk)
+    assert abs(got - ref) < 0.05 and got <= 1.0
+
+
+def test_minhash_save_load_and_fit_query(tmp_path):
+    """python/tests/test_minhash.py:85-183"""
+    from culsh_amd import MinHashLSH, MinHashLSHModel
+
+    X = sparse(1000, 200, 0.05)
+    lsh = MinHashLSH(n_hash_tables=16, n_hashes=4, seed=42)
+    model = lsh.fit(X)
+    path = os.path.join(tmp_path, "minhash_model.npz")
+    model.save(path)
+    loaded = MinHashLSHModel.load(path)
+    for getter in ("get_candidate_indices", "get_bucket_signatures", "get_bucket_candidate_offsets",
+                   "get_table_bucket_offsets", "get_hash_a", "get_hash_b"):
+        np.testing.assert_array_equal(getattr(loaded.index, getter)(), getattr(model.index, getter)())
+    assert model.index.sig_nbytes == 16 and model.index.get_hash_a().dtype == np.uint32
+    a, b = model.query(X[:100]), loaded.query(X[:100])
+    np.testing.assert_array_equal(a.get_indices(), b.get_indices())
+    fq, full = lsh.fit_query(X), model.query(X)
+    np.testing.assert_array_equal(fq.get_indices(), full.get_indices())
+    np.testing.assert_array_equal(fq.get_offsets(), full.get_offsets())
+    # signatures follow the documented definition for the seeded coefficients
+    A, B = model.index.get_hash_a(), model.index.get_hash_b()
+    exp = o.fit_index(o.minhash_hash(X.indices, X.indptr, A, B, 16, 4), 4)
+    np.testing.assert_array_equal(model.index.get_candidate_indices(), exp.all_candidate_indices)
+    np.testing.assert_array_equal(model.index.get_bucket_signatures(), exp.all_bucket_signatures)
+    X64 = X.copy()
+    X64.indices = X64.indices.astype(np.int64)
+    with pytest.raises(ValueError, match="requires int32 indices"):
+        lsh.fit(X64)
