@@ -27,6 +27,19 @@ __device__ __forceinline__ T wave_sum(T v) {
     return v;
 }
 
+// Inclusive prefix sum over the 64 lanes with DPP row shifts and row broadcasts (VALU only,
+// no LDS traffic).  All 64 lanes must be active.
+__device__ __forceinline__ uint32_t wave_inclusive_sum_dpp(uint32_t v) {
+    int x = static_cast<int>(v);
+    x += __builtin_amdgcn_update_dpp(0, x, 0x111, 0xf, 0xf, false);  // row_shr:1
+    x += __builtin_amdgcn_update_dpp(0, x, 0x112, 0xf, 0xf, false);  // row_shr:2
+    x += __builtin_amdgcn_update_dpp(0, x, 0x114, 0xf, 0xf, false);  // row_shr:4
+    x += __builtin_amdgcn_update_dpp(0, x, 0x118, 0xf, 0xf, false);  // row_shr:8
+    x += __builtin_amdgcn_update_dpp(0, x, 0x142, 0xa, 0xf, false);  // row_bcast:15 into rows 1 and 3
+    x += __builtin_amdgcn_update_dpp(0, x, 0x143, 0xc, 0xf, false);  // row_bcast:31 into rows 2 and 3
+    return static_cast<uint32_t>(x);
+}
+
 // Exclusive prefix sum over the workgroup (blockDim.x a multiple of 64, at most 1024).
 // `scratch` holds 17 words of type T in LDS.  Returns this thread's exclusive prefix and
 // stores the workgroup total in *total.  Contains three barriers; all threads must call it.

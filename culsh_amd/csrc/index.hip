@@ -26,14 +26,39 @@ __device__ __forceinline__ uint32_t is_head(const uint32_t* __restrict__ keys, s
     return diff != 0u;
 }
 
+// Flags of the IB_ITEMS consecutive items owned by one thread.  One-word keys of a full
+// run are fetched with two 16-byte loads plus the predecessor's key.
+__device__ __forceinline__ uint64_t thread_flags(const uint32_t* __restrict__ keys, size_t base, size_t N, int n,
+                                                 int W, uint32_t (&flag)[IB_ITEMS]) {
+    uint64_t c = 0;
+    if (W == 1 && base + IB_ITEMS <= N) {
+        static_assert(IB_ITEMS == 8, "two uint4 loads cover the thread's items");
+        const uint4 a = *reinterpret_cast<const uint4*>(keys + base);
+        const uint4 b = *reinterpret_cast<const uint4*>(keys + base + 4);
+        const uint32_t k[9] = {base ? keys[base - 1] : 0u, a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+        uint32_t r = static_cast<uint32_t>(base % n);  // position inside the table
+#pragma unroll
+        for (int i = 0; i < IB_ITEMS; ++i) {
+            flag[i] = (r == 0u) || (k[i + 1] != k[i]);
+            if (++r == static_cast<uint32_t>(n)) r = 0u;
+            c += flag[i];
+        }
+        return c;
+    }
+#pragma unroll
+    for (int i = 0; i < IB_ITEMS; ++i) {
+        flag[i] = (base + i < N) ? is_head(keys, base + i, n, W) : 0u;
+        c += flag[i];
+    }
+    return c;
+}
+
 __global__ __launch_bounds__(IB_THREADS) void count_heads_kernel(const uint32_t* __restrict__ keys, size_t N,
                                                                 int n, int W, uint64_t* __restrict__ tile_counts) {
     __shared__ uint64_t scratch[17];
     const size_t base = static_cast<size_t>(blockIdx.x) * IB_TILE + threadIdx.x * IB_ITEMS;
-    uint64_t c = 0;
-#pragma unroll
-    for (int i = 0; i < IB_ITEMS; ++i)
-        if (base + i < N) c += is_head(keys, base + i, n, W);
+    uint32_t flag[IB_ITEMS];
+    const uint64_t c = thread_flags(keys, base, N, n, W, flag);
     uint64_t total;
     block_exclusive_sum(c, scratch, &total);
     if (threadIdx.x == 0) tile_counts[blockIdx.x] = total;
@@ -47,12 +72,7 @@ __global__ __launch_bounds__(IB_THREADS) void build_index_kernel(
     __shared__ uint64_t scratch[17];
     const size_t base = static_cast<size_t>(blockIdx.x) * IB_TILE + threadIdx.x * IB_ITEMS;
     uint32_t flag[IB_ITEMS];
-    uint64_t c = 0;
-#pragma unroll
-    for (int i = 0; i < IB_ITEMS; ++i) {
-        flag[i] = (base + i < N) ? is_head(keys, base + i, n, W) : 0u;
-        c += flag[i];
-    }
+    const uint64_t c = thread_flags(keys, base, N, n, W, flag);
     uint64_t total;
     uint64_t run = tile_base[blockIdx.x] + block_exclusive_sum(c, scratch, &total);
 #pragma unroll

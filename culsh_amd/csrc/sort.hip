@@ -21,6 +21,13 @@ constexpr int SORT_ITEMS = 16;
 constexpr int SORT_TILE = SORT_THREADS * SORT_ITEMS;  // 4096 items per workgroup
 
 // vary[w] |= key[t][i][w] ^ key[t][0][w]
+__device__ __forceinline__ void publish_vary(uint32_t acc, uint32_t* __restrict__ slot) {
+#pragma unroll
+    for (int d = 32; d > 0; d >>= 1) acc |= __shfl_xor(acc, d, 64);
+    // most wavefronts add nothing new once a few have reported: skip their atomics
+    if ((threadIdx.x & 63) == 0 && (acc & ~__atomic_load_n(slot, __ATOMIC_RELAXED))) atomicOr(slot, acc);
+}
+
 __global__ __launch_bounds__(256) void varying_bits_kernel(const uint32_t* __restrict__ keys, int n,
                                                           int W, uint32_t* __restrict__ vary) {
     const int t = blockIdx.y;
@@ -31,12 +38,42 @@ __global__ __launch_bounds__(256) void varying_bits_kernel(const uint32_t* __res
     for (int w = 0; w < W; ++w) {
         const uint32_t first = tk[w];
         uint32_t acc = 0;
+#pragma unroll 4
         for (size_t i = (static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x) * W + w; i < total;
              i += stride)
             acc |= tk[i] ^ first;
-#pragma unroll
-        for (int d = 32; d > 0; d >>= 1) acc |= __shfl_xor(acc, d, 64);
-        if ((threadIdx.x & 63) == 0 && acc) atomicOr(&vary[w], acc);
+        publish_vary(acc, &vary[w]);
+    }
+}
+
+// Same for W in {1, 2, 4} with 16-byte loads (component c of a uint4 is word position c % W).
+__global__ __launch_bounds__(256) void varying_bits_vec_kernel(const uint32_t* __restrict__ keys, int n,
+                                                              int W, uint32_t* __restrict__ vary) {
+    const int t = blockIdx.y;
+    const uint32_t* tk = keys + static_cast<size_t>(t) * n * W;
+    const size_t nvec = static_cast<size_t>(n) * W / 4;  // caller guarantees n*W % 4 == 0
+    const uint4* tv = reinterpret_cast<const uint4*>(tk);
+    const uint32_t f0 = tk[0], f1 = tk[1 % W], f2 = tk[2 % W], f3 = tk[3 % W];
+    uint32_t a0 = 0, a1 = 0, a2 = 0, a3 = 0;
+    const size_t stride = static_cast<size_t>(gridDim.x) * blockDim.x;
+#pragma unroll 4
+    for (size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < nvec; i += stride) {
+        const uint4 v = tv[i];
+        a0 |= v.x ^ f0;
+        a1 |= v.y ^ f1;
+        a2 |= v.z ^ f2;
+        a3 |= v.w ^ f3;
+    }
+    if (W == 1) {
+        publish_vary(a0 | a1 | a2 | a3, &vary[0]);
+    } else if (W == 2) {
+        publish_vary(a0 | a2, &vary[0]);
+        publish_vary(a1 | a3, &vary[1]);
+    } else {
+        publish_vary(a0, &vary[0]);
+        publish_vary(a1, &vary[1]);
+        publish_vary(a2, &vary[2]);
+        publish_vary(a3, &vary[3]);
     }
 }
 
@@ -47,34 +84,57 @@ __global__ __launch_bounds__(256) void iota_rows_kernel(int32_t* __restrict__ ro
 
 __global__ __launch_bounds__(SORT_THREADS) void radix_hist_kernel(const uint32_t* __restrict__ keys, int n,
                                                                  int W, int word, int shift, int tiles,
-                                                                 uint32_t* __restrict__ hist) {
-    __shared__ uint32_t h[256];
-    const int tile = blockIdx.x, t = blockIdx.y;
-    h[threadIdx.x] = 0;
+                                                                 uint32_t* __restrict__ hist,
+                                                                 uint32_t* __restrict__ dtot) {
+    __shared__ uint32_t h[SORT_THREADS / 64][256];  // one copy per wavefront: fewer same-bank atomics
+    const int tile = blockIdx.x, t = blockIdx.y, wave = threadIdx.x >> 6;
+    for (int i = threadIdx.x; i < (SORT_THREADS / 64) * 256; i += SORT_THREADS) (&h[0][0])[i] = 0;
     __syncthreads();
     const uint32_t* tk = keys + static_cast<size_t>(t) * n * W;
-#pragma unroll 4
+    uint32_t k[SORT_ITEMS];
+#pragma unroll
     for (int j = 0; j < SORT_ITEMS; ++j) {
         const int idx = tile * SORT_TILE + j * SORT_THREADS + threadIdx.x;
-        if (idx < n) atomicAdd(&h[(tk[static_cast<size_t>(idx) * W + word] >> shift) & 255u], 1u);
+        k[j] = (idx < n) ? tk[static_cast<size_t>(idx) * W + word] : 0u;
+    }
+#pragma unroll
+    for (int j = 0; j < SORT_ITEMS; ++j) {
+        const int idx = tile * SORT_TILE + j * SORT_THREADS + threadIdx.x;
+        if (idx < n) atomicAdd(&h[wave][(k[j] >> shift) & 255u], 1u);
     }
     __syncthreads();
-    hist[(static_cast<size_t>(t) * 256 + threadIdx.x) * tiles + tile] = h[threadIdx.x];
+    uint32_t c = 0;
+#pragma unroll
+    for (int w = 0; w < SORT_THREADS / 64; ++w) c += h[w][threadIdx.x];
+    hist[(static_cast<size_t>(t) * 256 + threadIdx.x) * tiles + tile] = c;
+    if (c) atomicAdd(&dtot[t * 256 + threadIdx.x], c);  // digit totals of the table (zeroed by the host)
 }
 
-// In-place exclusive scan of one table's [256][tiles] histogram (digit major).
-__global__ __launch_bounds__(1024) void radix_scan_kernel(uint32_t* __restrict__ hist, int tiles) {
+// In-place exclusive scan of one table's [256][tiles] histogram (digit major).  The digit
+// totals give every digit row its base; each wavefront then scans whole rows with wave
+// scans only.  Grid (T, SCAN_PARTS): a workgroup handles 256 / SCAN_PARTS digit rows.
+constexpr int SCAN_PARTS = 8;
+__global__ __launch_bounds__(256) void radix_scan_kernel(uint32_t* __restrict__ hist,
+                                                        const uint32_t* __restrict__ dtot, int tiles) {
     __shared__ uint32_t scratch[17];
-    uint32_t* base = hist + static_cast<size_t>(blockIdx.x) * 256 * tiles;
-    const int len = 256 * tiles;
-    uint32_t carry = 0;
-    for (int start = 0; start < len; start += 1024) {
-        const int i = start + threadIdx.x;
-        const uint32_t v = (i < len) ? base[i] : 0;
-        uint32_t total;
-        const uint32_t ex = block_exclusive_sum(v, scratch, &total);
-        if (i < len) base[i] = carry + ex;
-        carry += total;
+    __shared__ uint32_t dbase[256];
+    const int t = blockIdx.x, part = blockIdx.y;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    uint32_t total;
+    dbase[threadIdx.x] = block_exclusive_sum(dtot[t * 256 + threadIdx.x], scratch, &total);
+    __syncthreads();
+    constexpr int ROWS_PER_WAVE = 256 / SCAN_PARTS / 4;
+    for (int k = 0; k < ROWS_PER_WAVE; ++k) {
+        const int d = part * (256 / SCAN_PARTS) + wave * ROWS_PER_WAVE + k;
+        uint32_t* row = hist + (static_cast<size_t>(t) * 256 + d) * tiles;
+        uint32_t carry = dbase[d];
+        for (int c0 = 0; c0 < tiles; c0 += 64) {
+            const int i = c0 + lane;
+            const uint32_t v = (i < tiles) ? row[i] : 0u;
+            const uint32_t incl = wave_inclusive_sum(v);
+            if (i < tiles) row[i] = carry + incl - v;
+            carry += __shfl(incl, 63, 64);
+        }
     }
 }
 
@@ -83,15 +143,23 @@ __global__ __launch_bounds__(SORT_THREADS) void radix_scatter_kernel(
     const uint32_t* __restrict__ keys_in, const int32_t* __restrict__ rows_in,
     uint32_t* __restrict__ keys_out, int32_t* __restrict__ rows_out,
     const uint32_t* __restrict__ hist_scanned, int n, int W, int word, int shift, int tiles) {
-    __shared__ uint32_t whist[SORT_THREADS / 64][256];
+    constexpr int NW = SORT_THREADS / 64;
+    __shared__ uint32_t whist[NW][256];   // per-wave digit counts, then per-wave offsets inside a digit run
+    __shared__ uint32_t dstart[256];      // start of each digit's run inside the sorted tile
+    __shared__ uint32_t gbase[256];       // global position of the run minus dstart (wraps, used additively)
+    __shared__ uint32_t scratch[17];
+    __shared__ uint32_t st_key[SORT_TILE];                 // ONE_WORD: key, else: source slot in the tile
+    __shared__ int32_t st_row[ONE_WORD ? SORT_TILE : 1];
     const int tile = blockIdx.x, t = blockIdx.y;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    for (int i = tid; i < (SORT_THREADS / 64) * 256; i += SORT_THREADS) (&whist[0][0])[i] = 0;
+    for (int i = tid; i < NW * 256; i += SORT_THREADS) (&whist[0][0])[i] = 0;
     __syncthreads();
 
     const size_t tbase = static_cast<size_t>(t) * n;
-    const int base_idx = tile * SORT_TILE + wave * (SORT_ITEMS * 64);
+    const int tile0 = tile * SORT_TILE;
+    const int base_idx = tile0 + wave * (SORT_ITEMS * 64);
     uint32_t kw[SORT_ITEMS], rank[SORT_ITEMS];
+    int32_t rw[ONE_WORD ? SORT_ITEMS : 1];
     const unsigned long long lt_mask = (1ull << lane) - 1ull;
 #pragma unroll
     for (int j = 0; j < SORT_ITEMS; ++j) {
@@ -99,6 +167,7 @@ __global__ __launch_bounds__(SORT_THREADS) void radix_scatter_kernel(
         const bool valid = idx < n;
         const uint32_t k = valid ? keys_in[(tbase + idx) * W + word] : 0u;
         kw[j] = k;
+        if (ONE_WORD) rw[j] = (valid && rows_in) ? rows_in[tbase + idx] : idx;
         const uint32_t d = (k >> shift) & 255u;
         // lanes holding the same digit
         unsigned long long peers = __builtin_amdgcn_ballot_w64(valid);
@@ -121,28 +190,50 @@ __global__ __launch_bounds__(SORT_THREADS) void radix_scatter_kernel(
         rank[j] = old + static_cast<uint32_t>(__popcll(peers & lt_mask));
     }
     __syncthreads();
-    {   // digit `tid`: global base of this tile, then exclusive over the waves
-        uint32_t b = hist_scanned[(static_cast<size_t>(t) * 256 + tid) * tiles + tile];
+    {   // digit `tid`: exclusive over the waves, then over the digits of the tile
+        uint32_t tot = 0;
 #pragma unroll
-        for (int w = 0; w < SORT_THREADS / 64; ++w) {
+        for (int w = 0; w < NW; ++w) {
             const uint32_t c = whist[w][tid];
-            whist[w][tid] = b;
-            b += c;
+            whist[w][tid] = tot;
+            tot += c;
         }
+        uint32_t tile_total;
+        const uint32_t ds = block_exclusive_sum(tot, scratch, &tile_total);
+        dstart[tid] = ds;
+        gbase[tid] = hist_scanned[(static_cast<size_t>(t) * 256 + tid) * tiles + tile] - ds;
     }
     __syncthreads();
+    // Stage the tile in digit order in LDS so that the global stores below walk
+    // consecutive addresses inside every digit run (full-line writes instead of 4-byte ones).
 #pragma unroll
     for (int j = 0; j < SORT_ITEMS; ++j) {
         const int idx = base_idx + j * 64 + lane;
         if (idx < n) {
             const uint32_t d = (kw[j] >> shift) & 255u;
-            const size_t dst = tbase + whist[wave][d] + rank[j];
+            const uint32_t lp = dstart[d] + whist[wave][d] + rank[j];
             if (ONE_WORD) {
-                keys_out[dst] = kw[j];
+                st_key[lp] = kw[j];
+                st_row[lp] = rw[j];
             } else {
-                for (int w = 0; w < W; ++w) keys_out[dst * W + w] = keys_in[(tbase + idx) * W + w];
+                st_key[lp] = static_cast<uint32_t>(idx - tile0);
             }
-            rows_out[dst] = rows_in ? rows_in[tbase + idx] : idx;
+        }
+    }
+    __syncthreads();
+    const int cnt = min(SORT_TILE, n - tile0);
+    for (int slot = tid; slot < cnt; slot += SORT_THREADS) {
+        if (ONE_WORD) {
+            const uint32_t k = st_key[slot];
+            const size_t dst = tbase + static_cast<uint32_t>(gbase[(k >> shift) & 255u] + slot);
+            keys_out[dst] = k;
+            rows_out[dst] = st_row[slot];
+        } else {
+            const int src = tile0 + static_cast<int>(st_key[slot]);
+            const uint32_t* ks = keys_in + (tbase + src) * W;
+            const size_t dst = tbase + static_cast<uint32_t>(gbase[(ks[word] >> shift) & 255u] + slot);
+            for (int w = 0; w < W; ++w) keys_out[dst * W + w] = ks[w];
+            rows_out[dst] = rows_in ? rows_in[tbase + src] : src;
         }
     }
 }
@@ -167,8 +258,15 @@ culsh_status sort_tables(culsh_ctx* ctx, uint32_t* keys_in, uint32_t* keys_tmp, 
     CULSH_TRY(arena_alloc_t(ctx, static_cast<size_t>(W), &vary_dev));
     CULSH_HIP(hipMemsetAsync(vary_dev, 0, W * sizeof(uint32_t), ctx->stream));
     {
-        const unsigned bx = std::max(1u, std::min(64u, div_up(n, 256 * 8)));
-        CULSH_LAUNCH(ctx, varying_bits_kernel, dim3(bx, T), dim3(256), 0, ctx->stream, keys_in, n, W, vary_dev);
+        const bool vec = (W == 1 || W == 2 || W == 4) && (static_cast<size_t>(n) * W) % 4 == 0 &&
+                         reinterpret_cast<uintptr_t>(keys_in) % 16 == 0;
+        if (vec) {
+            const unsigned bx = std::max(1u, std::min(64u, div_up(static_cast<size_t>(n) * W / 4, 256 * 4)));
+            CULSH_LAUNCH(ctx, varying_bits_vec_kernel, dim3(bx, T), dim3(256), 0, ctx->stream, keys_in, n, W, vary_dev);
+        } else {
+            const unsigned bx = std::max(1u, std::min(64u, div_up(n, 256 * 8)));
+            CULSH_LAUNCH(ctx, varying_bits_kernel, dim3(bx, T), dim3(256), 0, ctx->stream, keys_in, n, W, vary_dev);
+        }
         CULSH_LAUNCH_CHECK();
     }
     uint32_t vary[64];
@@ -193,15 +291,19 @@ culsh_status sort_tables(culsh_ctx* ctx, uint32_t* keys_in, uint32_t* keys_tmp, 
     uint32_t* kin = keys_in;
     uint32_t* kout = keys_tmp;
     const int np = static_cast<int>(passes.size());
+    uint32_t* dtot = nullptr;  // [pass][T][256] digit totals, accumulated by the histogram kernel
+    CULSH_TRY(arena_alloc_t(ctx, static_cast<size_t>(np) * T * 256, &dtot));
+    CULSH_HIP(hipMemsetAsync(dtot, 0, static_cast<size_t>(np) * T * 256 * sizeof(uint32_t), ctx->stream));
     const int32_t* rin = nullptr;
     for (int p = 0; p < np; ++p) {
         // the last pass must land in rows_out
         int32_t* rout = ((np - 1 - p) % 2 == 0) ? rows_out : rows_tmp;
         const dim3 grid(tiles, T);
         CULSH_LAUNCH(ctx, radix_hist_kernel, grid, dim3(SORT_THREADS), 0, ctx->stream, kin, n, W,
-                           passes[p].word, passes[p].shift, tiles, hist);
+                           passes[p].word, passes[p].shift, tiles, hist, dtot + static_cast<size_t>(p) * T * 256);
         CULSH_LAUNCH_CHECK();
-        CULSH_LAUNCH(ctx, radix_scan_kernel, dim3(T), dim3(1024), 0, ctx->stream, hist, tiles);
+        CULSH_LAUNCH(ctx, radix_scan_kernel, dim3(T, SCAN_PARTS), dim3(256), 0, ctx->stream, hist,
+                     dtot + static_cast<size_t>(p) * T * 256, tiles);
         CULSH_LAUNCH_CHECK();
         if (W == 1)
             CULSH_LAUNCH(ctx, radix_scatter_kernel<true>, grid, dim3(SORT_THREADS), 0, ctx->stream, kin, rin,
