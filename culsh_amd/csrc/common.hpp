@@ -184,17 +184,20 @@ culsh_status launch_minhash(culsh_ctx* ctx, const int32_t* indices, const int32_
 // signature bytes [T][n][S] -> key words [T][n][W]
 culsh_status launch_sig_to_keys(culsh_ctx* ctx, const uint8_t* sig, size_t n_items, int S,
                                 KeyEnc enc, int W, uint32_t* keys);
-// key words [count][W] -> signature bytes [count][S]
-culsh_status launch_keys_to_sig(culsh_ctx* ctx, const uint32_t* keys, size_t count, int S,
-                                KeyEnc enc, int W, uint8_t* sig);
+// key words [count][W] -> signature bytes [count][S]; count_dev (may be null) caps count by a
+// value that only the device knows yet
+culsh_status launch_keys_to_sig(culsh_ctx* ctx, const uint32_t* keys, size_t count, const uint64_t* count_dev,
+                                int S, KeyEnc enc, int W, uint8_t* sig);
 
 // ---------------------------------------------------------------- sort (sort.hip)
 // Stable sort of each table's n items by key words (word 0 most significant), starting
 // from the identity permutation.  keys_in [T][n][W] is clobbered.  On return
 // *sorted_keys points at whichever of keys_in / keys_tmp holds the sorted keys and
-// rows_out [T][n] holds the row ids in sorted order.
+// rows_out [T][n] holds the row ids in sorted order.  known_vary (host, [W], may be null):
+// bits that may differ between keys; when null they are measured (one host sync).
 culsh_status sort_tables(culsh_ctx* ctx, uint32_t* keys_in, uint32_t* keys_tmp, int32_t* rows_tmp,
-                         int32_t* rows_out, int n, int T, int W, uint32_t** sorted_keys);
+                         int32_t* rows_out, int n, int T, int W, const uint32_t* known_vary,
+                         uint32_t** sorted_keys);
 size_t sort_scratch_bytes(int n, int T, int W);
 
 // ---------------------------------------------------------------- index build (index.hip)

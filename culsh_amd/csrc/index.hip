@@ -5,6 +5,8 @@
 // two passes over the sorted items: count bucket heads per tile, then (after a scan of
 // the tile counts) write bucket offsets, bucket keys, table offsets and, optionally, the
 // (row, table) -> bucket map.
+#include <algorithm>
+
 #include "block_utils.hpp"
 #include "common.hpp"
 
@@ -66,7 +68,8 @@ __global__ __launch_bounds__(IB_THREADS) void count_heads_kernel(const uint32_t*
 
 __global__ __launch_bounds__(IB_THREADS) void build_index_kernel(
     const uint32_t* __restrict__ keys, const int32_t* __restrict__ rows, size_t N, int n, int T, int W,
-    const uint64_t* __restrict__ tile_base, int n_buckets, int32_t* __restrict__ bucket_candidate_offsets,
+    const uint64_t* __restrict__ tile_base, const uint64_t* __restrict__ n_buckets_dev,
+    int32_t* __restrict__ bucket_candidate_offsets,
     uint32_t* __restrict__ bucket_keys, int32_t* __restrict__ table_bucket_offsets,
     int32_t* __restrict__ item_to_bucket) {
     __shared__ uint64_t scratch[17];
@@ -92,6 +95,7 @@ __global__ __launch_bounds__(IB_THREADS) void build_index_kernel(
         }
     }
     if (blockIdx.x == 0 && threadIdx.x == 0) {  // terminators, fit.cuh:351-357
+        const int32_t n_buckets = static_cast<int32_t>(*n_buckets_dev);
         table_bucket_offsets[T] = n_buckets;
         bucket_candidate_offsets[n_buckets] = static_cast<int32_t>(N);
     }
@@ -121,8 +125,10 @@ __global__ __launch_bounds__(256) void sig_to_keys_kernel(const uint8_t* __restr
 }
 
 __global__ __launch_bounds__(256) void keys_to_sig_kernel(const uint32_t* __restrict__ keys, size_t count,
-                                                         int S, int enc, int W, uint8_t* __restrict__ sig) {
+                                                         const uint64_t* __restrict__ count_dev, int S, int enc,
+                                                         int W, uint8_t* __restrict__ sig) {
     const size_t idx = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (count_dev) count = min(count, static_cast<size_t>(*count_dev));  // exact count known on the device only
     if (idx >= count * S) return;
     const size_t item = idx / S;
     const int byte = static_cast<int>(idx - item * S);
@@ -146,13 +152,13 @@ culsh_status launch_sig_to_keys(culsh_ctx* ctx, const uint8_t* sig, size_t n_ite
     return CULSH_OK;
 }
 
-culsh_status launch_keys_to_sig(culsh_ctx* ctx, const uint32_t* keys, size_t count, int S, KeyEnc enc, int W,
-                                uint8_t* sig) {
+culsh_status launch_keys_to_sig(culsh_ctx* ctx, const uint32_t* keys, size_t count, const uint64_t* count_dev,
+                                int S, KeyEnc enc, int W, uint8_t* sig) {
     if (count == 0) return CULSH_OK;
     const size_t total = count * S;
     CULSH_REQUIRE(total / 256 < (1ull << 31), CULSH_ERR_LIMIT, "too many buckets");
-    CULSH_LAUNCH(ctx, keys_to_sig_kernel, dim3(div_up(total, 256)), dim3(256), 0, ctx->stream, keys, count, S,
-                       static_cast<int>(enc), W, sig);
+    CULSH_LAUNCH(ctx, keys_to_sig_kernel, dim3(div_up(total, 256)), dim3(256), 0, ctx->stream, keys, count,
+                 count_dev, S, static_cast<int>(enc), W, sig);
     CULSH_LAUNCH_CHECK();
     return CULSH_OK;
 }
@@ -170,27 +176,37 @@ culsh_status build_index_from_sorted(culsh_ctx* ctx, const uint32_t* sorted_keys
                        sorted_keys, N, n, W, tile_counts);
     CULSH_LAUNCH_CHECK();
     CULSH_TRY(exclusive_scan_u64(ctx, tile_counts, tile_base, tiles));
-    uint64_t n_buckets64 = 0;
-    CULSH_TRY(read_back_u64(ctx, tile_base + tiles, 1, &n_buckets64));  // the one host sync (fit.cuh:332-337)
-    const int B = static_cast<int>(n_buckets64);
+    const uint64_t* total_dev = tile_base + tiles;
 
+    // Sign-bit keys admit at most 2^S buckets per table.  When that bound is small the bucket
+    // arrays are sized by it and the exact count is fetched at the end of the call, so the
+    // device never waits for the host in the middle of the build.
+    size_t B_bound = N;
+    if (enc == ENC_BITS && S < 31) B_bound = std::min<size_t>(N, static_cast<size_t>(T) << S);
+    const bool deferred = B_bound * (8 + static_cast<size_t>(4) * W + S) <= (static_cast<size_t>(256) << 20);
+    uint64_t n_buckets64 = 0;
+    if (!deferred) {
+        CULSH_TRY(read_back_u64(ctx, total_dev, 1, &n_buckets64));  // host sync (fit.cuh:332-337)
+        B_bound = static_cast<size_t>(n_buckets64);
+    }
     index->all_candidate_indices = rows_sorted_owned;
     index->n_total_candidates = static_cast<int>(N);
-    index->n_total_buckets = B;
     index->n_hash_tables = T;
     index->n_hashes = H;
     index->sig_nbytes = S;
     index->enc = enc;
     index->key_w = W;
-    CULSH_HIP(hipMalloc(&index->bucket_candidate_offsets, (static_cast<size_t>(B) + 1) * sizeof(int32_t)));
+    CULSH_HIP(hipMalloc(&index->bucket_candidate_offsets, (B_bound + 1) * sizeof(int32_t)));
     CULSH_HIP(hipMalloc(&index->table_bucket_offsets, (static_cast<size_t>(T) + 1) * sizeof(int32_t)));
-    CULSH_HIP(hipMalloc(&index->bucket_keys, std::max<size_t>(1, static_cast<size_t>(B) * W) * sizeof(uint32_t)));
-    CULSH_HIP(hipMalloc(&index->all_bucket_signatures, std::max<size_t>(1, static_cast<size_t>(B) * S)));
+    CULSH_HIP(hipMalloc(&index->bucket_keys, std::max<size_t>(1, B_bound * W) * sizeof(uint32_t)));
+    CULSH_HIP(hipMalloc(&index->all_bucket_signatures, std::max<size_t>(1, B_bound * S)));
     CULSH_LAUNCH(ctx, build_index_kernel, dim3(static_cast<unsigned>(tiles)), dim3(IB_THREADS), 0, ctx->stream,
-                       sorted_keys, rows_sorted_owned, N, n, T, W, tile_base, B, index->bucket_candidate_offsets,
+                       sorted_keys, rows_sorted_owned, N, n, T, W, tile_base, total_dev, index->bucket_candidate_offsets,
                        index->bucket_keys, index->table_bucket_offsets, item_to_bucket_opt);
     CULSH_LAUNCH_CHECK();
-    CULSH_TRY(launch_keys_to_sig(ctx, index->bucket_keys, B, S, enc, W, index->all_bucket_signatures));
+    CULSH_TRY(launch_keys_to_sig(ctx, index->bucket_keys, B_bound, total_dev, S, enc, W, index->all_bucket_signatures));
+    if (deferred) CULSH_TRY(read_back_u64(ctx, total_dev, 1, &n_buckets64));
+    index->n_total_buckets = static_cast<int>(n_buckets64);
     return CULSH_OK;
 }
 
@@ -207,7 +223,18 @@ culsh_status fit_index_from_keys(culsh_ctx* ctx, uint32_t* keys, int n, int T, i
     CULSH_HIP(hipMalloc(&rows_out, N * sizeof(int32_t)));
     index->all_candidate_indices = rows_out;  // owned by the index from here on (freed with it)
     uint32_t* sorted = nullptr;
-    CULSH_TRY(sort_tables(ctx, keys, keys_tmp, rows_tmp, rows_out, n, T, W, &sorted));
+    uint32_t bits_vary[64];
+    const uint32_t* known_vary = nullptr;
+    if (enc == ENC_BITS && W <= 64) {
+        // sign-bit keys: exactly the top S bits of the key string can differ, so the radix
+        // passes are known without looking at the data (and without a host round trip)
+        for (int w = 0; w < W; ++w) {
+            const int nbits = std::min(32, S - 32 * w);
+            bits_vary[w] = nbits >= 32 ? 0xFFFFFFFFu : (0xFFFFFFFFu << (32 - nbits));
+        }
+        known_vary = bits_vary;
+    }
+    CULSH_TRY(sort_tables(ctx, keys, keys_tmp, rows_tmp, rows_out, n, T, W, known_vary, &sorted));
     return build_index_from_sorted(ctx, sorted, rows_out, n, T, H, S, enc, W, item_to_bucket_opt, index);
 }
 

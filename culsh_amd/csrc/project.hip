@@ -14,8 +14,6 @@ namespace {
 
 constexpr int BM = 128;        // rows of X per workgroup
 constexpr int BN = 128;        // (virtual) hash columns per workgroup
-constexpr int BK = 32;         // features per LDS stage
-constexpr int PITCH = BK + 4;  // LDS row pitch in floats (bank spread for 16-byte reads)
 constexpr int NTHREADS = 256;  // 4 wavefronts as 2 x 2, each 64 x 64 of the tile
 
 struct ProjArgs {
@@ -63,8 +61,15 @@ __device__ __forceinline__ float4 load4(const float* __restrict__ base, size_t r
     return v;
 }
 
-template <int EPI>
+// VEC: n_features is a multiple of 4 and X, P are 16-byte aligned, so a stage is fetched
+// with unconditional 16-byte loads.  Rows past the end of X and padding columns read a
+// valid row instead of zeros: their accumulators are never stored.
+template <int EPI, bool VEC, int BK>
 __global__ __launch_bounds__(NTHREADS) void project_f32_kernel(ProjArgs a) {
+    constexpr int PITCH = BK + 4;  // LDS row pitch in floats (bank spread for 16-byte reads)
+    constexpr int F4 = BK / 4;     // float4 per tile row and stage
+    constexpr int NLD = BM * F4 / NTHREADS;  // float4 fetched per thread, tile and stage
+    constexpr int RSTEP = NTHREADS / F4;     // tile rows covered by one fetch of all threads
     __shared__ __attribute__((aligned(16))) float As[BM * PITCH];
     __shared__ __attribute__((aligned(16))) float Bs[BN * PITCH];
     __shared__ uint32_t tw[(EPI == EPI_SIGN_KEYS) ? BM * (BN / 32) : 1];
@@ -88,19 +93,39 @@ __global__ __launch_bounds__(NTHREADS) void project_f32_kernel(ProjArgs a) {
     const int TH = T * H;
 
     // global -> LDS staging: thread loads float4 number (tid + 256*i), i < 4, of each tile
-    const int lrow = tid >> 3, c4 = (tid & 7) * 4;
-    size_t xoff[4], poff[4];
-    bool xok[4], pok[4];
+    const int lrow = tid / F4, c4 = (tid % F4) * 4;
+    size_t xoff[NLD], poff[NLD];
+    bool xok[NLD], pok[NLD];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const int row = rt * BM + lrow + 32 * i;
+    for (int i = 0; i < NLD; ++i) {
+        const int row = rt * BM + lrow + RSTEP * i;
         xok[i] = row < n;
-        xoff[i] = static_cast<size_t>(row) * d;
-        const int vc = ct * BN + lrow + 32 * i;
+        xoff[i] = static_cast<size_t>(VEC ? min(row, n - 1) : row) * d;
+        const int vc = ct * BN + lrow + RSTEP * i;
         const int prow = (EPI == EPI_SIGN_KEYS) ? sign_vcol_to_prow(vc, T, H) : (vc < TH ? vc : -1);
         pok[i] = prow >= 0;
         poff[i] = static_cast<size_t>(prow < 0 ? 0 : prow) * d;
     }
+    // stage fetch: 4 + 4 float4 per thread
+    auto fetch = [&](int k, float4 (&ra)[NLD], float4 (&rb)[NLD]) {
+        if (VEC) {
+            const int kk = min(k, d - 4);
+            const bool inside = k < d;  // a float4 is entirely inside or entirely outside [0, d)
+#pragma unroll
+            for (int i = 0; i < NLD; ++i) {
+                const float4 va = *reinterpret_cast<const float4*>(a.X + xoff[i] + kk);
+                const float4 vb = *reinterpret_cast<const float4*>(a.P + poff[i] + kk);
+                ra[i] = inside ? va : make_float4(0.f, 0.f, 0.f, 0.f);
+                rb[i] = inside ? vb : make_float4(0.f, 0.f, 0.f, 0.f);
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < NLD; ++i) {
+                ra[i] = load4(a.X, xoff[i], k, d, xok[i], 0);
+                rb[i] = load4(a.P, poff[i], k, d, pok[i], 0);
+            }
+        }
+    };
 
     f32x16 acc[2][2];
 #pragma unroll
@@ -110,40 +135,30 @@ __global__ __launch_bounds__(NTHREADS) void project_f32_kernel(ProjArgs a) {
 #pragma unroll
             for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
 
-    float4 ra[4], rb[4];
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        ra[i] = load4(a.X, xoff[i], c4, d, xok[i], a.vec_x);
-        rb[i] = load4(a.P, poff[i], c4, d, pok[i], a.vec_p);
-    }
+    float4 ra[NLD], rb[NLD];
+    fetch(c4, ra, rb);
 
     const int nk = (d + BK - 1) / BK;
     for (int kt = 0; kt < nk; ++kt) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            *reinterpret_cast<float4*>(&As[(lrow + 32 * i) * PITCH + c4]) = ra[i];
-            *reinterpret_cast<float4*>(&Bs[(lrow + 32 * i) * PITCH + c4]) = rb[i];
+        for (int i = 0; i < NLD; ++i) {
+            *reinterpret_cast<float4*>(&As[(lrow + RSTEP * i) * PITCH + c4]) = ra[i];
+            *reinterpret_cast<float4*>(&Bs[(lrow + RSTEP * i) * PITCH + c4]) = rb[i];
         }
         __syncthreads();
-        if (kt + 1 < nk) {
-            const int k0 = (kt + 1) * BK + c4;
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                ra[i] = load4(a.X, xoff[i], k0, d, xok[i], a.vec_x);
-                rb[i] = load4(a.P, poff[i], k0, d, pok[i], a.vec_p);
-            }
-        }
+        if (kt + 1 < nk) fetch((kt + 1) * BK + c4, ra, rb);
         // The 32x32x2 MFMA takes, per lane, A[row = lane%32][k = lane/32] and
         // B[k = lane/32][col = lane%32].  Any pairing of k between A and B that covers each
         // feature once is a valid dot product, so lanes 0-31 walk features 0..15 of the
-        // stage and lanes 32-63 features 16..31: each lane reads 16 consecutive floats.
-        float af[2][16], bf[2][16];
+        // stage and lanes 32-63 features BK/2..BK-1: each lane reads BK/2 consecutive floats.
+        constexpr int KH = BK / 2;  // features per lane and stage
+        float af[2][KH], bf[2][KH];
 #pragma unroll
         for (int i = 0; i < 2; ++i) {
-            const float* pa = &As[(wm * 64 + i * 32 + r32) * PITCH + half * 16];
-            const float* pb = &Bs[(wn * 64 + i * 32 + r32) * PITCH + half * 16];
+            const float* pa = &As[(wm * 64 + i * 32 + r32) * PITCH + half * KH];
+            const float* pb = &Bs[(wn * 64 + i * 32 + r32) * PITCH + half * KH];
 #pragma unroll
-            for (int q = 0; q < 4; ++q) {
+            for (int q = 0; q < KH / 4; ++q) {
                 const float4 va = *reinterpret_cast<const float4*>(pa + 4 * q);
                 const float4 vb = *reinterpret_cast<const float4*>(pb + 4 * q);
                 af[i][4 * q + 0] = va.x; af[i][4 * q + 1] = va.y;
@@ -153,7 +168,7 @@ __global__ __launch_bounds__(NTHREADS) void project_f32_kernel(ProjArgs a) {
             }
         }
 #pragma unroll
-        for (int k = 0; k < 16; ++k)
+        for (int k = 0; k < KH; ++k)
 #pragma unroll
             for (int i = 0; i < 2; ++i)
 #pragma unroll
@@ -321,12 +336,19 @@ culsh_status launch_project_f32(culsh_ctx* ctx, const float* X, const float* P, 
     const long long blocks = groups * 8 * a.n_col_tiles;
     CULSH_REQUIRE(blocks < (1ll << 31), CULSH_ERR_LIMIT, "projection grid too large");
     dim3 grid(static_cast<unsigned>(blocks)), block(NTHREADS);
+    const bool vec = a.vec_x && a.vec_p;
+#define PROJ_CASE(E)                                                                              \
+    case E:                                                                                       \
+        if (vec) CULSH_LAUNCH(ctx, (project_f32_kernel<E, true, 32>), grid, block, 0, ctx->stream, a);   \
+        else CULSH_LAUNCH(ctx, (project_f32_kernel<E, false, 32>), grid, block, 0, ctx->stream, a);      \
+        break;
     switch (epi) {
-        case EPI_SIGN_KEYS: CULSH_LAUNCH(ctx, project_f32_kernel<EPI_SIGN_KEYS>, grid, block, 0, ctx->stream, a); break;
-        case EPI_SIGN_BYTES: CULSH_LAUNCH(ctx, project_f32_kernel<EPI_SIGN_BYTES>, grid, block, 0, ctx->stream, a); break;
-        case EPI_FLOOR_KEYS: CULSH_LAUNCH(ctx, project_f32_kernel<EPI_FLOOR_KEYS>, grid, block, 0, ctx->stream, a); break;
-        case EPI_FLOOR_I32: CULSH_LAUNCH(ctx, project_f32_kernel<EPI_FLOOR_I32>, grid, block, 0, ctx->stream, a); break;
+        PROJ_CASE(EPI_SIGN_KEYS)
+        PROJ_CASE(EPI_SIGN_BYTES)
+        PROJ_CASE(EPI_FLOOR_KEYS)
+        PROJ_CASE(EPI_FLOOR_I32)
     }
+#undef PROJ_CASE
     CULSH_LAUNCH_CHECK();
     return CULSH_OK;
 }

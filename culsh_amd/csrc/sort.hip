@@ -247,17 +247,21 @@ size_t sort_scratch_bytes(int n, int T, int W) {
 }
 
 culsh_status sort_tables(culsh_ctx* ctx, uint32_t* keys_in, uint32_t* keys_tmp, int32_t* rows_tmp,
-                         int32_t* rows_out, int n, int T, int W, uint32_t** sorted_keys) {
+                         int32_t* rows_out, int n, int T, int W, const uint32_t* known_vary,
+                         uint32_t** sorted_keys) {
     CULSH_REQUIRE(n > 0 && T > 0 && W > 0 && W <= 64, CULSH_ERR_INVALID, "sort: bad sizes (W must be <= 64 words)");
     CULSH_REQUIRE(T <= 65535, CULSH_ERR_LIMIT, "n_hash_tables > 65535 is not supported");
     const int tiles = (n + SORT_TILE - 1) / SORT_TILE;
     const size_t N = static_cast<size_t>(n) * T;
 
-    // which byte positions differ anywhere
-    uint32_t* vary_dev = nullptr;
-    CULSH_TRY(arena_alloc_t(ctx, static_cast<size_t>(W), &vary_dev));
-    CULSH_HIP(hipMemsetAsync(vary_dev, 0, W * sizeof(uint32_t), ctx->stream));
-    {
+    // which byte positions differ anywhere (given by the caller, or measured on the keys)
+    uint32_t vary[64];
+    if (known_vary) {
+        for (int w = 0; w < W; ++w) vary[w] = known_vary[w];
+    } else {
+        uint32_t* vary_dev = nullptr;
+        CULSH_TRY(arena_alloc_t(ctx, static_cast<size_t>(W), &vary_dev));
+        CULSH_HIP(hipMemsetAsync(vary_dev, 0, W * sizeof(uint32_t), ctx->stream));
         const bool vec = (W == 1 || W == 2 || W == 4) && (static_cast<size_t>(n) * W) % 4 == 0 &&
                          reinterpret_cast<uintptr_t>(keys_in) % 16 == 0;
         if (vec) {
@@ -268,9 +272,8 @@ culsh_status sort_tables(culsh_ctx* ctx, uint32_t* keys_in, uint32_t* keys_tmp, 
             CULSH_LAUNCH(ctx, varying_bits_kernel, dim3(bx, T), dim3(256), 0, ctx->stream, keys_in, n, W, vary_dev);
         }
         CULSH_LAUNCH_CHECK();
+        CULSH_TRY(read_back_u32(ctx, vary_dev, W, vary));
     }
-    uint32_t vary[64];
-    CULSH_TRY(read_back_u32(ctx, vary_dev, W, vary));
 
     // least significant digit first: last word, low byte
     struct Pass { int word, shift; };
