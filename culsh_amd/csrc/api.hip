@@ -200,6 +200,7 @@ void free_index_arrays(culsh_index* ix) {
     (void)hipFree(ix->b);
     (void)hipFree(ix->A);
     (void)hipFree(ix->B);
+    free_ps_codec(ix);
     ix->all_candidate_indices = nullptr;
     ix->all_bucket_signatures = nullptr;
     ix->bucket_candidate_offsets = nullptr;
@@ -250,26 +251,52 @@ static culsh_status check_fit_args(culsh_ctx* ctx, const void* X, int n, int d, 
 // ---------------------------------------------------------------- hashing to key words
 enum Family { FAM_RPLSH, FAM_PSLSH };
 
-// Dense rows -> key words [T][rows][W] in the arena.
+// Dense rows -> key words [T][rows][W] in the arena.  For p-stable hashing at fit time
+// (`fit_ix` given) the key encoding is chosen here and recorded in the index; at query time
+// (`ix` given) the index's encoding is used.
 template <typename T>
 static culsh_status hash_dense_to_keys(culsh_ctx* ctx, Family fam, const T* X, int rows, int d, int nT, int H,
-                                       const void* P, const void* b, uint32_t** keys_out, int* W_out) {
+                                       const void* P, const void* b, culsh_index* fit_ix, const culsh_index* ix,
+                                       uint32_t** keys_out, int* W_out) {
     const size_t N = static_cast<size_t>(rows) * nT;
-    const KeyEnc enc = (fam == FAM_RPLSH) ? ENC_BITS : ENC_BE;
-    const int S = (fam == FAM_RPLSH) ? H : 4 * H;
-    const int W = key_words(enc, S);
     uint32_t* keys = nullptr;
-    CULSH_TRY(arena_alloc_t(ctx, N * W, &keys));
-    if constexpr (std::is_same_v<T, float>) {
-        CULSH_TRY(launch_project_f32(ctx, X, static_cast<const float*>(P), static_cast<const float*>(b), rows, d, nT,
-                                     H, fam == FAM_RPLSH ? EPI_SIGN_KEYS : EPI_FLOOR_KEYS, keys));
-    } else {
-        uint8_t* sig = nullptr;
-        CULSH_TRY(arena_alloc_t(ctx, N * S, &sig));
-        CULSH_TRY(launch_project_f64(ctx, X, static_cast<const double*>(P), static_cast<const double*>(b), rows, d,
-                                     nT, H, fam == FAM_RPLSH ? EPI_SIGN_BYTES : EPI_FLOOR_I32, sig));
-        CULSH_TRY(launch_sig_to_keys(ctx, sig, N, S, enc, W, keys));
+    if (fam == FAM_RPLSH) {
+        const int W = key_words(ENC_BITS, H);
+        CULSH_TRY(arena_alloc_t(ctx, N * W, &keys));
+        if constexpr (std::is_same_v<T, float>) {
+            CULSH_TRY(launch_project_f32(ctx, X, static_cast<const float*>(P), nullptr, rows, d, nT, H, EPI_SIGN_KEYS, keys));
+        } else {
+            uint8_t* sig = nullptr;
+            CULSH_TRY(arena_alloc_t(ctx, N * H, &sig));
+            CULSH_TRY(launch_project_f64(ctx, X, static_cast<const double*>(P), nullptr, rows, d, nT, H, EPI_SIGN_BYTES, sig));
+            CULSH_TRY(launch_sig_to_keys(ctx, sig, N, H, ENC_BITS, W, keys));
+        }
+        *keys_out = keys;
+        *W_out = W;
+        return CULSH_OK;
     }
+    // p-stable: int32 hashes in the reference layout first (pslsh/hash.cuh:25-47)
+    int32_t* sig = nullptr;
+    CULSH_TRY(arena_alloc_t(ctx, N * H, &sig));
+    if constexpr (std::is_same_v<T, float>) {
+        CULSH_TRY(launch_project_f32(ctx, X, static_cast<const float*>(P), static_cast<const float*>(b), rows, d, nT, H,
+                                     EPI_FLOOR_I32, sig));
+    } else {
+        CULSH_TRY(launch_project_f64(ctx, X, static_cast<const double*>(P), static_cast<const double*>(b), rows, d, nT,
+                                     H, EPI_FLOOR_I32, sig));
+    }
+    if (fit_ix) {
+        bool compressed = false;
+        CULSH_TRY(ps_build_codec(ctx, sig, rows, nT, H, fit_ix, &compressed));
+        if (!compressed) { fit_ix->enc = ENC_BE; fit_ix->key_w = H; }
+        ix = fit_ix;
+    }
+    const int W = ix->key_w;
+    CULSH_TRY(arena_alloc_t(ctx, N * W, &keys));
+    if (ix->enc == ENC_PSC)
+        CULSH_TRY(launch_ps_compress(ctx, sig, rows, nT, H, ix, keys));
+    else
+        CULSH_TRY(launch_sig_to_keys(ctx, reinterpret_cast<const uint8_t*>(sig), N, 4 * H, ENC_BE, W, keys));
     *keys_out = keys;
     *W_out = W;
     return CULSH_OK;
@@ -354,7 +381,7 @@ static culsh_status dense_query(culsh_ctx* ctx, Family fam, const T* Q, int nq, 
         uint32_t* keys = nullptr;
         int W = 0;
         CULSH_TRY(hash_dense_to_keys<T>(ctx, fam, Q + static_cast<size_t>(start) * d, bn, d, nT, H, ix->P, ix->b,
-                                        &keys, &W));
+                                        nullptr, ix, &keys, &W));
         CandPtr part(new (std::nothrow) culsh_candidates());
         CULSH_REQUIRE(part, CULSH_ERR_NOMEM, "host allocation failed");
         part->device = ctx->device;
@@ -431,8 +458,8 @@ static culsh_status dense_fit(culsh_ctx* ctx, Family fam, const T* X, int n, int
     }
     uint32_t* keys = nullptr;
     int W = 0;
-    CULSH_TRY(hash_dense_to_keys<T>(ctx, fam, X, n, d, nT, H, ix->P, ix->b, &keys, &W));
-    const KeyEnc enc = (fam == FAM_RPLSH) ? ENC_BITS : ENC_BE;
+    CULSH_TRY(hash_dense_to_keys<T>(ctx, fam, X, n, d, nT, H, ix->P, ix->b, ix.get(), nullptr, &keys, &W));
+    const KeyEnc enc = (fam == FAM_RPLSH) ? ENC_BITS : ix->enc;
     const int S = (fam == FAM_RPLSH) ? H : 4 * H;  // rplsh.cu:37, pslsh.cu:39
     CandPtr cands;
     if (cands_out) {
@@ -799,6 +826,10 @@ static culsh_status sig_query_keys(culsh_ctx* ctx, const void* Q_sig, int nq, in
     CULSH_REQUIRE(S == ix->sig_nbytes, CULSH_ERR_INVALID, "sig_nbytes (%d) != index sig_nbytes (%d)", S,
                   ix->sig_nbytes);  // core/query.cuh:494
     CULSH_TRY(arena_alloc_t(ctx, static_cast<size_t>(nq) * ix->n_hash_tables * ix->key_w, keys));
+    if (ix->enc == ENC_PSC) {
+        CULSH_REQUIRE(reinterpret_cast<uintptr_t>(Q_sig) % 4 == 0, CULSH_ERR_INVALID, "signatures must be 4-byte aligned");
+        return launch_ps_compress(ctx, static_cast<const int32_t*>(Q_sig), nq, ix->n_hash_tables, ix->n_hashes, ix, *keys);
+    }
     return launch_sig_to_keys(ctx, static_cast<const uint8_t*>(Q_sig), static_cast<size_t>(nq) * ix->n_hash_tables,
                               S, ix->enc, ix->key_w, *keys);
 }

@@ -54,11 +54,23 @@ struct Status {
 // unsigned word-lexicographic order is that byte order:
 //   ENC_BE   word w = big-endian load of signature bytes [4w, 4w+4), zero padded
 //   ENC_BITS (signatures made of 0/1 bytes) hash h -> bit (31 - h%32) of word h/32
-enum KeyEnc : int { ENC_BE = 0, ENC_BITS = 1 };
+//   ENC_PSC  (p-stable int32 hashes) per-hash ranks in byte order, `bits` each, MSB first;
+//            the width comes from the index's codec (pscodec.hip)
+enum KeyEnc : int { ENC_BE = 0, ENC_BITS = 1, ENC_PSC = 2 };
 
 inline int key_words(KeyEnc enc, int sig_nbytes) {
     return enc == ENC_BITS ? (sig_nbytes + 31) / 32 : (sig_nbytes + 3) / 4;
 }
+
+// Rank tables of the p-stable key compression (device arrays, owned by the index).
+struct PsCodec {
+    int bits = 0;             // bits per hash in a compressed key
+    int rmax = 0;             // row pitch of fwd / inv
+    int32_t* vmin = nullptr;  // [T*H] smallest hash value seen at fit time
+    int32_t* range = nullptr; // [T*H] number of values in [vmin, vmax]
+    uint32_t* fwd = nullptr;  // [T*H][rmax] value - vmin -> rank in byte order (0-based)
+    int32_t* inv = nullptr;   // [T*H][rmax] rank -> value
+};
 
 }  // namespace culsh_amd
 
@@ -97,6 +109,7 @@ struct culsh_index {
     uint32_t* bucket_keys = nullptr;
     culsh_amd::KeyEnc enc = culsh_amd::ENC_BE;
     int key_w = 0;
+    culsh_amd::PsCodec psc;  // enc == ENC_PSC only
     // family parameters (device): rplsh/index.cuh, pslsh/index.cuh, minhash/index.cuh
     culsh_kind kind = CULSH_KIND_CORE;
     bool is_double = false;
@@ -166,7 +179,6 @@ culsh_status read_back_u32(culsh_ctx* ctx, const uint32_t* dev, int count, uint3
 enum ProjEpilogue : int {
     EPI_SIGN_KEYS = 0,   // RPLSH, fused: packed sign bits -> key words [T][n][W] (ENC_BITS)
     EPI_SIGN_BYTES = 1,  // RPLSH, reference layout: uint8 [T][n][H]
-    EPI_FLOOR_KEYS = 2,  // p-stable, fused: byte-swapped floor(x+b) -> key words [T][n][H] (ENC_BE)
     EPI_FLOOR_I32 = 3    // p-stable, reference layout: int32 [T][n][H]
 };
 culsh_status launch_project_f32(culsh_ctx* ctx, const float* X, const float* P, const float* b,
@@ -188,6 +200,19 @@ culsh_status launch_sig_to_keys(culsh_ctx* ctx, const uint8_t* sig, size_t n_ite
 // value that only the device knows yet
 culsh_status launch_keys_to_sig(culsh_ctx* ctx, const uint32_t* keys, size_t count, const uint64_t* count_dev,
                                 int S, KeyEnc enc, int W, uint8_t* sig);
+
+// ---------------------------------------------------------------- p-stable key compression (pscodec.hip)
+// Measures the value range of every (table, hash) of sig [T][n][H]; when the ranges are
+// narrow, fills ix->psc, sets ix->enc = ENC_PSC and ix->key_w, and reports compressed = true.
+culsh_status ps_build_codec(culsh_ctx* ctx, const int32_t* sig, int n, int T, int H, culsh_index* ix,
+                            bool* compressed);
+// int32 hashes [T][rows][H] -> compressed key words [T][rows][ix->key_w]
+culsh_status launch_ps_compress(culsh_ctx* ctx, const int32_t* sig, size_t rows, int T, int H, const culsh_index* ix,
+                                uint32_t* keys);
+// ix->bucket_keys -> little-endian int32 signatures of the buckets (needs table_bucket_offsets)
+culsh_status launch_ps_keys_to_sig(culsh_ctx* ctx, const culsh_index* ix, size_t count, const uint64_t* count_dev,
+                                   uint8_t* sig);
+void free_ps_codec(culsh_index* ix);
 
 // ---------------------------------------------------------------- sort (sort.hip)
 // Stable sort of each table's n items by key words (word 0 most significant), starting

@@ -204,7 +204,10 @@ culsh_status build_index_from_sorted(culsh_ctx* ctx, const uint32_t* sorted_keys
                        sorted_keys, rows_sorted_owned, N, n, T, W, tile_base, total_dev, index->bucket_candidate_offsets,
                        index->bucket_keys, index->table_bucket_offsets, item_to_bucket_opt);
     CULSH_LAUNCH_CHECK();
-    CULSH_TRY(launch_keys_to_sig(ctx, index->bucket_keys, B_bound, total_dev, S, enc, W, index->all_bucket_signatures));
+    if (enc == ENC_PSC)
+        CULSH_TRY(launch_ps_keys_to_sig(ctx, index, B_bound, total_dev, index->all_bucket_signatures));
+    else
+        CULSH_TRY(launch_keys_to_sig(ctx, index->bucket_keys, B_bound, total_dev, S, enc, W, index->all_bucket_signatures));
     if (deferred) CULSH_TRY(read_back_u64(ctx, total_dev, 1, &n_buckets64));
     index->n_total_buckets = static_cast<int>(n_buckets64);
     return CULSH_OK;
@@ -225,7 +228,14 @@ culsh_status fit_index_from_keys(culsh_ctx* ctx, uint32_t* keys, int n, int T, i
     uint32_t* sorted = nullptr;
     uint32_t bits_vary[64];
     const uint32_t* known_vary = nullptr;
-    if (enc == ENC_BITS && W <= 64) {
+    if (enc == ENC_PSC && W <= 64) {
+        const int nb = H * index->psc.bits;  // compressed keys occupy the top H*bits bits
+        for (int w = 0; w < W; ++w) {
+            const int nbits = std::min(32, nb - 32 * w);
+            bits_vary[w] = nbits >= 32 ? 0xFFFFFFFFu : (0xFFFFFFFFu << (32 - nbits));
+        }
+        known_vary = bits_vary;
+    } else if (enc == ENC_BITS && W <= 64) {
         // sign-bit keys: exactly the top S bits of the key string can differ, so the radix
         // passes are known without looking at the data (and without a host round trip)
         for (int w = 0; w < W; ++w) {

@@ -234,7 +234,7 @@ __global__ __launch_bounds__(NTHREADS) void project_f32_kernel(ProjArgs a) {
                 const int col = ct * BN + wn * 64 + j * 32 + r32;
                 if (col >= TH) continue;
                 const int t = col / H, h = col - t * H;
-                const float bias = (EPI == EPI_FLOOR_KEYS || EPI == EPI_FLOOR_I32) ? a.b[col] : 0.f;
+                const float bias = (EPI == EPI_FLOOR_I32) ? a.b[col] : 0.f;
 #pragma unroll
                 for (int v = 0; v < 16; ++v) {
                     const int row = rt * BM + wm * 64 + i * 32 + 8 * (v >> 2) + 4 * half + (v & 3);
@@ -245,11 +245,7 @@ __global__ __launch_bounds__(NTHREADS) void project_f32_kernel(ProjArgs a) {
                         static_cast<uint8_t*>(a.out)[off] =
                             static_cast<uint8_t>((__float_as_uint(x) >> 31) ^ 1u);
                     } else {
-                        const int32_t f = static_cast<int32_t>(floorf(x + bias));  // pslsh/hash.cuh:46
-                        if (EPI == EPI_FLOOR_I32)
-                            static_cast<int32_t*>(a.out)[off] = f;
-                        else
-                            static_cast<uint32_t*>(a.out)[off] = __builtin_bswap32(static_cast<uint32_t>(f));
+                        static_cast<int32_t*>(a.out)[off] = static_cast<int32_t>(floorf(x + bias));  // pslsh/hash.cuh:46
                     }
                 }
             }
@@ -314,7 +310,7 @@ culsh_status launch_project_f32(culsh_ctx* ctx, const float* X, const float* P, 
                                 int n, int d, int T, int H, ProjEpilogue epi, void* out) {
     CULSH_REQUIRE(X && P && out, CULSH_ERR_INVALID, "projection: null pointer");
     CULSH_REQUIRE(n > 0 && d > 0 && T > 0 && H > 0, CULSH_ERR_INVALID, "projection: sizes must be positive");
-    const bool floor_epi = (epi == EPI_FLOOR_KEYS || epi == EPI_FLOOR_I32);
+    const bool floor_epi = (epi == EPI_FLOOR_I32);
     CULSH_REQUIRE(!floor_epi || b, CULSH_ERR_INVALID, "projection: bias is required");
     CULSH_REQUIRE(static_cast<long long>(T) * H < (1ll << 30), CULSH_ERR_LIMIT, "T*H too large");
     long long n_vcols;
@@ -345,7 +341,6 @@ culsh_status launch_project_f32(culsh_ctx* ctx, const float* X, const float* P, 
     switch (epi) {
         PROJ_CASE(EPI_SIGN_KEYS)
         PROJ_CASE(EPI_SIGN_BYTES)
-        PROJ_CASE(EPI_FLOOR_KEYS)
         PROJ_CASE(EPI_FLOOR_I32)
     }
 #undef PROJ_CASE

@@ -1,0 +1,204 @@
+// Order-preserving key compression for p-stable signatures.
+//
+// A p-stable signature is H little-endian int32 hashes, and buckets are ordered by the
+// raw bytes (core/fit.cuh:265-272), i.e. every hash is ordered by its byte-swapped value.
+// Sorting those 4*H bytes directly needs up to 4*H radix passes over 4*H-byte keys.  The
+// hashes of real data span a few dozen values per hash function, so each hash is replaced
+// by its rank (1-based, 0 = "value never seen at fit time") in byte-swapped order among
+// the values of [min, max] observed for that (table, hash).  Ranks of `bits` bits are
+// concatenated most-significant first, which keeps the bucket order bit for bit and
+// shrinks keys from 32*H to bits*H bits.  The inverse table restores the signatures of
+// the buckets in the reference layout.
+#include <algorithm>
+#include <climits>
+#include <vector>
+
+#include "common.hpp"
+
+namespace culsh_amd {
+namespace {
+
+__global__ __launch_bounds__(256) void ps_minmax_kernel(const int32_t* __restrict__ sig, int n, int H,
+                                                       int32_t* __restrict__ mm /*[T*H][2]*/) {
+    __shared__ int32_t smin[1024], smax[1024];
+    const int t = blockIdx.y;
+    for (int h = threadIdx.x; h < H; h += 256) { smin[h] = INT_MAX; smax[h] = INT_MIN; }
+    __syncthreads();
+    const int32_t* ts = sig + static_cast<size_t>(t) * n * H;
+    const size_t total = static_cast<size_t>(n) * H;
+    const size_t stride = static_cast<size_t>(gridDim.x) * 256;
+    size_t e = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
+    if (256 % H == 0) {  // the thread always meets the same hash position
+        int32_t lo = INT_MAX, hi = INT_MIN;
+#pragma unroll 4
+        for (; e < total; e += stride) {
+            const int32_t v = ts[e];
+            lo = min(lo, v);
+            hi = max(hi, v);
+        }
+        if (lo <= hi) {
+            atomicMin(&smin[threadIdx.x % H], lo);
+            atomicMax(&smax[threadIdx.x % H], hi);
+        }
+    } else {
+        for (; e < total; e += stride) {
+            const int32_t v = ts[e];
+            const int h = static_cast<int>(e % H);
+            if (v < smin[h]) atomicMin(&smin[h], v);
+            if (v > smax[h]) atomicMax(&smax[h], v);
+        }
+    }
+    __syncthreads();
+    for (int h = threadIdx.x; h < H; h += 256) {
+        if (smin[h] <= smax[h]) {
+            atomicMin(&mm[(t * H + h) * 2 + 0], smin[h]);
+            atomicMax(&mm[(t * H + h) * 2 + 1], smax[h]);
+        }
+    }
+}
+
+__global__ __launch_bounds__(256) void ps_compress_kernel(const int32_t* __restrict__ sig, size_t rows, int T, int H,
+                                                         int bits, int rmax, int W,
+                                                         const int32_t* __restrict__ vmin,
+                                                         const int32_t* __restrict__ range,
+                                                         const uint32_t* __restrict__ fwd,
+                                                         uint32_t* __restrict__ keys) {
+    const size_t item = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (item >= rows * T) return;
+    const int t = static_cast<int>(item / rows);
+    const int32_t* s = sig + item * H;
+    uint32_t* k = keys + item * W;
+    unsigned long long acc = 0;
+    int nbits = 0, w = 0;
+    for (int h = 0; h < H; ++h) {
+        const int c = t * H + h;
+        const long long idx = static_cast<long long>(s[h]) - vmin[c];
+        const uint32_t code = (idx >= 0 && idx < range[c]) ? fwd[static_cast<size_t>(c) * rmax + idx] + 1u : 0u;
+        acc = (acc << bits) | code;
+        nbits += bits;
+        if (nbits >= 32) {
+            k[w++] = static_cast<uint32_t>(acc >> (nbits - 32));
+            nbits -= 32;
+            acc &= (1ull << nbits) - 1ull;
+        }
+    }
+    if (nbits > 0) k[w++] = static_cast<uint32_t>(acc << (32 - nbits));
+}
+
+__global__ __launch_bounds__(256) void ps_keys_to_sig_kernel(const uint32_t* __restrict__ keys, size_t count,
+                                                            const uint64_t* __restrict__ count_dev,
+                                                            const int32_t* __restrict__ table_bucket_offsets, int T,
+                                                            int H, int bits, int rmax, int W,
+                                                            const int32_t* __restrict__ inv,
+                                                            int32_t* __restrict__ sig) {
+    const size_t idx = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (count_dev) count = min(count, static_cast<size_t>(*count_dev));
+    if (idx >= count * H) return;
+    const size_t bucket = idx / H;
+    const int h = static_cast<int>(idx - bucket * H);
+    int lo = 0, hi = T;  // largest t with table_bucket_offsets[t] <= bucket
+    while (hi - lo > 1) {
+        const int mid = (lo + hi) >> 1;
+        if (static_cast<size_t>(table_bucket_offsets[mid]) <= bucket) lo = mid; else hi = mid;
+    }
+    const uint32_t* k = keys + bucket * W;
+    const int o = h * bits, w0 = o >> 5, sh = o & 31;
+    const unsigned long long two = (static_cast<unsigned long long>(k[w0]) << 32) | (w0 + 1 < W ? k[w0 + 1] : 0u);
+    const uint32_t code = static_cast<uint32_t>(two >> (64 - sh - bits)) & ((1u << bits) - 1u);
+    sig[idx] = code ? inv[static_cast<size_t>(lo * H + h) * rmax + (code - 1u)] : 0;
+}
+
+}  // namespace
+
+void free_ps_codec(culsh_index* ix) {
+    (void)hipFree(ix->psc.vmin);
+    (void)hipFree(ix->psc.range);
+    (void)hipFree(ix->psc.fwd);
+    (void)hipFree(ix->psc.inv);
+    ix->psc = PsCodec();
+}
+
+culsh_status ps_build_codec(culsh_ctx* ctx, const int32_t* sig, int n, int T, int H, culsh_index* ix,
+                            bool* compressed) {
+    *compressed = false;
+    const int TH = T * H;
+    if (H > 1024) return CULSH_OK;
+    std::vector<int32_t> mm(static_cast<size_t>(TH) * 2);
+    for (int c = 0; c < TH; ++c) { mm[2 * c] = INT_MAX; mm[2 * c + 1] = INT_MIN; }
+    int32_t* mm_dev = nullptr;
+    CULSH_TRY(arena_alloc_t(ctx, mm.size(), &mm_dev));
+    CULSH_HIP(hipMemcpyAsync(mm_dev, mm.data(), mm.size() * sizeof(int32_t), hipMemcpyHostToDevice, ctx->stream));
+    CULSH_HIP(hipStreamSynchronize(ctx->stream));  // `mm` is pageable: the copy must not outlive this scope's reuse
+    const unsigned bx = std::max(1u, std::min(256u, div_up(static_cast<size_t>(n) * H, 256 * 16)));
+    CULSH_LAUNCH(ctx, ps_minmax_kernel, dim3(bx, T), dim3(256), 0, ctx->stream, sig, n, H, mm_dev);
+    CULSH_LAUNCH_CHECK();
+    CULSH_HIP(hipMemcpyAsync(mm.data(), mm_dev, mm.size() * sizeof(int32_t), hipMemcpyDeviceToHost, ctx->stream));
+    CULSH_HIP(hipStreamSynchronize(ctx->stream));
+
+    long long rmax = 1;
+    for (int c = 0; c < TH; ++c) rmax = std::max(rmax, static_cast<long long>(mm[2 * c + 1]) - mm[2 * c] + 1);
+    int bits = 1;
+    while ((1ll << bits) < rmax + 1) ++bits;  // codes 1..range, 0 reserved
+    const int W = (H * bits + 31) / 32;
+    if (bits > 12 || W >= H) return CULSH_OK;  // wide value ranges: keep the plain byte order keys
+
+    std::vector<int32_t> vmin(TH), range(TH), inv(static_cast<size_t>(TH) * rmax, 0);
+    std::vector<uint32_t> fwd(static_cast<size_t>(TH) * rmax, 0);
+    std::vector<std::pair<uint32_t, int32_t>> order;
+    for (int c = 0; c < TH; ++c) {
+        vmin[c] = mm[2 * c];
+        range[c] = static_cast<int32_t>(static_cast<long long>(mm[2 * c + 1]) - mm[2 * c] + 1);
+        order.clear();
+        for (int i = 0; i < range[c]; ++i) {
+            const int32_t v = vmin[c] + i;
+            order.emplace_back(__builtin_bswap32(static_cast<uint32_t>(v)), v);  // byte order of a little-endian int32
+        }
+        std::sort(order.begin(), order.end());
+        for (int r = 0; r < range[c]; ++r) {
+            fwd[static_cast<size_t>(c) * rmax + (order[r].second - vmin[c])] = static_cast<uint32_t>(r);
+            inv[static_cast<size_t>(c) * rmax + r] = order[r].second;
+        }
+    }
+    PsCodec& pc = ix->psc;
+    pc.bits = bits;
+    pc.rmax = static_cast<int>(rmax);
+    CULSH_HIP(hipMalloc(&pc.vmin, TH * sizeof(int32_t)));
+    CULSH_HIP(hipMalloc(&pc.range, TH * sizeof(int32_t)));
+    CULSH_HIP(hipMalloc(&pc.fwd, fwd.size() * sizeof(uint32_t)));
+    CULSH_HIP(hipMalloc(&pc.inv, inv.size() * sizeof(int32_t)));
+    CULSH_HIP(hipMemcpy(pc.vmin, vmin.data(), TH * sizeof(int32_t), hipMemcpyHostToDevice));
+    CULSH_HIP(hipMemcpy(pc.range, range.data(), TH * sizeof(int32_t), hipMemcpyHostToDevice));
+    CULSH_HIP(hipMemcpy(pc.fwd, fwd.data(), fwd.size() * sizeof(uint32_t), hipMemcpyHostToDevice));
+    CULSH_HIP(hipMemcpy(pc.inv, inv.data(), inv.size() * sizeof(int32_t), hipMemcpyHostToDevice));
+    ix->enc = ENC_PSC;
+    ix->key_w = W;
+    *compressed = true;
+    return CULSH_OK;
+}
+
+culsh_status launch_ps_compress(culsh_ctx* ctx, const int32_t* sig, size_t rows, int T, int H, const culsh_index* ix,
+                                uint32_t* keys) {
+    const size_t items = rows * T;
+    if (items == 0) return CULSH_OK;
+    CULSH_REQUIRE(items / 256 < (1ull << 31), CULSH_ERR_LIMIT, "too many items");
+    const PsCodec& pc = ix->psc;
+    CULSH_LAUNCH(ctx, ps_compress_kernel, dim3(div_up(items, 256)), dim3(256), 0, ctx->stream, sig, rows, T, H,
+                 pc.bits, pc.rmax, ix->key_w, pc.vmin, pc.range, pc.fwd, keys);
+    CULSH_LAUNCH_CHECK();
+    return CULSH_OK;
+}
+
+culsh_status launch_ps_keys_to_sig(culsh_ctx* ctx, const culsh_index* ix, size_t count, const uint64_t* count_dev,
+                                   uint8_t* sig) {
+    if (count == 0) return CULSH_OK;
+    const size_t total = count * ix->n_hashes;
+    CULSH_REQUIRE(total / 256 < (1ull << 31), CULSH_ERR_LIMIT, "too many buckets");
+    const PsCodec& pc = ix->psc;
+    CULSH_LAUNCH(ctx, ps_keys_to_sig_kernel, dim3(div_up(total, 256)), dim3(256), 0, ctx->stream, ix->bucket_keys,
+                 count, count_dev, ix->table_bucket_offsets, ix->n_hash_tables, ix->n_hashes, pc.bits, pc.rmax,
+                 ix->key_w, pc.inv, reinterpret_cast<int32_t*>(sig));
+    CULSH_LAUNCH_CHECK();
+    return CULSH_OK;
+}
+
+}  // namespace culsh_amd
