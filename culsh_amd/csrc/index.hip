@@ -28,25 +28,46 @@ __device__ __forceinline__ uint32_t is_head(const uint32_t* __restrict__ keys, s
     return diff != 0u;
 }
 
-// Flags of the IB_ITEMS consecutive items owned by one thread.  One-word keys of a full
-// run are fetched with two 16-byte loads plus the predecessor's key.
+// Flags of the IB_ITEMS consecutive items owned by one thread.  Keys of 1, 2 or 4 words of a
+// full run are fetched with 16-byte loads plus the predecessor's key.
+template <int KW>
+__device__ __forceinline__ uint64_t thread_flags_vec(const uint32_t* __restrict__ keys, size_t base, int n,
+                                                     uint32_t (&flag)[IB_ITEMS]) {
+    constexpr int NV = IB_ITEMS * KW / 4;  // uint4 loads per thread
+    uint32_t k[(IB_ITEMS + 1) * KW];
+#pragma unroll
+    for (int w = 0; w < KW; ++w) k[w] = base ? keys[(base - 1) * KW + w] : 0u;
+#pragma unroll
+    for (int v = 0; v < NV; ++v) {
+        const uint4 q = *reinterpret_cast<const uint4*>(keys + base * KW + 4 * v);
+        k[KW + 4 * v + 0] = q.x;
+        k[KW + 4 * v + 1] = q.y;
+        k[KW + 4 * v + 2] = q.z;
+        k[KW + 4 * v + 3] = q.w;
+    }
+    uint64_t c = 0;
+    uint32_t r = static_cast<uint32_t>(base % n);  // position inside the table
+#pragma unroll
+    for (int i = 0; i < IB_ITEMS; ++i) {
+        uint32_t diff = 0;
+#pragma unroll
+        for (int w = 0; w < KW; ++w) diff |= k[(i + 1) * KW + w] ^ k[i * KW + w];
+        flag[i] = (r == 0u) || (diff != 0u);
+        c += flag[i];
+        if (++r == static_cast<uint32_t>(n)) r = 0u;
+    }
+    return c;
+}
+
 __device__ __forceinline__ uint64_t thread_flags(const uint32_t* __restrict__ keys, size_t base, size_t N, int n,
                                                  int W, uint32_t (&flag)[IB_ITEMS]) {
-    uint64_t c = 0;
-    if (W == 1 && base + IB_ITEMS <= N) {
-        static_assert(IB_ITEMS == 8, "two uint4 loads cover the thread's items");
-        const uint4 a = *reinterpret_cast<const uint4*>(keys + base);
-        const uint4 b = *reinterpret_cast<const uint4*>(keys + base + 4);
-        const uint32_t k[9] = {base ? keys[base - 1] : 0u, a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
-        uint32_t r = static_cast<uint32_t>(base % n);  // position inside the table
-#pragma unroll
-        for (int i = 0; i < IB_ITEMS; ++i) {
-            flag[i] = (r == 0u) || (k[i + 1] != k[i]);
-            if (++r == static_cast<uint32_t>(n)) r = 0u;
-            c += flag[i];
-        }
-        return c;
+    static_assert(IB_ITEMS == 8, "vector paths assume 8 items per thread");
+    if (base + IB_ITEMS <= N) {
+        if (W == 1) return thread_flags_vec<1>(keys, base, n, flag);
+        if (W == 2) return thread_flags_vec<2>(keys, base, n, flag);
+        if (W == 4) return thread_flags_vec<4>(keys, base, n, flag);
     }
+    uint64_t c = 0;
 #pragma unroll
     for (int i = 0; i < IB_ITEMS; ++i) {
         flag[i] = (base + i < N) ? is_head(keys, base + i, n, W) : 0u;

@@ -138,11 +138,13 @@ __global__ __launch_bounds__(256) void radix_scan_kernel(uint32_t* __restrict__ 
     }
 }
 
-template <bool ONE_WORD>
+// KW: key words known at compile time (1, 2 or 4: keys move as one vector), 0 = any W.
+template <int KW>
 __global__ __launch_bounds__(SORT_THREADS) void radix_scatter_kernel(
     const uint32_t* __restrict__ keys_in, const int32_t* __restrict__ rows_in,
     uint32_t* __restrict__ keys_out, int32_t* __restrict__ rows_out,
     const uint32_t* __restrict__ hist_scanned, int n, int W, int word, int shift, int tiles) {
+    constexpr bool ONE_WORD = (KW == 1);
     constexpr int NW = SORT_THREADS / 64;
     __shared__ uint32_t whist[NW][256];   // per-wave digit counts, then per-wave offsets inside a digit run
     __shared__ uint32_t dstart[256];      // start of each digit's run inside the sorted tile
@@ -231,9 +233,23 @@ __global__ __launch_bounds__(SORT_THREADS) void radix_scatter_kernel(
         } else {
             const int src = tile0 + static_cast<int>(st_key[slot]);
             const uint32_t* ks = keys_in + (tbase + src) * W;
-            const size_t dst = tbase + static_cast<uint32_t>(gbase[(ks[word] >> shift) & 255u] + slot);
-            for (int w = 0; w < W; ++w) keys_out[dst * W + w] = ks[w];
-            rows_out[dst] = rows_in ? rows_in[tbase + src] : src;
+            if (KW == 4) {
+                const uint4 v = *reinterpret_cast<const uint4*>(ks);
+                const uint32_t kd = word == 0 ? v.x : (word == 1 ? v.y : (word == 2 ? v.z : v.w));
+                const size_t dst = tbase + static_cast<uint32_t>(gbase[(kd >> shift) & 255u] + slot);
+                *reinterpret_cast<uint4*>(keys_out + dst * 4) = v;
+                rows_out[dst] = rows_in ? rows_in[tbase + src] : src;
+            } else if (KW == 2) {
+                const uint2 v = *reinterpret_cast<const uint2*>(ks);
+                const uint32_t kd = word == 0 ? v.x : v.y;
+                const size_t dst = tbase + static_cast<uint32_t>(gbase[(kd >> shift) & 255u] + slot);
+                *reinterpret_cast<uint2*>(keys_out + dst * 2) = v;
+                rows_out[dst] = rows_in ? rows_in[tbase + src] : src;
+            } else {
+                const size_t dst = tbase + static_cast<uint32_t>(gbase[(ks[word] >> shift) & 255u] + slot);
+                for (int w = 0; w < W; ++w) keys_out[dst * W + w] = ks[w];
+                rows_out[dst] = rows_in ? rows_in[tbase + src] : src;
+            }
         }
     }
 }
@@ -308,12 +324,15 @@ culsh_status sort_tables(culsh_ctx* ctx, uint32_t* keys_in, uint32_t* keys_tmp, 
         CULSH_LAUNCH(ctx, radix_scan_kernel, dim3(T, SCAN_PARTS), dim3(256), 0, ctx->stream, hist,
                      dtot + static_cast<size_t>(p) * T * 256, tiles);
         CULSH_LAUNCH_CHECK();
-        if (W == 1)
-            CULSH_LAUNCH(ctx, radix_scatter_kernel<true>, grid, dim3(SORT_THREADS), 0, ctx->stream, kin, rin,
-                               kout, rout, hist, n, W, passes[p].word, passes[p].shift, tiles);
-        else
-            CULSH_LAUNCH(ctx, radix_scatter_kernel<false>, grid, dim3(SORT_THREADS), 0, ctx->stream, kin, rin,
-                               kout, rout, hist, n, W, passes[p].word, passes[p].shift, tiles);
+        const bool aligned = reinterpret_cast<uintptr_t>(kin) % 16 == 0 && reinterpret_cast<uintptr_t>(kout) % 16 == 0;
+#define SCATTER(KW)                                                                                              \
+    CULSH_LAUNCH(ctx, radix_scatter_kernel<KW>, grid, dim3(SORT_THREADS), 0, ctx->stream, kin, rin, kout, rout, hist, \
+                 n, W, passes[p].word, passes[p].shift, tiles)
+        if (W == 1) SCATTER(1);
+        else if (W == 2 && aligned) SCATTER(2);
+        else if (W == 4 && aligned) SCATTER(4);
+        else SCATTER(0);
+#undef SCATTER
         CULSH_LAUNCH_CHECK();
         std::swap(kin, kout);
         rin = rout;
