@@ -347,10 +347,7 @@ static culsh_status concat_candidates(culsh_ctx* ctx, const std::vector<culsh_ca
 // query over key words that are already in the arena
 static culsh_status query_keys(culsh_ctx* ctx, const uint32_t* q_keys, int nq, const culsh_index* ix,
                                culsh_candidates* out) {
-    int32_t* matched = nullptr;
-    CULSH_TRY(arena_alloc_t(ctx, static_cast<size_t>(nq) * ix->n_hash_tables, &matched));
-    CULSH_TRY(launch_find_matching_buckets(ctx, q_keys, nq, ix, matched));
-    return query_from_matched(ctx, matched, nq, ix, out);
+    return query_from_keys(ctx, q_keys, nq, ix, out);
 }
 
 template <typename T>

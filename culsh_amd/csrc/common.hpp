@@ -235,10 +235,17 @@ culsh_status fit_index_from_keys(culsh_ctx* ctx, uint32_t* keys, int n, int T, i
                                  KeyEnc enc, int W, int32_t* item_to_bucket_opt, culsh_index* index);
 
 // ---------------------------------------------------------------- query (query.hip)
+// `matched` ([n_queries][T] bucket ids, -1 = none) and `spans` ([n_queries][T] int2 (start,
+// length) into all_candidate_indices) are both optional outputs; with `spans` the sum of
+// the span lengths is added to *raw_total (device).
 culsh_status launch_find_matching_buckets(culsh_ctx* ctx, const uint32_t* q_keys, int n_queries,
-                                          const culsh_index* index, int32_t* matched);
+                                          const culsh_index* index, int32_t* matched, void* spans = nullptr,
+                                          unsigned long long* raw_total = nullptr);
 culsh_status query_from_matched(culsh_ctx* ctx, const int32_t* matched, int n_queries,
                                 const culsh_index* index, culsh_candidates* out);
+// lookup + candidate retrieval from key words [T][n_queries][key_w]
+culsh_status query_from_keys(culsh_ctx* ctx, const uint32_t* q_keys, int n_queries, const culsh_index* index,
+                             culsh_candidates* out);
 
 // ---------------------------------------------------------------- scans (scan.hip)
 // Exclusive prefix sum of `n` u64 values; out[n] receives the total (out has n+1 slots).

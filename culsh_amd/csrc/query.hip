@@ -7,10 +7,17 @@
 // Here one workgroup owns a query and marks the row ids of its bucket spans in a bitmap
 // held in LDS (up to 2^20 rows per pass of 128 KiB); reading the bitmap in order yields
 // the ascending duplicate-free list directly, so raw candidates are never written to
-// memory and nothing is sorted.  A first launch counts, a scan places the queries, a
-// second launch emits; memory use is O(unique candidates).
+// memory and nothing is sorted.
+//
+// Where a query's list starts in the output depends on the counts of all queries before
+// it.  When the row range fits one bitmap pass, a single launch does everything: each
+// workgroup publishes its count and obtains the sum of its predecessors' counts by
+// looking back over their published values (a chained scan), then stores its list.  The
+// output is allocated for the number of raw candidates, an upper bound of the result.
+// Larger row ranges take two launches (count, scan, emit) with several passes each.
 #include <algorithm>
 #include <cstdlib>
+#include <vector>
 
 #include "block_utils.hpp"
 #include "common.hpp"
@@ -20,15 +27,23 @@ namespace {
 
 constexpr int DD_THREADS = 1024;
 
+// Binary search of every (query, table) key among the table's sorted bucket keys; writes
+// the matched bucket id (-1 = none) and / or its span (start, length) of candidate rows.
 __global__ __launch_bounds__(256) void lookup_kernel(const uint32_t* __restrict__ q_keys,
                                                     const uint32_t* __restrict__ bucket_keys,
                                                     const int32_t* __restrict__ table_bucket_offsets,
-                                                    int n_queries, int T, int W, int32_t* __restrict__ matched) {
+                                                    const int32_t* __restrict__ bucket_candidate_offsets,
+                                                    int n_queries, int T, int W, int32_t* __restrict__ matched,
+                                                    int2* __restrict__ spans,
+                                                    unsigned long long* __restrict__ raw_total) {
+    __shared__ unsigned long long block_raw;
+    if (threadIdx.x == 0) block_raw = 0ull;
+    __syncthreads();
     const size_t idx = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
-    if (idx >= static_cast<size_t>(n_queries) * T) return;
-    const int q = static_cast<int>(idx / T), t = static_cast<int>(idx - static_cast<size_t>(q) * T);
+    const bool live = idx < static_cast<size_t>(n_queries) * T;
+    const int q = live ? static_cast<int>(idx / T) : 0, t = live ? static_cast<int>(idx - static_cast<size_t>(q) * T) : 0;
     const uint32_t* key = q_keys + (static_cast<size_t>(t) * n_queries + q) * W;
-    int lo = table_bucket_offsets[t], hi = table_bucket_offsets[t + 1] - 1;
+    int lo = live ? table_bucket_offsets[t] : 0, hi = live ? table_bucket_offsets[t + 1] - 1 : -1;
     int found = -1;
     while (lo <= hi) {
         const int mid = lo + ((hi - lo) >> 1);
@@ -38,119 +53,210 @@ __global__ __launch_bounds__(256) void lookup_kernel(const uint32_t* __restrict_
         if (cmp == 0) { found = mid; break; }
         if (cmp < 0) hi = mid - 1; else lo = mid + 1;
     }
-    matched[idx] = found;
+    if (live && matched) matched[idx] = found;
+    if (spans) {
+        int2 sp = make_int2(0, 0);
+        if (found >= 0) {
+            sp.x = bucket_candidate_offsets[found];
+            sp.y = bucket_candidate_offsets[found + 1] - sp.x;
+        }
+        if (live) spans[idx] = sp;
+        // number of raw candidates: one atomic per wavefront in LDS, one per workgroup in memory
+        const unsigned long long wsum = wave_sum(static_cast<unsigned long long>(sp.y));
+        if ((threadIdx.x & 63) == 0 && wsum) atomicAdd(&block_raw, wsum);
+        __syncthreads();
+        if (threadIdx.x == 0 && block_raw) atomicAdd(raw_total, block_raw);
+    }
 }
 
-struct DedupArgs {
-    const int32_t* matched;                   // [n_queries][T]
-    const int32_t* bucket_candidate_offsets;  // [B+1]
-    const int32_t* cand;                      // all_candidate_indices
-    const uint64_t* offsets;                  // EMIT: per-query output offsets
-    uint64_t* counts;                         // COUNT: per-query unique counts
-    int32_t* out;                             // EMIT: candidate indices
-    int T, n;
-    int wpt;       // bitmap words per thread (power of two); a pass covers DD_THREADS*wpt*32 rows
-    int n_chunks;  // passes over the row range
-    unsigned long long* ticks;  // optional [8] phase timers (wall clock ticks of thread 0), or null
-};
+// Span of every matched bucket (count_candidates_kernel, core/query.cuh:114-132).
+__global__ __launch_bounds__(256) void span_kernel(const int32_t* __restrict__ matched,
+                                                  const int32_t* __restrict__ bucket_candidate_offsets,
+                                                  size_t pairs, int2* __restrict__ spans,
+                                                  unsigned long long* __restrict__ raw_total) {
+    __shared__ unsigned long long block_raw;
+    if (threadIdx.x == 0) block_raw = 0ull;
+    __syncthreads();
+    const size_t idx = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    int2 sp = make_int2(0, 0);
+    if (idx < pairs) {
+        const int b = matched[idx];
+        if (b >= 0) {
+            sp.x = bucket_candidate_offsets[b];
+            sp.y = bucket_candidate_offsets[b + 1] - sp.x;
+        }
+        spans[idx] = sp;
+    }
+    const unsigned long long wsum = wave_sum(static_cast<unsigned long long>(sp.y));
+    if ((threadIdx.x & 63) == 0 && wsum) atomicAdd(&block_raw, wsum);
+    __syncthreads();
+    if (threadIdx.x == 0 && block_raw) atomicAdd(raw_total, block_raw);
+}
 
 constexpr int NWAVES = DD_THREADS / 64;
-constexpr int WALK_U = 8;              // 64-row segments in flight per wavefront
-constexpr uint32_t ROUND = DD_THREADS * 64u;  // flat candidates per segment-table round
+constexpr int WALK_U = 16;  // pieces in flight per wavefront
 
-// Visits every row id of the concatenated spans ("flat" order: span 0, span 1, ...), 64
-// consecutive ids per wavefront step so that no lane idles on short spans.  The span that
-// owns the first id of every 64-id segment is looked up once per segment (one binary
-// search per thread, all segments in parallel) and kept in `lut`; lanes then only step
-// forward over span boundaries.  Contains barriers: all threads must call it.
+// Visits every row id of the query's spans.  The spans are cut into pieces of up to 64
+// consecutive ids (a piece never crosses a span boundary), pieces are dealt round-robin to
+// the wavefronts, and a wavefront reads a piece with one load per lane.  Where piece p
+// starts is looked up once per piece (one binary search per thread over the spans'
+// piece counts, all pieces of a round in parallel) and kept in `tab`, so the per-lane
+// work is an add, a compare and the load.  Contains barriers: all threads must call it.
 template <typename F>
 __device__ __forceinline__ void walk_candidates(const int32_t* __restrict__ cand, const int* s_start,
-                                                const uint32_t* s_pref, int T, uint32_t total, uint32_t* lut,
-                                                F&& f) {
+                                                const int* s_len, const uint32_t* s_ppref, int T,
+                                                uint32_t n_pieces, int2* tab, F&& f) {
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    for (uint32_t r0 = 0; r0 < total; r0 += ROUND) {
-        const uint32_t fseg = r0 + static_cast<uint32_t>(tid) * 64u;
-        if (fseg < total) {
-            int tl = 0, th = T;  // largest t with s_pref[t] <= fseg
+    for (uint32_t r0 = 0; r0 < n_pieces; r0 += DD_THREADS) {
+        const uint32_t pc = r0 + static_cast<uint32_t>(tid);
+        if (pc < n_pieces) {
+            int tl = 0, th = T;  // largest t with s_ppref[t] <= pc; that span owns the piece
             while (th - tl > 1) {
                 const int mid = (tl + th) >> 1;
-                if (s_pref[mid] <= fseg) tl = mid; else th = mid;
+                if (s_ppref[mid] <= pc) tl = mid; else th = mid;
             }
-            lut[tid] = static_cast<uint32_t>(tl);
+            const int first = static_cast<int>(pc - s_ppref[tl]) * 64;
+            tab[tid] = make_int2(s_start[tl] + first, min(64, s_len[tl] - first));
         }
         __syncthreads();
-        const uint32_t nseg = min(static_cast<uint32_t>(DD_THREADS), (total - r0 + 63u) >> 6);
-        for (uint32_t seg0 = wave; seg0 < nseg; seg0 += NWAVES * WALK_U) {
+        const uint32_t here = min(static_cast<uint32_t>(DD_THREADS), n_pieces - r0);
+        for (uint32_t p0 = wave; p0 < here; p0 += NWAVES * WALK_U) {
             int rows[WALK_U];
 #pragma unroll
             for (int u = 0; u < WALK_U; ++u) {
-                const uint32_t seg = seg0 + u * NWAVES;
+                const uint32_t pi = p0 + u * NWAVES;
                 rows[u] = -1;
-                if (seg < nseg) {  // uniform across the wavefront
-                    const uint32_t fi = r0 + seg * 64u + lane;
-                    if (fi < total) {
-                        uint32_t t = lut[seg];
-                        while (fi >= s_pref[t + 1]) ++t;
-                        rows[u] = cand[s_start[t] + (fi - s_pref[t])];
-                    }
+                if (pi < here) {  // uniform across the wavefront
+                    const int2 e = tab[pi];
+                    if (lane < e.y) rows[u] = cand[e.x + lane];
                 }
             }
 #pragma unroll
             for (int u = 0; u < WALK_U; ++u)
                 if (rows[u] >= 0) f(rows[u]);
         }
-        __syncthreads();  // lut is rewritten by the next round
+        __syncthreads();  // tab is rewritten by the next round
     }
 }
 
-// One workgroup per query.  COUNT (EMIT = false) marks the rows of the query's spans in an
-// LDS bitmap and counts the bits it set first.  EMIT marks them again, builds a rank table
-// (marked rows before every group of 8 bitmap words) and lets every occurrence of a row
-// store the row id at its rank: duplicates store the same value to the same place, so the
-// output is ascending and duplicate-free without sorting, flagging or compaction.
-template <bool EMIT>
+enum DedupMode { DD_COUNT = 0, DD_EMIT = 1, DD_FUSED = 2 };
+
+struct DedupArgs {
+    const int2* spans;            // [n_queries][T] (start, length) in `cand`
+    const int32_t* cand;          // all_candidate_indices
+    int32_t* out;                 // EMIT, FUSED: candidate indices
+    uint64_t* counts;             // COUNT, FUSED: per-query unique counts (written)
+    uint64_t* offsets;            // EMIT: per-query output offsets (read); FUSED: [n_queries+1] (written)
+    unsigned long long* state;    // FUSED: [n_queries] published counts / running sums, zero before the launch
+    unsigned int* err;            // FUSED: set when the look-back gave up or the output would overflow
+    unsigned long long capacity;  // FUSED: elements available in `out`
+    int T, n_queries;
+    int wpt;       // bitmap words per thread (power of two); a pass covers DD_THREADS*wpt*32 rows
+    int n_chunks;  // passes over the row range (FUSED: 1)
+    int spin_limit;  // FUSED: polls of an unpublished predecessor before giving up
+    unsigned long long* ticks;  // optional [n_queries][8] phase timers (wall clock ticks of thread 0), or null
+};
+
+// Chained scan over the queries' counts.  A published word holds a 2-bit tag and a value:
+// tag 1 = this query's count, tag 2 = sum of the counts of queries 0..q.  The caller (one
+// full wavefront) has published its count; here it sums its predecessors' counts back to
+// the nearest running sum, then publishes its own running sum.  Workgroups start in index order, so the
+// lowest unfinished query never waits on one that has not started; the poll count is
+// bounded all the same and a give-up is reported through `err`.
+constexpr unsigned long long TAG_COUNT = 1ull << 62, TAG_SUM = 2ull << 62, TAG_VALUE = TAG_COUNT - 1ull;
+
+__device__ __forceinline__ unsigned long long look_back(unsigned long long* state, int q, unsigned long long total,
+                                                        int spin_limit, unsigned int* err) {
+    const int lane = threadIdx.x & 63;
+    unsigned long long excl = 0;
+    int hi = q;  // queries [0, hi) are not accounted for yet
+    int polls = 0;
+    bool gave_up = false;
+    while (hi > 0) {
+        const int idx = hi - 1 - lane;  // lane 0 looks at the nearest predecessor
+        const unsigned long long v =
+            idx >= 0 ? __hip_atomic_load(&state[idx], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : TAG_SUM;
+        const unsigned tag = static_cast<unsigned>(v >> 62);
+        const unsigned long long has_sum = __ballot(tag == 2u), unpublished = __ballot(tag == 0u);
+        const int f = has_sum ? __ffsll(static_cast<long long>(has_sum)) - 1 : 64;  // nearest running sum
+        const unsigned long long needed = f >= 63 ? ~0ull : ((2ull << f) - 1ull);  // lanes 0..f
+        if (unpublished & needed) {
+            if (++polls > spin_limit) { gave_up = true; break; }
+            __builtin_amdgcn_s_sleep(2);
+            continue;
+        }
+        excl += wave_sum((lane <= f) ? (v & TAG_VALUE) : 0ull);
+        if (f < 64) break;
+        hi -= 64;
+    }
+    if (gave_up) {
+        if (lane == 0) atomicOr(err, 1u);
+        excl = 0;
+    }
+    if (lane == 0) __hip_atomic_store(&state[q], TAG_SUM | (excl + total), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    return excl;
+}
+
+// The `ew` (8, 4 or 1) consecutive bitmap words a lane owns in one read-out step.
+__device__ __forceinline__ void load_step_words(const uint32_t* p, int ew, uint32_t (&words)[8]) {
+    if (ew == 8) {
+        const uint4 v0 = *reinterpret_cast<const uint4*>(p), v1 = *reinterpret_cast<const uint4*>(p + 4);
+        words[0] = v0.x; words[1] = v0.y; words[2] = v0.z; words[3] = v0.w;
+        words[4] = v1.x; words[5] = v1.y; words[6] = v1.z; words[7] = v1.w;
+    } else if (ew == 4) {
+        const uint4 v0 = *reinterpret_cast<const uint4*>(p);
+        words[0] = v0.x; words[1] = v0.y; words[2] = v0.z; words[3] = v0.w;
+        words[4] = words[5] = words[6] = words[7] = 0u;
+    } else {
+        words[0] = p[0];
+        words[1] = words[2] = words[3] = words[4] = words[5] = words[6] = words[7] = 0u;
+    }
+}
+
+// One workgroup per query.  COUNT marks the rows of the query's spans in the LDS bitmap and
+// counts the bits it set first.  EMIT and FUSED mark them and read the bitmap out in row
+// order: the list is ascending and duplicate-free without sorting, and raw candidates
+// never reach memory.
+template <int MODE>
 __global__ __launch_bounds__(DD_THREADS) void dedup_kernel(DedupArgs a) {
     extern __shared__ uint32_t lds[];
     const int T = a.T, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int chunk_words = DD_THREADS * a.wpt;                  // multiple of 1024
-    const int n_groups = chunk_words >> 3;                       // rank groups of 8 words
     uint32_t* bm = lds;                                          // [chunk_words]
-    uint32_t* gpref = bm + chunk_words;                          // [n_groups] (EMIT)
-    int* s_start = reinterpret_cast<int*>(gpref + (EMIT ? n_groups : 0));  // [T]
-    uint32_t* s_pref = reinterpret_cast<uint32_t*>(s_start + T); // [T+1]
-    uint32_t* lut = s_pref + T + 1;                              // [DD_THREADS]
-    uint32_t* scratch = lut + DD_THREADS;                        // [17]
+    unsigned long long* sh_base = reinterpret_cast<unsigned long long*>(bm + chunk_words);  // [1]
+    int2* tab = reinterpret_cast<int2*>(sh_base + 1);            // [DD_THREADS]
+    int* s_start = reinterpret_cast<int*>(tab + DD_THREADS);     // [T]
+    int* s_len = s_start + T;                                    // [T]
+    uint32_t* s_ppref = reinterpret_cast<uint32_t*>(s_len + T);  // [T+1]
+    uint32_t* scratch = s_ppref + T + 1;                         // [17]
     uint32_t* wtot = scratch + 17;                               // [NWAVES + 1]
 
 #define DD_TICK(k)                                                                      \
     if (a.ticks && tid == 0) {                                                          \
         const unsigned long long now_ = wall_clock64();                                 \
-        atomicAdd(&a.ticks[k], now_ - tick_);                                           \
+        a.ticks[static_cast<size_t>(blockIdx.x) * 8 + (k)] += now_ - tick_;             \
         tick_ = now_;                                                                   \
     }
     unsigned long long tick_ = a.ticks ? wall_clock64() : 0ull;
 
     const int q = blockIdx.x;
-    uint32_t total;
+    uint32_t n_pieces;
     {
-        int s = 0, len = 0;
-        if (tid < T) {
-            const int b = a.matched[static_cast<size_t>(q) * T + tid];
-            if (b >= 0) {  // span of the matched bucket (count_candidates_kernel, query.cuh:114-132)
-                s = a.bucket_candidate_offsets[b];
-                len = a.bucket_candidate_offsets[b + 1] - s;
-            }
-        }
-        // the first pass's bitmap is cleared while those loads are in flight
+        int2 sp = make_int2(0, 0);
+        if (tid < T) sp = a.spans[static_cast<size_t>(q) * T + tid];
+        // the first pass's bitmap is cleared while that load is in flight
         uint4* bm4 = reinterpret_cast<uint4*>(bm);
         for (int i = tid; i < chunk_words / 4; i += DD_THREADS) bm4[i] = make_uint4(0u, 0u, 0u, 0u);
-        if (tid < T) s_start[tid] = s;
-        const uint32_t ex = block_exclusive_sum(static_cast<uint32_t>(len), scratch, &total);
-        if (tid < T) s_pref[tid] = ex;
-        if (tid == 0) s_pref[T] = total;
+        if (tid < T) {
+            s_start[tid] = sp.x;
+            s_len[tid] = sp.y;
+        }
+        const uint32_t ex = block_exclusive_sum((static_cast<uint32_t>(sp.y) + 63u) >> 6, scratch, &n_pieces);
+        if (tid < T) s_ppref[tid] = ex;
+        if (tid == 0) s_ppref[T] = n_pieces;
     }
     uint64_t running = 0;  // unique candidates found in earlier passes
-    const uint64_t out_base = EMIT ? a.offsets[q] : 0;
+    const uint64_t out_base = MODE == DD_EMIT ? a.offsets[q] : 0;
     const uint32_t chunk_rows = static_cast<uint32_t>(chunk_words) * 32u;
 
     for (int chunk = 0; chunk < a.n_chunks; ++chunk) {
@@ -162,22 +268,22 @@ __global__ __launch_bounds__(DD_THREADS) void dedup_kernel(DedupArgs a) {
         if (tid <= NWAVES) wtot[tid] = 0;
         __syncthreads();
         DD_TICK(0)  // setup + clear
-        // Mark the rows of this pass (collect_candidates_kernel, query.cuh:199-237, but into the
-        // bitmap instead of memory).  Rows outside [lo, lo + chunk_rows) belong to another pass.
+        // Mark the rows of this pass (collect_candidates_kernel, core/query.cuh:199-237, but into
+        // the bitmap instead of memory).  Rows outside [lo, lo + chunk_rows) belong to another pass.
         uint32_t fresh = 0;  // COUNT: bits this thread set first
-        walk_candidates(a.cand, s_start, s_pref, T, total, lut, [&](int row) {
+        walk_candidates(a.cand, s_start, s_len, s_ppref, T, n_pieces, tab, [&](int row) {
             const uint32_t bit = static_cast<uint32_t>(row) - lo;
             if (bit < chunk_rows) {
                 const uint32_t m = 1u << (bit & 31u);
-                if (EMIT) {
-                    atomicOr(&bm[bit >> 5], m);
-                } else {
+                if (MODE == DD_COUNT) {
                     fresh += (atomicOr(&bm[bit >> 5], m) & m) == 0u;
+                } else {
+                    atomicOr(&bm[bit >> 5], m);
                 }
             }
         });
         DD_TICK(1)  // gather
-        if (!EMIT) {
+        if (MODE == DD_COUNT) {
             // a row is counted by whichever lane set its bit first
             fresh = wave_sum(fresh);
             if (lane == 0 && fresh) atomicAdd(&wtot[NWAVES], fresh);
@@ -187,28 +293,27 @@ __global__ __launch_bounds__(DD_THREADS) void dedup_kernel(DedupArgs a) {
             DD_TICK(2)
             continue;
         }
-        // Rank table.  Wavefront w owns the consecutive groups [w*gpw, (w+1)*gpw); in step j its
-        // lanes take 64 consecutive groups, so group order = (wave, step, lane).
-        const int gpw = n_groups / NWAVES;           // >= 8
-        const int steps = (gpw + 63) >> 6;           // <= 4
-        uint32_t cnt[4], incl[4];
+        // Ordered read-out.  Wavefront w owns the consecutive words [w*wpw, (w+1)*wpw); in a step
+        // every lane takes EW consecutive words, so row order = (wave, step, lane, word, bit).
+        const int wpw = chunk_words / NWAVES;                 // words per wavefront, >= 64
+        const int ew = wpw >= 512 ? 8 : (wpw >= 256 ? 4 : 1);   // words per lane and step
+        const int steps = wpw / (64 * ew);
+        uint32_t* wbm = bm + wave * wpw;
         uint32_t wave_total = 0;
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            cnt[j] = 0;
-            incl[j] = 0;
-            if (j < steps) {
-                const int gl = j * 64 + lane;
-                if (gl < gpw) {
-                    const uint4* p = reinterpret_cast<const uint4*>(&bm[(wave * gpw + gl) << 3]);
-                    const uint4 v0 = p[0], v1 = p[1];
-                    cnt[j] = __popc(v0.x) + __popc(v0.y) + __popc(v0.z) + __popc(v0.w) + __popc(v1.x) +
-                             __popc(v1.y) + __popc(v1.z) + __popc(v1.w);
-                }
-                incl[j] = wave_inclusive_sum_dpp(cnt[j]) + wave_total;
-                wave_total = __shfl(incl[j], 63, 64);
+        for (int j = 0; j < steps; ++j) {
+            const uint32_t* p = wbm + (j * 64 + lane) * ew;
+            if (ew == 8) {
+                const uint4 v0 = *reinterpret_cast<const uint4*>(p), v1 = *reinterpret_cast<const uint4*>(p + 4);
+                wave_total += __popc(v0.x) + __popc(v0.y) + __popc(v0.z) + __popc(v0.w) + __popc(v1.x) +
+                              __popc(v1.y) + __popc(v1.z) + __popc(v1.w);
+            } else if (ew == 4) {
+                const uint4 v0 = *reinterpret_cast<const uint4*>(p);
+                wave_total += __popc(v0.x) + __popc(v0.y) + __popc(v0.z) + __popc(v0.w);
+            } else {
+                wave_total += __popc(p[0]);
             }
         }
+        wave_total = wave_sum(wave_total);
         if (lane == 0) wtot[wave] = wave_total;
         __syncthreads();
         uint32_t wave_base = 0, chunk_total = 0;
@@ -218,134 +323,291 @@ __global__ __launch_bounds__(DD_THREADS) void dedup_kernel(DedupArgs a) {
             wave_base += (w < wave) ? v : 0u;
             chunk_total += v;
         }
+        // FUSED: the first wavefront publishes the count before anything else, so that later
+        // queries can go on, and looks back only after lining up its own rows.
+        if (MODE == DD_FUSED && wave == 0 && lane == 0)
+            __hip_atomic_store(&a.state[q], TAG_COUNT | static_cast<unsigned long long>(chunk_total), __ATOMIC_RELAXED,
+                               __HIP_MEMORY_SCOPE_AGENT);
+        // Line-up.  A step's words go to registers, which frees its part of the bitmap: the rows are
+        // written there in list order, ready for full-width wavefront stores.  No step needs the
+        // position of the query's list for this.  A dense step (more rows than slots) is left alone.
+        const uint32_t region = 64u * ew;  // words (= list slots) a step covers
+        uint32_t st_total[4] = {0u, 0u, 0u, 0u};  // steps <= 4 for every geometry
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-            const int gl = j * 64 + lane;
-            if (j < steps && gl < gpw) gpref[wave * gpw + gl] = wave_base + incl[j] - cnt[j];
-        }
-        __syncthreads();
-        DD_TICK(2)  // rank table
-        int32_t* dst = a.out + out_base + running;
-        walk_candidates(a.cand, s_start, s_pref, T, total, lut, [&](int row) {
-            const uint32_t bit = static_cast<uint32_t>(row) - lo;
-            if (bit < chunk_rows) {
-                const uint32_t w = bit >> 5, g = w >> 3, k = w & 7u;
-                const uint4* p = reinterpret_cast<const uint4*>(&bm[g << 3]);
-                const uint4 v0 = p[0], v1 = p[1];
-                const uint32_t words[8] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w};
-                uint32_t pos = gpref[g];
-                uint32_t cur = 0;
+            if (j >= steps) break;
+            const int w0 = (j * 64 + lane) * ew;
+            uint32_t* sreg = wbm + j * region;
+            uint32_t words[8];
+            load_step_words(wbm + w0, ew, words);
+            uint32_t c = 0;
 #pragma unroll
-                for (uint32_t i = 0; i < 8; ++i) {
-                    pos += (i < k) ? __popc(words[i]) : 0;
-                    cur = (i == k) ? words[i] : cur;
+            for (int k = 0; k < 8; ++k) c += __popc(words[k]);
+            const uint32_t incl = wave_inclusive_sum_dpp(c);
+            st_total[j] = __shfl(incl, 63, 64);
+            if (st_total[j] <= region) {
+                uint32_t pos = incl - c;
+                const uint32_t row_base = lo + (static_cast<uint32_t>(wave * wpw + w0) << 5);
+#pragma unroll
+                for (int k = 0; k < 8; ++k) {
+                    uint32_t bits = words[k];
+                    const uint32_t r0 = row_base + (k << 5);
+                    while (bits) {
+                        sreg[pos++] = r0 + (__ffs(static_cast<int>(bits)) - 1);
+                        bits &= bits - 1u;
+                    }
                 }
-                pos += __popc(cur & ((1u << (bit & 31u)) - 1u));
-                dst[pos] = row;
             }
-        });
+        }
+        uint64_t base = out_base + running;
+        bool store = true;
+        if (MODE == DD_FUSED) {
+            if (wave == 0) {
+                const unsigned long long excl = look_back(a.state, q, chunk_total, a.spin_limit, a.err);
+                if (lane == 0) {
+                    unsigned long long b = excl;
+                    if (excl + chunk_total > a.capacity) {  // cannot happen with capacity = raw candidates
+                        atomicOr(a.err, 2u);
+                        b = ~0ull;
+                    }
+                    *sh_base = b;
+                    a.counts[q] = chunk_total;
+                    a.offsets[q] = excl;
+                    if (q == a.n_queries - 1) a.offsets[a.n_queries] = excl + chunk_total;
+                }
+            }
+            __syncthreads();
+            base = *sh_base;
+            store = base != ~0ull;
+        }
+        DD_TICK(2)  // count, line-up (+ look-back)
+        if (store) {
+            int32_t* dst = a.out + base + wave_base;
+            __builtin_amdgcn_wave_barrier();  // LDS accesses of one wavefront complete in order
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                if (j >= steps) break;
+                const uint32_t* sreg = wbm + j * region;
+                if (st_total[j] <= region) {
+                    for (uint32_t i = lane; i < st_total[j]; i += 64) dst[i] = static_cast<int32_t>(sreg[i]);
+                } else {  // dense step: every lane stores the rows of its own words
+                    const int w0 = (j * 64 + lane) * ew;
+                    uint32_t words[8];
+                    load_step_words(wbm + w0, ew, words);
+                    uint32_t c = 0;
+#pragma unroll
+                    for (int k = 0; k < 8; ++k) c += __popc(words[k]);
+                    uint32_t pos = wave_inclusive_sum_dpp(c) - c;
+                    const uint32_t row_base = lo + (static_cast<uint32_t>(wave * wpw + w0) << 5);
+#pragma unroll
+                    for (int k = 0; k < 8; ++k) {
+                        uint32_t bits = words[k];
+                        const uint32_t r0 = row_base + (k << 5);
+                        while (bits) {
+                            dst[pos++] = static_cast<int32_t>(r0 + (__ffs(static_cast<int>(bits)) - 1));
+                            bits &= bits - 1u;
+                        }
+                    }
+                }
+                dst += st_total[j];
+            }
+        }
         running += chunk_total;
-        DD_TICK(3)  // rank + store
+        __syncthreads();  // bitmap and wtot are rewritten by the next pass
+        DD_TICK(3)  // ordered store
     }
-    if (!EMIT && tid == 0) a.counts[q] = running;
+    if (MODE == DD_COUNT && tid == 0) a.counts[q] = running;
 #undef DD_TICK
 }
 
 }  // namespace
 
 culsh_status launch_find_matching_buckets(culsh_ctx* ctx, const uint32_t* q_keys, int n_queries,
-                                          const culsh_index* index, int32_t* matched) {
+                                          const culsh_index* index, int32_t* matched, void* spans,
+                                          unsigned long long* raw_total) {
     const size_t pairs = static_cast<size_t>(n_queries) * index->n_hash_tables;
     CULSH_REQUIRE(pairs / 256 < (1ull << 31), CULSH_ERR_LIMIT, "too many (query, table) pairs");
+    CULSH_REQUIRE(!spans || raw_total, CULSH_ERR_INTERNAL, "spans need a raw candidate counter");
     CULSH_LAUNCH(ctx, lookup_kernel, dim3(div_up(pairs, 256)), dim3(256), 0, ctx->stream, q_keys,
-                       index->bucket_keys, index->table_bucket_offsets, n_queries, index->n_hash_tables,
-                       index->key_w, matched);
+                 index->bucket_keys, index->table_bucket_offsets, index->bucket_candidate_offsets, n_queries,
+                 index->n_hash_tables, index->key_w, matched, static_cast<int2*>(spans), raw_total);
     CULSH_LAUNCH_CHECK();
     return CULSH_OK;
 }
 
-culsh_status query_from_matched(culsh_ctx* ctx, const int32_t* matched, int n_queries,
-                                const culsh_index* index, culsh_candidates* out) {
+namespace {
+
+int env_int(const char* name, int dflt) {
+    const char* v = std::getenv(name);
+    return (v && *v) ? std::atoi(v) : dflt;
+}
+
+// `raw_total` (device) holds the number of raw candidates = sum of all span lengths.
+culsh_status query_from_spans(culsh_ctx* ctx, const int2* spans, const unsigned long long* raw_total, int n_queries,
+                              const culsh_index* index, culsh_candidates* out) {
     const int T = index->n_hash_tables;
-    CULSH_REQUIRE(T <= DD_THREADS, CULSH_ERR_LIMIT, "query: n_hash_tables > 1024 is not supported");
-    CULSH_REQUIRE(n_queries > 0, CULSH_ERR_INVALID, "query: n_queries must be positive");
     // rows addressed by the index: candidates are row ids < n = n_total_candidates / T
     const int n = index->n_total_candidates / T;
-    CULSH_REQUIRE(n > 0, CULSH_ERR_INVALID, "query: empty index");
 
-    // Geometry of a pass: DD_THREADS * wpt bitmap words (wpt a power of two); the emit launch
-    // adds one rank word per 4 bitmap words.  Smaller bitmaps mean more passes over the row
-    // range but let more workgroups share a CU; CULSH_DEDUP_WPT overrides the default cap.
-    auto env_int = [](const char* name, int dflt) {
-        const char* v = std::getenv(name);
-        return (v && *v) ? std::atoi(v) : dflt;
-    };
-    const size_t fixed = (static_cast<size_t>(2 * T) + 1 + DD_THREADS + 17 + (DD_THREADS / 64 + 1) + 8) * sizeof(uint32_t);
-    auto lds_need = [&](int w, bool emit) {
-        const size_t cw = static_cast<size_t>(DD_THREADS) * w;
-        return (cw + (emit ? cw / 8 : 0)) * 4 + fixed;
-    };
+    // Geometry of a pass: DD_THREADS * wpt bitmap words, wpt a power of two.  Debug knobs:
+    // CULSH_DEDUP_WPT lowers the cap on wpt (more passes), CULSH_DEDUP_TWO_PASS=1 forces the
+    // count / scan / emit path, CULSH_DEDUP_TRACE=1 prints phase timers.
+    const size_t fixed = (2 + static_cast<size_t>(3 * T) + 1 + 2 * DD_THREADS + 17 + (NWAVES + 1) + 8) * sizeof(uint32_t);
+    auto lds_need = [&](int w) { return static_cast<size_t>(DD_THREADS) * w * 4 + fixed; };
     int wpt_max = 1;
     const int wpt_limit = std::max(1, std::min(32, env_int("CULSH_DEDUP_WPT", 32)));
-    while (wpt_max * 2 <= wpt_limit && lds_need(wpt_max * 2, true) <= static_cast<size_t>(ctx->lds_max)) wpt_max *= 2;
+    while (wpt_max * 2 <= wpt_limit && lds_need(wpt_max * 2) <= static_cast<size_t>(ctx->lds_max)) wpt_max *= 2;
     int wpt = 1;
     while (wpt < wpt_max && static_cast<long long>(DD_THREADS) * wpt * 32 < n) wpt *= 2;
-    DedupArgs a;
-    a.matched = matched;
-    a.bucket_candidate_offsets = index->bucket_candidate_offsets;
-    a.cand = index->all_candidate_indices;
-    a.T = T;
-    a.n = n;
-    a.wpt = wpt;
-    a.ticks = nullptr;
+    const long long chunk_rows = static_cast<long long>(DD_THREADS) * wpt * 32;
+    const int n_chunks = static_cast<int>((n + chunk_rows - 1) / chunk_rows);
+    const size_t lds_bytes = lds_need(wpt);
+    CULSH_REQUIRE(lds_bytes <= static_cast<size_t>(ctx->lds_max), CULSH_ERR_INTERNAL, "LDS budget exceeded");
     const bool trace = env_int("CULSH_DEDUP_TRACE", 0) != 0;
     unsigned long long* ticks_dev = nullptr;
     if (trace) {
-        CULSH_TRY(arena_alloc_t(ctx, 16, &ticks_dev));
-        CULSH_HIP(hipMemsetAsync(ticks_dev, 0, 16 * sizeof(unsigned long long), ctx->stream));
+        CULSH_TRY(arena_alloc_t(ctx, static_cast<size_t>(n_queries) * 8, &ticks_dev));
+        CULSH_HIP(hipMemsetAsync(ticks_dev, 0, static_cast<size_t>(n_queries) * 8 * sizeof(unsigned long long), ctx->stream));
     }
-    const long long chunk_rows = static_cast<long long>(DD_THREADS) * wpt * 32;
-    a.n_chunks = static_cast<int>((n + chunk_rows - 1) / chunk_rows);
-    const size_t lds_count = lds_need(wpt, false), lds_emit = lds_need(wpt, true);
-    CULSH_REQUIRE(lds_emit <= static_cast<size_t>(ctx->lds_max), CULSH_ERR_INTERNAL, "LDS budget exceeded");
-    CULSH_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(dedup_kernel<false>),
-                                  hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_count)));
-    CULSH_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(dedup_kernel<true>),
-                                  hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_emit)));
 
     out->n_queries = n_queries;
     CULSH_HIP(hipMalloc(&out->query_candidate_counts, static_cast<size_t>(n_queries) * sizeof(uint64_t)));
     CULSH_HIP(hipMalloc(&out->query_candidate_offsets, (static_cast<size_t>(n_queries) + 1) * sizeof(uint64_t)));
 
-    a.counts = out->query_candidate_counts;
-    a.offsets = nullptr;
+    DedupArgs a;
+    a.spans = spans;
+    a.cand = index->all_candidate_indices;
     a.out = nullptr;
-    a.ticks = ticks_dev;
-    CULSH_LAUNCH(ctx, dedup_kernel<false>, dim3(n_queries), dim3(DD_THREADS), lds_count, ctx->stream, a);
-    CULSH_LAUNCH_CHECK();
-    CULSH_TRY(exclusive_scan_u64(ctx, out->query_candidate_counts, out->query_candidate_offsets, n_queries));
-    uint64_t U = 0;
-    CULSH_TRY(read_back_u64(ctx, out->query_candidate_offsets + n_queries, 1, &U));  // the one host sync
-    out->n_total_candidates = U;
-    if (U == 0) {  // query.cuh:358-365: counts/offsets stay, indices stay null
-        out->query_candidate_indices = nullptr;
-        return CULSH_OK;
-    }
-    CULSH_HIP(hipMalloc(&out->query_candidate_indices, U * sizeof(int32_t)));
+    a.counts = out->query_candidate_counts;
     a.offsets = out->query_candidate_offsets;
-    a.out = out->query_candidate_indices;
-    a.ticks = ticks_dev ? ticks_dev + 8 : nullptr;
-    CULSH_LAUNCH(ctx, dedup_kernel<true>, dim3(n_queries), dim3(DD_THREADS), lds_emit, ctx->stream, a);
-    CULSH_LAUNCH_CHECK();
+    a.state = nullptr;
+    a.err = nullptr;
+    a.capacity = 0;
+    a.T = T;
+    a.n_queries = n_queries;
+    a.wpt = wpt;
+    a.n_chunks = n_chunks;
+    a.spin_limit = 1 << 16;
+    a.ticks = ticks_dev;
+
+    bool fused = n_chunks == 1 && env_int("CULSH_DEDUP_TWO_PASS", 0) == 0;
+    uint64_t U = 0;
+    if (fused) {
+        uint64_t R = 0;
+        CULSH_TRY(read_back_u64(ctx, reinterpret_cast<const uint64_t*>(raw_total), 1, &R));  // host sync 1 of 2
+        if (R == 0) {  // no query matched any bucket (query.cuh:358-365: counts/offsets stay, indices stay null)
+            CULSH_HIP(hipMemsetAsync(out->query_candidate_counts, 0, static_cast<size_t>(n_queries) * sizeof(uint64_t), ctx->stream));
+            CULSH_HIP(hipMemsetAsync(out->query_candidate_offsets, 0, (static_cast<size_t>(n_queries) + 1) * sizeof(uint64_t), ctx->stream));
+            out->n_total_candidates = 0;
+            out->query_candidate_indices = nullptr;
+            return CULSH_OK;
+        }
+        // a query holds at most n distinct rows, which bounds the output when buckets overlap heavily
+        const uint64_t cap = std::min<uint64_t>(R, static_cast<uint64_t>(n_queries) * static_cast<uint64_t>(n));
+        unsigned int* err = nullptr;
+        CULSH_TRY(arena_alloc_t(ctx, static_cast<size_t>(n_queries), &a.state));
+        CULSH_TRY(arena_alloc_t(ctx, 1, &err));
+        CULSH_HIP(hipMemsetAsync(a.state, 0, static_cast<size_t>(n_queries) * sizeof(unsigned long long), ctx->stream));
+        CULSH_HIP(hipMemsetAsync(err, 0, sizeof(unsigned int), ctx->stream));
+        CULSH_HIP(hipMalloc(&out->query_candidate_indices, cap * sizeof(int32_t)));
+        a.out = out->query_candidate_indices;
+        a.err = err;
+        a.capacity = cap;
+        CULSH_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(dedup_kernel<DD_FUSED>),
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes)));
+        CULSH_LAUNCH(ctx, dedup_kernel<DD_FUSED>, dim3(n_queries), dim3(DD_THREADS), lds_bytes, ctx->stream, a);
+        CULSH_LAUNCH_CHECK();
+        CULSH_HIP(hipMemcpyAsync(&ctx->pinned[0], out->query_candidate_offsets + n_queries, sizeof(uint64_t),
+                                 hipMemcpyDeviceToHost, ctx->stream));
+        CULSH_HIP(hipMemcpyAsync(&ctx->pinned[1], err, sizeof(unsigned int), hipMemcpyDeviceToHost, ctx->stream));
+        CULSH_HIP(hipStreamSynchronize(ctx->stream));  // host sync 2 of 2
+        U = ctx->pinned[0];
+        const unsigned int e = static_cast<unsigned int>(ctx->pinned[1] & 0xffffffffu);
+        if (e != 0) {  // never seen; the two-launch path below needs no cooperation between workgroups
+            (void)hipFree(out->query_candidate_indices);
+            out->query_candidate_indices = nullptr;
+            fused = false;
+        } else if (U == 0) {
+            (void)hipFree(out->query_candidate_indices);
+            out->query_candidate_indices = nullptr;
+        } else if (U <= cap / 2 && (cap - U) * sizeof(int32_t) > (size_t(16) << 20)) {
+            // heavy overlap between tables: hand out an exact-size array instead of the bound
+            int32_t* exact = nullptr;
+            CULSH_HIP(hipMalloc(&exact, U * sizeof(int32_t)));
+            CULSH_HIP(hipMemcpyAsync(exact, out->query_candidate_indices, U * sizeof(int32_t), hipMemcpyDeviceToDevice, ctx->stream));
+            CULSH_HIP(hipStreamSynchronize(ctx->stream));
+            (void)hipFree(out->query_candidate_indices);
+            out->query_candidate_indices = exact;
+        }
+    }
+    if (!fused) {
+        CULSH_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(dedup_kernel<DD_COUNT>),
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes)));
+        CULSH_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(dedup_kernel<DD_EMIT>),
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes)));
+        CULSH_LAUNCH(ctx, dedup_kernel<DD_COUNT>, dim3(n_queries), dim3(DD_THREADS), lds_bytes, ctx->stream, a);
+        CULSH_LAUNCH_CHECK();
+        CULSH_TRY(exclusive_scan_u64(ctx, out->query_candidate_counts, out->query_candidate_offsets, n_queries));
+        CULSH_TRY(read_back_u64(ctx, out->query_candidate_offsets + n_queries, 1, &U));
+        if (U != 0) {
+            CULSH_HIP(hipMalloc(&out->query_candidate_indices, U * sizeof(int32_t)));
+            a.out = out->query_candidate_indices;
+            a.ticks = nullptr;
+            CULSH_LAUNCH(ctx, dedup_kernel<DD_EMIT>, dim3(n_queries), dim3(DD_THREADS), lds_bytes, ctx->stream, a);
+            CULSH_LAUNCH_CHECK();
+        } else {
+            out->query_candidate_indices = nullptr;
+        }
+    }
+    out->n_total_candidates = U;
     if (trace) {  // 100 MHz wall clock ticks of thread 0, summed over workgroups
-        uint64_t tk[16];
-        CULSH_TRY(read_back_u64(ctx, reinterpret_cast<const uint64_t*>(ticks_dev), 16, tk));
-        fprintf(stderr, "[dedup trace] wpt=%d chunks=%d | count: setup %llu gather %llu reduce %llu | emit: setup %llu gather %llu ranktable %llu rank+store %llu (ticks)\n",
-                wpt, a.n_chunks, (unsigned long long)tk[0], (unsigned long long)tk[1], (unsigned long long)tk[2],
-                (unsigned long long)tk[8], (unsigned long long)tk[9], (unsigned long long)tk[10],
-                (unsigned long long)tk[11]);
+        std::vector<uint64_t> all(static_cast<size_t>(n_queries) * 8);
+        CULSH_HIP(hipStreamSynchronize(ctx->stream));
+        CULSH_HIP(hipMemcpy(all.data(), ticks_dev, all.size() * sizeof(uint64_t), hipMemcpyDeviceToHost));
+        uint64_t tk[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+        for (size_t i = 0; i < all.size(); ++i) tk[i & 7] += all[i];
+        fprintf(stderr, "[dedup trace] wpt=%d chunks=%d fused=%d | setup %llu gather %llu count %llu store %llu (ticks)\n",
+                wpt, n_chunks, int(fused), (unsigned long long)tk[0], (unsigned long long)tk[1],
+                (unsigned long long)tk[2], (unsigned long long)tk[3]);
     }
     return CULSH_OK;
+}
+
+culsh_status check_query_args(int n_queries, const culsh_index* index) {
+    CULSH_REQUIRE(index->n_hash_tables <= DD_THREADS, CULSH_ERR_LIMIT, "query: n_hash_tables > 1024 is not supported");
+    CULSH_REQUIRE(n_queries > 0, CULSH_ERR_INVALID, "query: n_queries must be positive");
+    CULSH_REQUIRE(index->n_total_candidates / index->n_hash_tables > 0, CULSH_ERR_INVALID, "query: empty index");
+    return CULSH_OK;
+}
+
+}  // namespace
+
+culsh_status query_from_matched(culsh_ctx* ctx, const int32_t* matched, int n_queries,
+                                const culsh_index* index, culsh_candidates* out) {
+    CULSH_TRY(check_query_args(n_queries, index));
+    const size_t pairs = static_cast<size_t>(n_queries) * index->n_hash_tables;
+    CULSH_REQUIRE(pairs / 256 < (1ull << 31), CULSH_ERR_LIMIT, "too many (query, table) pairs");
+    int2* spans = nullptr;
+    unsigned long long* raw_total = nullptr;
+    CULSH_TRY(arena_alloc_t(ctx, pairs, &spans));
+    CULSH_TRY(arena_alloc_t(ctx, 1, &raw_total));
+    CULSH_HIP(hipMemsetAsync(raw_total, 0, sizeof(unsigned long long), ctx->stream));
+    CULSH_LAUNCH(ctx, span_kernel, dim3(div_up(pairs, 256)), dim3(256), 0, ctx->stream, matched,
+                 index->bucket_candidate_offsets, pairs, spans, raw_total);
+    CULSH_LAUNCH_CHECK();
+    return query_from_spans(ctx, spans, raw_total, n_queries, index, out);
+}
+
+culsh_status query_from_keys(culsh_ctx* ctx, const uint32_t* q_keys, int n_queries, const culsh_index* index,
+                             culsh_candidates* out) {
+    CULSH_TRY(check_query_args(n_queries, index));
+    int2* spans = nullptr;
+    unsigned long long* raw_total = nullptr;
+    CULSH_TRY(arena_alloc_t(ctx, static_cast<size_t>(n_queries) * index->n_hash_tables, &spans));
+    CULSH_TRY(arena_alloc_t(ctx, 1, &raw_total));
+    CULSH_HIP(hipMemsetAsync(raw_total, 0, sizeof(unsigned long long), ctx->stream));
+    CULSH_TRY(launch_find_matching_buckets(ctx, q_keys, n_queries, index, nullptr, spans, raw_total));
+    return query_from_spans(ctx, spans, raw_total, n_queries, index, out);
 }
 
 }  // namespace culsh_amd

@@ -233,6 +233,39 @@ def test_core_query_wide_row_range(ctx, c_oracle, n):
     ctx.free_index(ih)
 
 
+def test_core_query_two_launch_path(ctx, monkeypatch):
+    """The count / scan / emit path (taken for row ranges beyond one bitmap pass) on a small case."""
+    _announce("two_launch_path")
+    monkeypatch.setenv("CULSH_DEDUP_TWO_PASS", "1")
+    rng = np.random.default_rng(91)
+    T, n, nq, H = 5, 4000, 150, 2
+    sig = random_sigs(rng, T, n, H, "rplsh")
+    qsig = random_sigs(rng, T, nq, H, "rplsh")
+    ih, _ = ctx.core_fit_index(sig, H)
+    from abi import assert_candidates_match
+
+    assert_candidates_match(ctx.core_query_index(qsig, ih), o.query_index(qsig, o.fit_index(sig, H)))
+    ctx.free_index(ih)
+
+
+def test_core_query_tables_that_overlap_completely(ctx, c_oracle):
+    """Identical tables: the raw candidates outnumber the distinct ones eightfold, so the result
+    array is cut down from its upper bound to the exact size."""
+    _announce("overlapping_tables")
+    rng = np.random.default_rng(17)
+    T, n, nq, H = 8, 20000, 64, 1
+    one = rng.integers(0, 2, size=(1, n, H), dtype=np.uint8)
+    sig = np.ascontiguousarray(np.repeat(one, T, axis=0))
+    qsig = np.ascontiguousarray(np.repeat(rng.integers(0, 2, size=(1, nq, H), dtype=np.uint8), T, axis=0))
+    ih, _ = ctx.core_fit_index(sig, H)
+    from abi import assert_candidates_match
+
+    cix = c_oracle.fit_index_c(sig, H)
+    got = ctx.core_query_index(qsig, ih)
+    assert_candidates_match(got, c_oracle.query_index_c(qsig, cix))
+    ctx.free_index(ih)
+
+
 @pytest.mark.parametrize("kind", ["rplsh", "pslsh", "minhash"])
 def test_core_fit_query(ctx, kind):
     """fit_query == fit + query on the same signatures (python/tests/test_rplsh.py:145-174)."""
