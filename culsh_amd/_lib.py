@@ -105,6 +105,7 @@ _SPECIAL = {
     "culsh_last_error": (C.c_char_p, []),
     "culsh_version": (C.c_char_p, []),
     "culsh_ctx_destroy": (None, [_P]),
+    "culsh_memory_trim": (None, []),
     "culsh_ctx_stream": (_P, [_P]),
     "culsh_profile_count": (C.c_int, [_P]),
     "culsh_index_free": (None, [_P]),

@@ -191,15 +191,15 @@ static void gen_minhash(uint64_t seed, size_t count, uint32_t* A, uint32_t* B) {
 // ---------------------------------------------------------------- object helpers
 void free_index_arrays(culsh_index* ix) {
     if (!ix) return;
-    (void)hipFree(ix->all_candidate_indices);
-    (void)hipFree(ix->all_bucket_signatures);
-    (void)hipFree(ix->bucket_candidate_offsets);
-    (void)hipFree(ix->table_bucket_offsets);
-    (void)hipFree(ix->bucket_keys);
-    (void)hipFree(ix->P);
-    (void)hipFree(ix->b);
-    (void)hipFree(ix->A);
-    (void)hipFree(ix->B);
+    dev_free(ix->all_candidate_indices);
+    dev_free(ix->all_bucket_signatures);
+    dev_free(ix->bucket_candidate_offsets);
+    dev_free(ix->table_bucket_offsets);
+    dev_free(ix->bucket_keys);
+    dev_free(ix->P);
+    dev_free(ix->b);
+    dev_free(ix->A);
+    dev_free(ix->B);
     free_ps_codec(ix);
     ix->all_candidate_indices = nullptr;
     ix->all_bucket_signatures = nullptr;
@@ -212,9 +212,9 @@ void free_index_arrays(culsh_index* ix) {
 
 void free_candidates_arrays(culsh_candidates* c) {
     if (!c) return;
-    (void)hipFree(c->query_candidate_indices);
-    (void)hipFree(c->query_candidate_counts);
-    (void)hipFree(c->query_candidate_offsets);
+    dev_free(c->query_candidate_indices);
+    dev_free(c->query_candidate_counts);
+    dev_free(c->query_candidate_offsets);
     c->query_candidate_indices = nullptr;
     c->query_candidate_counts = nullptr;
     c->query_candidate_offsets = nullptr;
@@ -233,7 +233,7 @@ template <typename T>
 static culsh_status upload(const T* host, size_t count, T** dev) {
     *dev = nullptr;
     if (count == 0) return CULSH_OK;  // empty array -> nullptr (array_utils.cuh:34-36)
-    CULSH_HIP(hipMalloc(reinterpret_cast<void**>(dev), count * sizeof(T)));
+    CULSH_HIP(dev_malloc(dev, count * sizeof(T)));
     CULSH_HIP(hipMemcpy(*dev, host, count * sizeof(T), hipMemcpyHostToDevice));
     return CULSH_OK;
 }
@@ -319,9 +319,9 @@ static culsh_status concat_candidates(culsh_ctx* ctx, const std::vector<culsh_ca
     CULSH_REQUIRE(nq < (1ull << 31), CULSH_ERR_LIMIT, "too many queries");
     out->n_queries = static_cast<int>(nq);
     out->n_total_candidates = total;
-    CULSH_HIP(hipMalloc(&out->query_candidate_counts, std::max<size_t>(1, nq) * sizeof(uint64_t)));
-    CULSH_HIP(hipMalloc(&out->query_candidate_offsets, (nq + 1) * sizeof(uint64_t)));
-    if (total) CULSH_HIP(hipMalloc(&out->query_candidate_indices, total * sizeof(int32_t)));
+    CULSH_HIP(dev_malloc(&out->query_candidate_counts, std::max<size_t>(1, nq) * sizeof(uint64_t)));
+    CULSH_HIP(dev_malloc(&out->query_candidate_offsets, (nq + 1) * sizeof(uint64_t)));
+    if (total) CULSH_HIP(dev_malloc(&out->query_candidate_indices, total * sizeof(int32_t)));
     size_t q0 = 0;
     uint64_t c0 = 0;
     CULSH_HIP(hipMemsetAsync(out->query_candidate_offsets, 0, sizeof(uint64_t), ctx->stream));
@@ -613,6 +613,8 @@ culsh_status culsh_ctx_synchronize(culsh_ctx* ctx) {
 }
 
 void* culsh_ctx_stream(culsh_ctx* ctx) { return ctx ? static_cast<void*>(ctx->stream) : nullptr; }
+
+void culsh_memory_trim(void) { culsh_amd::dev_trim(); }
 
 culsh_status culsh_profile_enable(culsh_ctx* ctx, int on) {
     CULSH_REQUIRE(ctx, CULSH_ERR_INVALID, "null argument");
@@ -1019,7 +1021,7 @@ culsh_status culsh_index_load(culsh_ctx* ctx, culsh_kind kind, int is_double, co
         CULSH_TRY(upload(static_cast<const uint32_t*>(param0), TH, &ix->A));
         CULSH_TRY(upload(static_cast<const uint32_t*>(param1), TH, &ix->B));
     }
-    CULSH_HIP(hipMalloc(&ix->bucket_keys, std::max<size_t>(1, static_cast<size_t>(n_total_buckets) * ix->key_w) * 4));
+    CULSH_HIP(dev_malloc(&ix->bucket_keys, std::max<size_t>(1, static_cast<size_t>(n_total_buckets) * ix->key_w) * 4));
     CULSH_TRY(launch_sig_to_keys(ctx, ix->all_bucket_signatures, n_total_buckets, S, enc, ix->key_w, ix->bucket_keys));
     CULSH_TRY(arena_end(ctx));
     *out = ix.release();

@@ -133,6 +133,19 @@ struct culsh_candidates {
 
 namespace culsh_amd {
 
+// ---------------------------------------------------------------- object memory (pool.hip)
+// Device blocks owned by index / candidate objects; freed blocks are cached for reuse.
+hipError_t dev_malloc(void** out, size_t bytes);
+template <typename T>
+inline hipError_t dev_malloc(T** out, size_t bytes) {
+    void* p = nullptr;
+    const hipError_t e = dev_malloc(&p, bytes);
+    *out = static_cast<T*>(p);
+    return e;
+}
+void dev_free(void* ptr);
+void dev_trim();
+
 // ---------------------------------------------------------------- scratch arena
 culsh_status arena_begin(culsh_ctx* ctx);                 // start of an API call
 culsh_status arena_alloc(culsh_ctx* ctx, size_t bytes, void** out);

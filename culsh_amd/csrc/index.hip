@@ -217,10 +217,10 @@ culsh_status build_index_from_sorted(culsh_ctx* ctx, const uint32_t* sorted_keys
     index->sig_nbytes = S;
     index->enc = enc;
     index->key_w = W;
-    CULSH_HIP(hipMalloc(&index->bucket_candidate_offsets, (B_bound + 1) * sizeof(int32_t)));
-    CULSH_HIP(hipMalloc(&index->table_bucket_offsets, (static_cast<size_t>(T) + 1) * sizeof(int32_t)));
-    CULSH_HIP(hipMalloc(&index->bucket_keys, std::max<size_t>(1, B_bound * W) * sizeof(uint32_t)));
-    CULSH_HIP(hipMalloc(&index->all_bucket_signatures, std::max<size_t>(1, B_bound * S)));
+    CULSH_HIP(dev_malloc(&index->bucket_candidate_offsets, (B_bound + 1) * sizeof(int32_t)));
+    CULSH_HIP(dev_malloc(&index->table_bucket_offsets, (static_cast<size_t>(T) + 1) * sizeof(int32_t)));
+    CULSH_HIP(dev_malloc(&index->bucket_keys, std::max<size_t>(1, B_bound * W) * sizeof(uint32_t)));
+    CULSH_HIP(dev_malloc(&index->all_bucket_signatures, std::max<size_t>(1, B_bound * S)));
     CULSH_LAUNCH(ctx, build_index_kernel, dim3(static_cast<unsigned>(tiles)), dim3(IB_THREADS), 0, ctx->stream,
                        sorted_keys, rows_sorted_owned, N, n, T, W, tile_base, total_dev, index->bucket_candidate_offsets,
                        index->bucket_keys, index->table_bucket_offsets, item_to_bucket_opt);
@@ -244,7 +244,7 @@ culsh_status fit_index_from_keys(culsh_ctx* ctx, uint32_t* keys, int n, int T, i
     int32_t* rows_out = nullptr;
     CULSH_TRY(arena_alloc_t(ctx, N * W, &keys_tmp));
     CULSH_TRY(arena_alloc_t(ctx, N, &rows_tmp));
-    CULSH_HIP(hipMalloc(&rows_out, N * sizeof(int32_t)));
+    CULSH_HIP(dev_malloc(&rows_out, N * sizeof(int32_t)));
     index->all_candidate_indices = rows_out;  // owned by the index from here on (freed with it)
     uint32_t* sorted = nullptr;
     uint32_t bits_vary[64];

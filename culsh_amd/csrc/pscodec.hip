@@ -111,10 +111,10 @@ __global__ __launch_bounds__(256) void ps_keys_to_sig_kernel(const uint32_t* __r
 }  // namespace
 
 void free_ps_codec(culsh_index* ix) {
-    (void)hipFree(ix->psc.vmin);
-    (void)hipFree(ix->psc.range);
-    (void)hipFree(ix->psc.fwd);
-    (void)hipFree(ix->psc.inv);
+    dev_free(ix->psc.vmin);
+    dev_free(ix->psc.range);
+    dev_free(ix->psc.fwd);
+    dev_free(ix->psc.inv);
     ix->psc = PsCodec();
 }
 
@@ -162,10 +162,10 @@ culsh_status ps_build_codec(culsh_ctx* ctx, const int32_t* sig, int n, int T, in
     PsCodec& pc = ix->psc;
     pc.bits = bits;
     pc.rmax = static_cast<int>(rmax);
-    CULSH_HIP(hipMalloc(&pc.vmin, TH * sizeof(int32_t)));
-    CULSH_HIP(hipMalloc(&pc.range, TH * sizeof(int32_t)));
-    CULSH_HIP(hipMalloc(&pc.fwd, fwd.size() * sizeof(uint32_t)));
-    CULSH_HIP(hipMalloc(&pc.inv, inv.size() * sizeof(int32_t)));
+    CULSH_HIP(dev_malloc(&pc.vmin, TH * sizeof(int32_t)));
+    CULSH_HIP(dev_malloc(&pc.range, TH * sizeof(int32_t)));
+    CULSH_HIP(dev_malloc(&pc.fwd, fwd.size() * sizeof(uint32_t)));
+    CULSH_HIP(dev_malloc(&pc.inv, inv.size() * sizeof(int32_t)));
     CULSH_HIP(hipMemcpy(pc.vmin, vmin.data(), TH * sizeof(int32_t), hipMemcpyHostToDevice));
     CULSH_HIP(hipMemcpy(pc.range, range.data(), TH * sizeof(int32_t), hipMemcpyHostToDevice));
     CULSH_HIP(hipMemcpy(pc.fwd, fwd.data(), fwd.size() * sizeof(uint32_t), hipMemcpyHostToDevice));

@@ -471,8 +471,8 @@ culsh_status query_from_spans(culsh_ctx* ctx, const int2* spans, const unsigned 
     }
 
     out->n_queries = n_queries;
-    CULSH_HIP(hipMalloc(&out->query_candidate_counts, static_cast<size_t>(n_queries) * sizeof(uint64_t)));
-    CULSH_HIP(hipMalloc(&out->query_candidate_offsets, (static_cast<size_t>(n_queries) + 1) * sizeof(uint64_t)));
+    CULSH_HIP(dev_malloc(&out->query_candidate_counts, static_cast<size_t>(n_queries) * sizeof(uint64_t)));
+    CULSH_HIP(dev_malloc(&out->query_candidate_offsets, (static_cast<size_t>(n_queries) + 1) * sizeof(uint64_t)));
 
     DedupArgs a;
     a.spans = spans;
@@ -509,7 +509,7 @@ culsh_status query_from_spans(culsh_ctx* ctx, const int2* spans, const unsigned 
         CULSH_TRY(arena_alloc_t(ctx, 1, &err));
         CULSH_HIP(hipMemsetAsync(a.state, 0, static_cast<size_t>(n_queries) * sizeof(unsigned long long), ctx->stream));
         CULSH_HIP(hipMemsetAsync(err, 0, sizeof(unsigned int), ctx->stream));
-        CULSH_HIP(hipMalloc(&out->query_candidate_indices, cap * sizeof(int32_t)));
+        CULSH_HIP(dev_malloc(&out->query_candidate_indices, cap * sizeof(int32_t)));
         a.out = out->query_candidate_indices;
         a.err = err;
         a.capacity = cap;
@@ -524,19 +524,19 @@ culsh_status query_from_spans(culsh_ctx* ctx, const int2* spans, const unsigned 
         U = ctx->pinned[0];
         const unsigned int e = static_cast<unsigned int>(ctx->pinned[1] & 0xffffffffu);
         if (e != 0) {  // never seen; the two-launch path below needs no cooperation between workgroups
-            (void)hipFree(out->query_candidate_indices);
+            dev_free(out->query_candidate_indices);
             out->query_candidate_indices = nullptr;
             fused = false;
         } else if (U == 0) {
-            (void)hipFree(out->query_candidate_indices);
+            dev_free(out->query_candidate_indices);
             out->query_candidate_indices = nullptr;
         } else if (U <= cap / 2 && (cap - U) * sizeof(int32_t) > (size_t(16) << 20)) {
             // heavy overlap between tables: hand out an exact-size array instead of the bound
             int32_t* exact = nullptr;
-            CULSH_HIP(hipMalloc(&exact, U * sizeof(int32_t)));
+            CULSH_HIP(dev_malloc(&exact, U * sizeof(int32_t)));
             CULSH_HIP(hipMemcpyAsync(exact, out->query_candidate_indices, U * sizeof(int32_t), hipMemcpyDeviceToDevice, ctx->stream));
             CULSH_HIP(hipStreamSynchronize(ctx->stream));
-            (void)hipFree(out->query_candidate_indices);
+            dev_free(out->query_candidate_indices);
             out->query_candidate_indices = exact;
         }
     }
@@ -550,7 +550,7 @@ culsh_status query_from_spans(culsh_ctx* ctx, const int2* spans, const unsigned 
         CULSH_TRY(exclusive_scan_u64(ctx, out->query_candidate_counts, out->query_candidate_offsets, n_queries));
         CULSH_TRY(read_back_u64(ctx, out->query_candidate_offsets + n_queries, 1, &U));
         if (U != 0) {
-            CULSH_HIP(hipMalloc(&out->query_candidate_indices, U * sizeof(int32_t)));
+            CULSH_HIP(dev_malloc(&out->query_candidate_indices, U * sizeof(int32_t)));
             a.out = out->query_candidate_indices;
             a.ticks = nullptr;
             CULSH_LAUNCH(ctx, dedup_kernel<DD_EMIT>, dim3(n_queries), dim3(DD_THREADS), lds_bytes, ctx->stream, a);

@@ -103,6 +103,13 @@ culsh_status culsh_profile_reset(culsh_ctx* ctx);
 int culsh_profile_count(const culsh_ctx* ctx);
 culsh_status culsh_profile_get(const culsh_ctx* ctx, int i, const char** name, double* total_ms, int64_t* launches);
 
+/* ---- object memory ------------------------------------------------------------------
+ * No counterpart in the reference (it allocates with cudaMalloc per array,
+ * core/index.cuh:42-77, core/candidates.cuh:42-70).  Index and candidate arrays come from
+ * a per-device cache of freed blocks (bounded by CULSH_POOL_MAX_MB, default 8192, 0 = off);
+ * this call hands every cached block back to the driver. */
+void culsh_memory_trim(void);
+
 /* ---- seeded hash parameters (host side) -------------------------------------------------
  * Role of generate_random_projections (rplsh/hash.cuh:58-78),
  * generate_random_projections_biases (pslsh/hash.cuh:59-89) and generate_hash_integers

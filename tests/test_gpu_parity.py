@@ -480,3 +480,24 @@ def test_pslsh_wide_value_range_keeps_plain_keys(ctx):
     assert_index_matches(ctx.index_arrays(ih), exp_ix)
     assert_candidates_match(ctx.pslsh_query(X[:200], ih), o.query_index(sig[:, :200], exp_ix))
     ctx.free_index(ih)
+
+
+def test_object_memory_is_reused_and_trimmed(ctx):
+    """Index and candidate arrays come from a cache of freed blocks: results must not depend on
+    whether a block is fresh or reused, and trimming the cache must leave everything working."""
+    _announce("memory_pool")
+    rng = np.random.default_rng(3)
+    T, n, nq, H = 4, 3000, 100, 3
+    sig = random_sigs(rng, T, n, H, "rplsh")
+    qsig = random_sigs(rng, T, nq, H, "rplsh")
+    exp_ix = o.fit_index(sig, H)
+    exp = o.query_index(qsig, exp_ix)
+    from abi import assert_candidates_match, assert_index_matches
+
+    for round_ in range(3):
+        ih, _ = ctx.core_fit_index(sig, H)
+        assert_index_matches(ctx.index_arrays(ih), exp_ix)
+        assert_candidates_match(ctx.core_query_index(qsig, ih), exp)
+        ctx.free_index(ih)
+        if round_ == 1:
+            ctx.lib.culsh_memory_trim()
