@@ -148,7 +148,10 @@ def main() -> int:
         achieved = flops_step / (ms_step * 1e-3) / 1e12
         roofline = {"kernel": proj_name, "bound": "mfma", "achieved": round(achieved, 3),
                     "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s",
-                    "frac": round(achieved / PEAK_FP32_MFMA_TFLOPS, 4), "traffic": None,
+                    "frac": round(achieved / PEAK_FP32_MFMA_TFLOPS, 4),
+                    # HBM bytes of the fit launch at the default size: rocprofv3 FETCH_SIZE x 2.0
+                    # (494.7 MiB) + WRITE_SIZE x 1.0 (122.1 MiB), scale factors from a 1 GiB copy
+                    "traffic": 646_800_000 if (n, nq) == (1_000_000, 10_000) else None,
                     "work": "2*(n+q)*d*T*H flop per step over the fit and query launches",
                     "dominant_kernel_by_time": dominant}
 
