@@ -64,7 +64,8 @@ __device__ __forceinline__ float4 load4(const float* __restrict__ base, size_t r
 // VEC: n_features is a multiple of 4 and X, P are 16-byte aligned, so a stage is fetched
 // with unconditional 16-byte loads.  Rows past the end of X and padding columns read a
 // valid row instead of zeros: their accumulators are never stored.
-template <int EPI, bool VEC, int BK>
+// FULLK (with VEC): n_features is a multiple of BK, so no stage needs zero filling.
+template <int EPI, bool VEC, int BK, bool FULLK>
 __global__ __launch_bounds__(NTHREADS) void project_f32_kernel(ProjArgs a) {
     constexpr int PITCH = BK + 4;  // LDS row pitch in floats (bank spread for 16-byte reads)
     constexpr int F4 = BK / 4;     // float4 per tile row and stage
@@ -108,7 +109,15 @@ __global__ __launch_bounds__(NTHREADS) void project_f32_kernel(ProjArgs a) {
     }
     // stage fetch: 4 + 4 float4 per thread
     auto fetch = [&](int k, float4 (&ra)[NLD], float4 (&rb)[NLD]) {
-        if (VEC) {
+        if (VEC && FULLK) {
+#pragma unroll
+            for (int i = 0; i < NLD; ++i) {
+                const float4 va = *reinterpret_cast<const float4*>(a.X + xoff[i] + k);
+                const float4 vb = *reinterpret_cast<const float4*>(a.P + poff[i] + k);
+                ra[i] = make_float4(va.x, va.y, va.z, va.w);
+                rb[i] = make_float4(vb.x, vb.y, vb.z, vb.w);
+            }
+        } else if (VEC) {
             const int kk = min(k, d - 4);
             const bool inside = k < d;  // a float4 is entirely inside or entirely outside [0, d)
 #pragma unroll
@@ -184,33 +193,43 @@ __global__ __launch_bounds__(NTHREADS) void project_f32_kernel(ProjArgs a) {
         for (int i = 0; i < 2; ++i)
 #pragma unroll
             for (int j = 0; j < 2; ++j) {
-                uint32_t mine = 0;
+                int mine = 0;
 #pragma unroll
                 for (int v = 0; v < 16; ++v) {
                     // hash bit = 1 iff the sign bit is clear (rplsh/hash.cuh:47)
                     const unsigned long long m =
                         __builtin_amdgcn_ballot_w64((__float_as_uint(acc[i][j][v]) >> 31) == 0u);
+                    // the low half of the ballot is the word of row rlo, the high half that of row
+                    // rlo + 4: each goes to the lane of that number
                     const int rlo = 8 * (v >> 2) + (v & 3);
-                    mine = (lane == rlo) ? static_cast<uint32_t>(m) : mine;
-                    mine = (lane == rlo + 4) ? static_cast<uint32_t>(m >> 32) : mine;
+                    const uint32_t m_lo = static_cast<uint32_t>(m), m_hi = static_cast<uint32_t>(m >> 32);
+                    // (on gfx950 a vector instruction may not read an SGPR in the two issue slots after
+                    // the vector compare that wrote it; the compiler does not pad inline assembly)
+                    asm("s_nop 1\n\tv_writelane_b32 %0, %1, %3\n\tv_writelane_b32 %0, %2, %4"
+                        : "+v"(mine)
+                        : "s"(m_lo), "s"(m_hi), "n"(rlo), "n"(rlo + 4));
                 }
-                if (lane < 32) tw[(wm * 64 + i * 32 + lane) * (BN / 32) + (wn * 2 + j)] = mine;
+                if (lane < 32) tw[(wm * 64 + i * 32 + lane) * (BN / 32) + (wn * 2 + j)] = static_cast<uint32_t>(mine);
             }
         __syncthreads();
         uint32_t* keys = static_cast<uint32_t*>(a.out);
         if (H <= 32) {
             const int tpt = 32 / H;
             const uint32_t mask = (H == 32) ? 0xFFFFFFFFu : ((1u << H) - 1u);
-            const int total = (BN / 32) * tpt * BM;
-            for (int idx = tid; idx < total; idx += NTHREADS) {
-                const int tl = idx / BM, row = idx - tl * BM;
-                const int tc = tl / tpt, sub = tl - tc * tpt;
+            // (table slot tl, row) pairs, rows fastest: a thread keeps its row and steps tl by
+            // NTHREADS / BM, carrying (tc, sub) = (tl / tpt, tl % tpt) along without dividing
+            constexpr int TL_STEP = NTHREADS / BM;
+            const int row = tid % BM, grow = rt * BM + row;
+            int tl = tid / BM;
+            int tc = tl / tpt, sub = tl - tc * tpt;
+            for (; tl < (BN / 32) * tpt; tl += TL_STEP) {
                 const int table = (ct * (BN / 32) + tc) * tpt + sub;
-                const int grow = rt * BM + row;
                 if (table < T && grow < n) {
                     const uint32_t field = (tw[row * (BN / 32) + tc] >> (sub * H)) & mask;
                     keys[static_cast<size_t>(table) * n + grow] = field << (32 - H);
                 }
+                sub += TL_STEP;
+                while (sub >= tpt) { sub -= tpt; ++tc; }
             }
         } else {
             const int wt = (H + 31) >> 5;
@@ -335,8 +354,9 @@ culsh_status launch_project_f32(culsh_ctx* ctx, const float* X, const float* P, 
     const bool vec = a.vec_x && a.vec_p;
 #define PROJ_CASE(E)                                                                              \
     case E:                                                                                       \
-        if (vec) CULSH_LAUNCH(ctx, (project_f32_kernel<E, true, 32>), grid, block, 0, ctx->stream, a);   \
-        else CULSH_LAUNCH(ctx, (project_f32_kernel<E, false, 32>), grid, block, 0, ctx->stream, a);      \
+        if (vec && d % 32 == 0) CULSH_LAUNCH(ctx, (project_f32_kernel<E, true, 32, true>), grid, block, 0, ctx->stream, a); \
+        else if (vec) CULSH_LAUNCH(ctx, (project_f32_kernel<E, true, 32, false>), grid, block, 0, ctx->stream, a);         \
+        else CULSH_LAUNCH(ctx, (project_f32_kernel<E, false, 32, false>), grid, block, 0, ctx->stream, a);                 \
         break;
     switch (epi) {
         PROJ_CASE(EPI_SIGN_KEYS)
