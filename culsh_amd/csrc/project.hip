@@ -93,27 +93,31 @@ __global__ __launch_bounds__(NTHREADS) void project_f32_kernel(ProjArgs a) {
     const int n = a.n, d = a.d, T = a.T, H = a.H;
     const int TH = T * H;
 
-    // global -> LDS staging: thread loads float4 number (tid + 256*i), i < 4, of each tile
+    // global -> LDS staging: thread loads float4 number (tid + 256*i), i < 4, of each tile.
+    // Addresses are a wavefront-uniform tile base plus a 32-bit element offset per thread.
     const int lrow = tid / F4, c4 = (tid % F4) * 4;
-    size_t xoff[NLD], poff[NLD];
+    const float* xbase = a.X + static_cast<size_t>(rt) * BM * d;
+    uint32_t xoff[NLD], poff[NLD];
     bool xok[NLD], pok[NLD];
 #pragma unroll
     for (int i = 0; i < NLD; ++i) {
-        const int row = rt * BM + lrow + RSTEP * i;
+        const int lr = lrow + RSTEP * i;  // row inside the tile
+        const int row = rt * BM + lr;
         xok[i] = row < n;
-        xoff[i] = static_cast<size_t>(VEC ? min(row, n - 1) : row) * d;
-        const int vc = ct * BN + lrow + RSTEP * i;
+        // VEC reads a valid row instead of predicating: the last row of X for rows past the end
+        xoff[i] = static_cast<uint32_t>(VEC ? min(lr, n - 1 - rt * BM) : lr) * static_cast<uint32_t>(d);
+        const int vc = ct * BN + lr;
         const int prow = (EPI == EPI_SIGN_KEYS) ? sign_vcol_to_prow(vc, T, H) : (vc < TH ? vc : -1);
         pok[i] = prow >= 0;
-        poff[i] = static_cast<size_t>(prow < 0 ? 0 : prow) * d;
+        poff[i] = static_cast<uint32_t>(prow < 0 ? 0 : prow) * static_cast<uint32_t>(d);
     }
     // stage fetch: 4 + 4 float4 per thread
     auto fetch = [&](int k, float4 (&ra)[NLD], float4 (&rb)[NLD]) {
         if (VEC && FULLK) {
 #pragma unroll
             for (int i = 0; i < NLD; ++i) {
-                const float4 va = *reinterpret_cast<const float4*>(a.X + xoff[i] + k);
-                const float4 vb = *reinterpret_cast<const float4*>(a.P + poff[i] + k);
+                const float4 va = *reinterpret_cast<const float4*>(xbase + (xoff[i] + static_cast<uint32_t>(k)));
+                const float4 vb = *reinterpret_cast<const float4*>(a.P + (poff[i] + static_cast<uint32_t>(k)));
                 ra[i] = make_float4(va.x, va.y, va.z, va.w);
                 rb[i] = make_float4(vb.x, vb.y, vb.z, vb.w);
             }
@@ -122,15 +126,15 @@ __global__ __launch_bounds__(NTHREADS) void project_f32_kernel(ProjArgs a) {
             const bool inside = k < d;  // a float4 is entirely inside or entirely outside [0, d)
 #pragma unroll
             for (int i = 0; i < NLD; ++i) {
-                const float4 va = *reinterpret_cast<const float4*>(a.X + xoff[i] + kk);
-                const float4 vb = *reinterpret_cast<const float4*>(a.P + poff[i] + kk);
+                const float4 va = *reinterpret_cast<const float4*>(xbase + (xoff[i] + static_cast<uint32_t>(kk)));
+                const float4 vb = *reinterpret_cast<const float4*>(a.P + (poff[i] + static_cast<uint32_t>(kk)));
                 ra[i] = inside ? va : make_float4(0.f, 0.f, 0.f, 0.f);
                 rb[i] = inside ? vb : make_float4(0.f, 0.f, 0.f, 0.f);
             }
         } else {
 #pragma unroll
             for (int i = 0; i < NLD; ++i) {
-                ra[i] = load4(a.X, xoff[i], k, d, xok[i], 0);
+                ra[i] = load4(xbase, xoff[i], k, d, xok[i], 0);
                 rb[i] = load4(a.P, poff[i], k, d, pok[i], 0);
             }
         }
@@ -332,6 +336,8 @@ culsh_status launch_project_f32(culsh_ctx* ctx, const float* X, const float* P, 
     const bool floor_epi = (epi == EPI_FLOOR_I32);
     CULSH_REQUIRE(!floor_epi || b, CULSH_ERR_INVALID, "projection: bias is required");
     CULSH_REQUIRE(static_cast<long long>(T) * H < (1ll << 30), CULSH_ERR_LIMIT, "T*H too large");
+    CULSH_REQUIRE(static_cast<long long>(T) * H * d < (1ll << 32) && static_cast<long long>(BM) * d < (1ll << 31),
+                  CULSH_ERR_LIMIT, "projection: T*H*n_features must be below 2^32");
     long long n_vcols;
     if (epi == EPI_SIGN_KEYS) {
         const long long tiles = (H <= 32) ? (T + (32 / H) - 1) / (32 / H)
