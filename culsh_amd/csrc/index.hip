@@ -87,6 +87,9 @@ __global__ __launch_bounds__(IB_THREADS) void count_heads_kernel(const uint32_t*
     if (threadIdx.x == 0) tile_counts[blockIdx.x] = total;
 }
 
+// Bucket heads of a tile are first gathered in LDS in order, then their offsets and keys are
+// written by consecutive threads to consecutive addresses (a head-per-thread write would touch
+// one cache line per lane when most items open a bucket of their own).
 __global__ __launch_bounds__(IB_THREADS) void build_index_kernel(
     const uint32_t* __restrict__ keys, const int32_t* __restrict__ rows, size_t N, int n, int T, int W,
     const uint64_t* __restrict__ tile_base, const uint64_t* __restrict__ n_buckets_dev,
@@ -94,11 +97,16 @@ __global__ __launch_bounds__(IB_THREADS) void build_index_kernel(
     uint32_t* __restrict__ bucket_keys, int32_t* __restrict__ table_bucket_offsets,
     int32_t* __restrict__ item_to_bucket) {
     __shared__ uint64_t scratch[17];
-    const size_t base = static_cast<size_t>(blockIdx.x) * IB_TILE + threadIdx.x * IB_ITEMS;
+    __shared__ uint16_t head_slot[IB_TILE];  // tile-local item numbers of the heads, ascending
+    const size_t tile_start = static_cast<size_t>(blockIdx.x) * IB_TILE;
+    const size_t base = tile_start + threadIdx.x * IB_ITEMS;
     uint32_t flag[IB_ITEMS];
     const uint64_t c = thread_flags(keys, base, N, n, W, flag);
     uint64_t total;
-    uint64_t run = tile_base[blockIdx.x] + block_exclusive_sum(c, scratch, &total);
+    const uint64_t first_bucket = tile_base[blockIdx.x];
+    const uint64_t ex = block_exclusive_sum(c, scratch, &total);
+    uint64_t run = first_bucket + ex;
+    uint32_t local = static_cast<uint32_t>(ex);
 #pragma unroll
     for (int i = 0; i < IB_ITEMS; ++i) {
         const size_t pos = base + i;
@@ -106,13 +114,26 @@ __global__ __launch_bounds__(IB_THREADS) void build_index_kernel(
         run += flag[i];
         const int32_t bucket = static_cast<int32_t>(run) - 1;  // scan + flag - 1 (fit.cuh:183)
         if (flag[i]) {
-            bucket_candidate_offsets[bucket] = static_cast<int32_t>(pos);  // fit.cuh:190-191
-            for (int w = 0; w < W; ++w) bucket_keys[static_cast<size_t>(bucket) * W + w] = keys[pos * W + w];
+            head_slot[local++] = static_cast<uint16_t>(threadIdx.x * IB_ITEMS + i);
             if (pos % n == 0) table_bucket_offsets[pos / n] = bucket;      // fit.cuh:317-326
         }
         if (item_to_bucket) {
             const size_t t = pos / n;
             item_to_bucket[static_cast<size_t>(rows[pos]) * T + t] = bucket;  // fit.cuh:180-185
+        }
+    }
+    __syncthreads();
+    const uint32_t heads = static_cast<uint32_t>(total);
+    for (uint32_t j = threadIdx.x; j < heads; j += IB_THREADS)
+        bucket_candidate_offsets[first_bucket + j] = static_cast<int32_t>(tile_start + head_slot[j]);  // fit.cuh:190-191
+    uint32_t* kout = bucket_keys + first_bucket * W;
+    if (W == 1) {
+        for (uint32_t j = threadIdx.x; j < heads; j += IB_THREADS) kout[j] = keys[tile_start + head_slot[j]];
+    } else {
+        const uint32_t words = heads * static_cast<uint32_t>(W);
+        for (uint32_t idx = threadIdx.x; idx < words; idx += IB_THREADS) {
+            const uint32_t j = idx / static_cast<uint32_t>(W), w = idx - j * static_cast<uint32_t>(W);
+            kout[idx] = keys[(tile_start + head_slot[j]) * W + w];
         }
     }
     if (blockIdx.x == 0 && threadIdx.x == 0) {  // terminators, fit.cuh:351-357
@@ -145,19 +166,30 @@ __global__ __launch_bounds__(256) void sig_to_keys_kernel(const uint8_t* __restr
     keys[idx] = k;
 }
 
+// Four consecutive signature bytes per thread (one 32-bit store where all four exist).
 __global__ __launch_bounds__(256) void keys_to_sig_kernel(const uint32_t* __restrict__ keys, size_t count,
                                                          const uint64_t* __restrict__ count_dev, int S, int enc,
                                                          int W, uint8_t* __restrict__ sig) {
-    const size_t idx = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
     if (count_dev) count = min(count, static_cast<size_t>(*count_dev));  // exact count known on the device only
-    if (idx >= count * S) return;
-    const size_t item = idx / S;
-    const int byte = static_cast<int>(idx - item * S);
-    const uint32_t* k = keys + item * W;
-    if (enc == ENC_BE)
-        sig[idx] = static_cast<uint8_t>(k[byte >> 2] >> (24 - 8 * (byte & 3)));
-    else
-        sig[idx] = static_cast<uint8_t>((k[byte >> 5] >> (31 - (byte & 31))) & 1u);
+    const size_t total = count * S;
+    const size_t b0 = (static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x) * 4;
+    if (b0 >= total) return;
+    size_t item = b0 / S;
+    int byte = static_cast<int>(b0 - item * S);
+    uint32_t packed = 0;
+    const int nb = static_cast<int>(min(static_cast<size_t>(4), total - b0));
+    for (int j = 0; j < nb; ++j) {
+        const uint32_t* k = keys + item * W;
+        const uint32_t v = (enc == ENC_BE) ? ((k[byte >> 2] >> (24 - 8 * (byte & 3))) & 0xFFu)
+                                           : ((k[byte >> 5] >> (31 - (byte & 31))) & 1u);
+        packed |= v << (8 * j);
+        if (++byte == S) { byte = 0; ++item; }
+    }
+    if (nb == 4) {
+        *reinterpret_cast<uint32_t*>(sig + b0) = packed;  // sig comes from the allocator: 4-byte aligned
+    } else {
+        for (int j = 0; j < nb; ++j) sig[b0 + j] = static_cast<uint8_t>(packed >> (8 * j));
+    }
 }
 
 }  // namespace
@@ -177,8 +209,9 @@ culsh_status launch_keys_to_sig(culsh_ctx* ctx, const uint32_t* keys, size_t cou
                                 int S, KeyEnc enc, int W, uint8_t* sig) {
     if (count == 0) return CULSH_OK;
     const size_t total = count * S;
-    CULSH_REQUIRE(total / 256 < (1ull << 31), CULSH_ERR_LIMIT, "too many buckets");
-    CULSH_LAUNCH(ctx, keys_to_sig_kernel, dim3(div_up(total, 256)), dim3(256), 0, ctx->stream, keys, count,
+    CULSH_REQUIRE(total / 1024 < (1ull << 31), CULSH_ERR_LIMIT, "too many buckets");
+    CULSH_REQUIRE(reinterpret_cast<uintptr_t>(sig) % 4 == 0, CULSH_ERR_INTERNAL, "signature array is not 4-byte aligned");
+    CULSH_LAUNCH(ctx, keys_to_sig_kernel, dim3(div_up(div_up(total, 4), 256)), dim3(256), 0, ctx->stream, keys, count,
                  count_dev, S, static_cast<int>(enc), W, sig);
     CULSH_LAUNCH_CHECK();
     return CULSH_OK;
