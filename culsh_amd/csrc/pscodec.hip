@@ -85,27 +85,43 @@ __global__ __launch_bounds__(256) void ps_compress_kernel(const int32_t* __restr
     if (nbits > 0) k[w++] = static_cast<uint32_t>(acc << (32 - nbits));
 }
 
+// A workgroup restores the signatures of PS_BPB consecutive buckets: the table of each bucket
+// is searched once and kept in LDS with the bucket's key words, then (bucket, hash) pairs are
+// written by consecutive threads to consecutive addresses.
+constexpr int PS_BPB = 256;
 __global__ __launch_bounds__(256) void ps_keys_to_sig_kernel(const uint32_t* __restrict__ keys, size_t count,
                                                             const uint64_t* __restrict__ count_dev,
                                                             const int32_t* __restrict__ table_bucket_offsets, int T,
                                                             int H, int bits, int rmax, int W,
                                                             const int32_t* __restrict__ inv,
                                                             int32_t* __restrict__ sig) {
-    const size_t idx = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    extern __shared__ uint32_t ps_lds[];  // [PS_BPB] table ids, then [PS_BPB][W] key words
+    uint32_t* tb = ps_lds;
+    uint32_t* kw = ps_lds + PS_BPB;
     if (count_dev) count = min(count, static_cast<size_t>(*count_dev));
-    if (idx >= count * H) return;
-    const size_t bucket = idx / H;
-    const int h = static_cast<int>(idx - bucket * H);
-    int lo = 0, hi = T;  // largest t with table_bucket_offsets[t] <= bucket
-    while (hi - lo > 1) {
-        const int mid = (lo + hi) >> 1;
-        if (static_cast<size_t>(table_bucket_offsets[mid]) <= bucket) lo = mid; else hi = mid;
+    const size_t b0 = static_cast<size_t>(blockIdx.x) * PS_BPB;
+    if (b0 >= count) return;
+    const int nb = static_cast<int>(min(static_cast<size_t>(PS_BPB), count - b0));
+    if (static_cast<int>(threadIdx.x) < nb) {
+        const size_t bucket = b0 + threadIdx.x;
+        int lo = 0, hi = T;  // largest t with table_bucket_offsets[t] <= bucket
+        while (hi - lo > 1) {
+            const int mid = (lo + hi) >> 1;
+            if (static_cast<size_t>(table_bucket_offsets[mid]) <= bucket) lo = mid; else hi = mid;
+        }
+        tb[threadIdx.x] = static_cast<uint32_t>(lo);
     }
-    const uint32_t* k = keys + bucket * W;
-    const int o = h * bits, w0 = o >> 5, sh = o & 31;
-    const unsigned long long two = (static_cast<unsigned long long>(k[w0]) << 32) | (w0 + 1 < W ? k[w0 + 1] : 0u);
-    const uint32_t code = static_cast<uint32_t>(two >> (64 - sh - bits)) & ((1u << bits) - 1u);
-    sig[idx] = code ? inv[static_cast<size_t>(lo * H + h) * rmax + (code - 1u)] : 0;
+    for (int i = threadIdx.x; i < nb * W; i += 256) kw[i] = keys[b0 * W + i];
+    __syncthreads();
+    const uint32_t mask = (1u << bits) - 1u;
+    for (int i = threadIdx.x; i < nb * H; i += 256) {
+        const int bl = i / H, h = i - bl * H;
+        const uint32_t* k = kw + bl * W;
+        const int o = h * bits, w0 = o >> 5, sh = o & 31;
+        const unsigned long long two = (static_cast<unsigned long long>(k[w0]) << 32) | (w0 + 1 < W ? k[w0 + 1] : 0u);
+        const uint32_t code = static_cast<uint32_t>(two >> (64 - sh - bits)) & mask;
+        sig[b0 * H + i] = code ? inv[static_cast<size_t>(tb[bl] * H + h) * rmax + (code - 1u)] : 0;
+    }
 }
 
 }  // namespace
@@ -191,10 +207,10 @@ culsh_status launch_ps_compress(culsh_ctx* ctx, const int32_t* sig, size_t rows,
 culsh_status launch_ps_keys_to_sig(culsh_ctx* ctx, const culsh_index* ix, size_t count, const uint64_t* count_dev,
                                    uint8_t* sig) {
     if (count == 0) return CULSH_OK;
-    const size_t total = count * ix->n_hashes;
-    CULSH_REQUIRE(total / 256 < (1ull << 31), CULSH_ERR_LIMIT, "too many buckets");
+    CULSH_REQUIRE(count / PS_BPB < (1ull << 31), CULSH_ERR_LIMIT, "too many buckets");
     const PsCodec& pc = ix->psc;
-    CULSH_LAUNCH(ctx, ps_keys_to_sig_kernel, dim3(div_up(total, 256)), dim3(256), 0, ctx->stream, ix->bucket_keys,
+    const size_t lds = static_cast<size_t>(PS_BPB) * (1 + ix->key_w) * sizeof(uint32_t);
+    CULSH_LAUNCH(ctx, ps_keys_to_sig_kernel, dim3(div_up(count, PS_BPB)), dim3(256), lds, ctx->stream, ix->bucket_keys,
                  count, count_dev, ix->table_bucket_offsets, ix->n_hash_tables, ix->n_hashes, pc.bits, pc.rmax,
                  ix->key_w, pc.inv, reinterpret_cast<int32_t*>(sig));
     CULSH_LAUNCH_CHECK();
