@@ -125,6 +125,18 @@ culsh_status read_back_u64(culsh_ctx* ctx, const uint64_t* dev, int count, uint6
     return CULSH_OK;
 }
 
+culsh_status read_back_pair(culsh_ctx* ctx, const uint64_t* dev_a, const uint32_t* dev_b_or_null, uint64_t* a,
+                            uint32_t* b) {
+    ctx->pinned[1] = 0;
+    CULSH_HIP(hipMemcpyAsync(&ctx->pinned[0], dev_a, sizeof(uint64_t), hipMemcpyDeviceToHost, ctx->stream));
+    if (dev_b_or_null)
+        CULSH_HIP(hipMemcpyAsync(&ctx->pinned[1], dev_b_or_null, sizeof(uint32_t), hipMemcpyDeviceToHost, ctx->stream));
+    CULSH_HIP(hipStreamSynchronize(ctx->stream));
+    *a = ctx->pinned[0];
+    *b = static_cast<uint32_t>(ctx->pinned[1] & 0xffffffffu);
+    return CULSH_OK;
+}
+
 culsh_status read_back_u32(culsh_ctx* ctx, const uint32_t* dev, int count, uint32_t* host) {
     CULSH_REQUIRE(count <= 128, CULSH_ERR_INTERNAL, "read_back: too many words");
     CULSH_HIP(hipMemcpyAsync(ctx->pinned, dev, count * sizeof(uint32_t), hipMemcpyDeviceToHost, ctx->stream));
@@ -414,7 +426,7 @@ static culsh_status finish_fit(culsh_ctx* ctx, uint32_t* keys, int n, int T, int
 }
 
 template <typename T>
-static culsh_status dense_fit(culsh_ctx* ctx, Family fam, const T* X, int n, int d, int nT, int H, int window,
+static culsh_status dense_fit_once(culsh_ctx* ctx, Family fam, const T* X, int n, int d, int nT, int H, int window,
                               uint64_t seed, const T* P_host, const T* b_host, culsh_index** index_out,
                               culsh_candidates** cands_out) {
     CULSH_TRY(check_fit_args(ctx, X, n, d, nT, H, index_out ? static_cast<void*>(index_out) : static_cast<void*>(cands_out)));
@@ -473,7 +485,7 @@ static culsh_status dense_fit(culsh_ctx* ctx, Family fam, const T* X, int n, int
     return CULSH_OK;
 }
 
-static culsh_status minhash_fit_impl(culsh_ctx* ctx, const int32_t* indices, const int32_t* indptr, int n, int d,
+static culsh_status minhash_fit_once(culsh_ctx* ctx, const int32_t* indices, const int32_t* indptr, int n, int d,
                                      int nT, int H, uint64_t seed, const uint32_t* A_host, const uint32_t* B_host,
                                      culsh_index** index_out, culsh_candidates** cands_out) {
     CULSH_TRY(check_fit_args(ctx, indptr, n, d, nT, H, index_out ? static_cast<void*>(index_out) : static_cast<void*>(cands_out)));
@@ -552,6 +564,40 @@ static culsh_status index_array(const culsh_index* ix, culsh_array which, const 
 using namespace culsh_amd;
 
 // ======================================================================================
+// The radix sort's chained scan cannot stall as long as workgroups start in index order;
+// should it ever give up, the context switches to unchained passes and the fit is repeated
+// from the hashing step (the sort has overwritten its input by then).
+template <typename F>
+static culsh_status with_sort_retry(culsh_ctx* ctx, F&& fit) {
+    culsh_status s = fit();
+    if (s == CULSH_RETRY_UNCHAINED && ctx) {
+        ctx->sort_unchained = true;
+        s = fit();
+    }
+    if (s == CULSH_RETRY_UNCHAINED) {
+        set_error("radix sort: chained scan gave up and no unchained retry was possible");
+        s = CULSH_ERR_INTERNAL;
+    }
+    return s;
+}
+
+template <typename T>
+static culsh_status dense_fit(culsh_ctx* ctx, Family fam, const T* X, int n, int d, int nT, int H, int window,
+                              uint64_t seed, const T* P_host, const T* b_host, culsh_index** index_out,
+                              culsh_candidates** cands_out) {
+    return with_sort_retry(ctx, [&] {
+        return dense_fit_once<T>(ctx, fam, X, n, d, nT, H, window, seed, P_host, b_host, index_out, cands_out);
+    });
+}
+
+static culsh_status minhash_fit_impl(culsh_ctx* ctx, const int32_t* indices, const int32_t* indptr, int n, int d,
+                                     int nT, int H, uint64_t seed, const uint32_t* A_host, const uint32_t* B_host,
+                                     culsh_index** index_out, culsh_candidates** cands_out) {
+    return with_sort_retry(ctx, [&] {
+        return minhash_fit_once(ctx, indices, indptr, n, d, nT, H, seed, A_host, B_host, index_out, cands_out);
+    });
+}
+
 extern "C" {
 
 const char* culsh_last_error(void) { return g_last_error.c_str(); }
@@ -798,7 +844,7 @@ culsh_status culsh_minhash_compute(culsh_ctx* ctx, const int32_t* indices, const
     return arena_end(ctx);
 }
 
-culsh_status culsh_core_fit_index(culsh_ctx* ctx, const void* X_sig, int n, int T, int H, int S,
+static culsh_status core_fit_index_once(culsh_ctx* ctx, const void* X_sig, int n, int T, int H, int S,
                                   int32_t* item_to_bucket, culsh_index** out) {
     CULSH_TRY(check_fit_args(ctx, X_sig, n, 1, T, H, out));
     CULSH_REQUIRE(S > 0, CULSH_ERR_INVALID, "sig_nbytes must be > 0");  // core/fit.cuh:224
@@ -816,6 +862,11 @@ culsh_status culsh_core_fit_index(culsh_ctx* ctx, const void* X_sig, int n, int 
     CULSH_TRY(arena_end(ctx));
     *out = ix.release();
     return CULSH_OK;
+}
+
+culsh_status culsh_core_fit_index(culsh_ctx* ctx, const void* X_sig, int n, int T, int H, int S,
+                                  int32_t* item_to_bucket, culsh_index** out) {
+    return with_sort_retry(ctx, [&] { return core_fit_index_once(ctx, X_sig, n, T, H, S, item_to_bucket, out); });
 }
 
 static culsh_status sig_query_keys(culsh_ctx* ctx, const void* Q_sig, int nq, int S, const culsh_index* ix,
@@ -874,7 +925,7 @@ culsh_status culsh_core_query_from_matched_buckets(culsh_ctx* ctx, const int32_t
     return CULSH_OK;
 }
 
-culsh_status culsh_core_fit_query(culsh_ctx* ctx, const void* X_sig, int n, int T, int H, int S,
+static culsh_status core_fit_query_once(culsh_ctx* ctx, const void* X_sig, int n, int T, int H, int S,
                                   culsh_candidates** out) {
     CULSH_TRY(check_fit_args(ctx, X_sig, n, 1, T, H, out));
     CULSH_REQUIRE(S > 0 && S <= 256, CULSH_ERR_INVALID, "sig_nbytes must be in [1, 256]");
@@ -892,6 +943,11 @@ culsh_status culsh_core_fit_query(culsh_ctx* ctx, const void* X_sig, int n, int 
     CULSH_TRY(arena_end(ctx));
     *out = c.release();
     return CULSH_OK;
+}
+
+culsh_status culsh_core_fit_query(culsh_ctx* ctx, const void* X_sig, int n, int T, int H, int S,
+                                  culsh_candidates** out) {
+    return with_sort_retry(ctx, [&] { return core_fit_query_once(ctx, X_sig, n, T, H, S, out); });
 }
 
 // ---- index object

@@ -85,6 +85,10 @@ struct culsh_ctx {
     size_t arena_want = 0;               // high-water mark incl. overflow blocks
     std::vector<void*> overflow;         // freed at the end of the call
     uint64_t* pinned = nullptr;          // 64 x u64 pinned host words for D2H scalars
+    // chained scan of the radix sort: give-up flag of the last sort (device, arena) and the
+    // switch to the unchained passes after a give-up
+    uint32_t* sort_err_dev = nullptr;
+    bool sort_unchained = false;
     int lds_max = 0;                     // max LDS bytes per workgroup
     int n_cus = 0;
     // per-kernel timing with HIP events on `stream` (off unless enabled)
@@ -186,6 +190,12 @@ void profile_collect(culsh_ctx* ctx);  // call with the stream idle
 // Reads `count` (<= 64) device u64/u32 words into host memory; synchronises the stream.
 culsh_status read_back_u64(culsh_ctx* ctx, const uint64_t* dev, int count, uint64_t* host);
 culsh_status read_back_u32(culsh_ctx* ctx, const uint32_t* dev, int count, uint32_t* host);
+// one u64 and (optionally) one u32 from different places with a single synchronisation
+culsh_status read_back_pair(culsh_ctx* ctx, const uint64_t* dev_a, const uint32_t* dev_b_or_null, uint64_t* a,
+                            uint32_t* b);
+// Internal status: the radix sort's chained scan gave up; the caller switches the context to
+// unchained passes and repeats the fit.  Never returned through the C ABI.
+constexpr culsh_status CULSH_RETRY_UNCHAINED = static_cast<culsh_status>(7);
 
 // ---------------------------------------------------------------- projection (project.hip)
 // Output modes of the projection kernels.

@@ -262,7 +262,15 @@ culsh_status build_index_from_sorted(culsh_ctx* ctx, const uint32_t* sorted_keys
         CULSH_TRY(launch_ps_keys_to_sig(ctx, index, B_bound, total_dev, index->all_bucket_signatures));
     else
         CULSH_TRY(launch_keys_to_sig(ctx, index->bucket_keys, B_bound, total_dev, S, enc, W, index->all_bucket_signatures));
-    if (deferred) CULSH_TRY(read_back_u64(ctx, total_dev, 1, &n_buckets64));
+    // end-of-build read-back: the bucket count (unless fetched above) and the sort's give-up flag
+    uint32_t sort_gave_up = 0;
+    if (deferred) {
+        CULSH_TRY(read_back_pair(ctx, total_dev, ctx->sort_err_dev, &n_buckets64, &sort_gave_up));
+    } else if (ctx->sort_err_dev) {
+        CULSH_TRY(read_back_u32(ctx, ctx->sort_err_dev, 1, &sort_gave_up));
+    }
+    ctx->sort_err_dev = nullptr;
+    if (sort_gave_up) return CULSH_RETRY_UNCHAINED;
     index->n_total_buckets = static_cast<int>(n_buckets64);
     return CULSH_OK;
 }

@@ -7,9 +7,18 @@
 // key of its table are skipped - for sign-bit keys of H hashes that leaves ceil(H/8)
 // passes instead of H + 1.
 //
-// One pass = three launches with no inter-workgroup waiting: per-tile digit histograms,
-// an exclusive scan of [table][digit][tile], and a scatter that ranks items inside the
-// tile with wavefront ballots (stable: tile order, then wave order, then lane order).
+// A pass is one scatter launch that ranks items inside a tile with wavefront ballots
+// (stable: tile order, then wave order, then lane order).  Where a tile's digit runs start
+// is found by a chained scan: one launch before the first pass counts every digit of every
+// pass per table (the counts do not depend on the order of the items), and in a pass the
+// workgroup of tile k publishes its digit counts and sums those of tiles < k by looking
+// back over the published words.  Workgroups are numbered tile-major, so the tiles of one
+// table that run at the same time are few and the look-back is short.  The poll count is
+// bounded; a give-up is reported and the caller repeats the fit with the unchained form of
+// a pass: per-tile digit histograms, an exclusive scan of [table][digit][tile], scatter.
+#include <cstdlib>
+#include <vector>
+
 #include "block_utils.hpp"
 #include "common.hpp"
 
@@ -82,6 +91,55 @@ __global__ __launch_bounds__(256) void iota_rows_kernel(int32_t* __restrict__ ro
     if (i < total) rows[i] = static_cast<int32_t>(i % n);
 }
 
+constexpr int MAX_PASSES_PER_LAUNCH = 16;
+struct PassList {
+    int count;
+    int word[MAX_PASSES_PER_LAUNCH];
+    int shift[MAX_PASSES_PER_LAUNCH];
+};
+
+// Digit totals per (pass, table, digit) for up to 16 passes in one read of the keys.
+__global__ __launch_bounds__(SORT_THREADS) void radix_totals_kernel(const uint32_t* __restrict__ keys, int n, int W,
+                                                                   PassList pl, int T,
+                                                                   uint32_t* __restrict__ dtot /*[pass][T][256]*/) {
+    __shared__ uint32_t h[MAX_PASSES_PER_LAUNCH][256];
+    const int tile = blockIdx.x, t = blockIdx.y;
+    // few passes leave room for one histogram copy per wavefront (fewer same-address atomics)
+    const int copies = pl.count <= MAX_PASSES_PER_LAUNCH / 4 ? 4 : (pl.count <= MAX_PASSES_PER_LAUNCH / 2 ? 2 : 1);
+    const int mine = (threadIdx.x >> 6) % copies;
+    for (int i = threadIdx.x; i < copies * pl.count * 256; i += SORT_THREADS) (&h[0][0])[i] = 0;
+    __syncthreads();
+    const uint32_t* tk = keys + static_cast<size_t>(t) * n * W;
+    uint32_t kw[SORT_ITEMS];
+    int last_word = -1;
+    for (int p = 0; p < pl.count; ++p) {  // passes are ordered by word, so a word is fetched once
+        if (pl.word[p] != last_word) {
+            last_word = pl.word[p];
+#pragma unroll
+            for (int j = 0; j < SORT_ITEMS; ++j) {
+                const int idx = tile * SORT_TILE + j * SORT_THREADS + threadIdx.x;
+                kw[j] = (idx < n) ? tk[static_cast<size_t>(idx) * W + last_word] : 0u;
+            }
+        }
+        uint32_t* hp = h[mine * pl.count + p];
+        const int shift = pl.shift[p];
+#pragma unroll
+        for (int j = 0; j < SORT_ITEMS; ++j) {
+            const int idx = tile * SORT_TILE + j * SORT_THREADS + threadIdx.x;
+            if (idx < n) atomicAdd(&hp[(kw[j] >> shift) & 255u], 1u);
+        }
+    }
+    __syncthreads();
+    for (int p = 0; p < pl.count; ++p) {
+        uint32_t c = 0;
+        for (int r = 0; r < copies; ++r) c += h[r * pl.count + p][threadIdx.x];
+        if (c) atomicAdd(&dtot[(static_cast<size_t>(p) * T + t) * 256 + threadIdx.x], c);
+    }
+}
+
+// Published word of the chained scan: 2-bit tag, 30-bit value.
+constexpr uint32_t ST_COUNT = 1u << 30, ST_SUM = 2u << 30, ST_VALUE = ST_COUNT - 1u;
+
 __global__ __launch_bounds__(SORT_THREADS) void radix_hist_kernel(const uint32_t* __restrict__ keys, int n,
                                                                  int W, int word, int shift, int tiles,
                                                                  uint32_t* __restrict__ hist,
@@ -139,11 +197,16 @@ __global__ __launch_bounds__(256) void radix_scan_kernel(uint32_t* __restrict__ 
 }
 
 // KW: key words known at compile time (1, 2 or 4: keys move as one vector), 0 = any W.
-template <int KW>
+// CHAINED: `hist_scanned` is null; `dtot` holds this pass's digit totals [T][256], `state`
+// the published words [T][tiles][256] (zero at launch), `err` the give-up flag; the grid is
+// one-dimensional and tile-major.
+template <int KW, bool CHAINED>
 __global__ __launch_bounds__(SORT_THREADS) void radix_scatter_kernel(
     const uint32_t* __restrict__ keys_in, const int32_t* __restrict__ rows_in,
     uint32_t* __restrict__ keys_out, int32_t* __restrict__ rows_out,
-    const uint32_t* __restrict__ hist_scanned, int n, int W, int word, int shift, int tiles) {
+    const uint32_t* __restrict__ hist_scanned, int n, int W, int word, int shift, int tiles, int T,
+    const uint32_t* __restrict__ dtot, uint32_t* __restrict__ state, uint32_t* __restrict__ err,
+    int spin_limit) {
     constexpr bool ONE_WORD = (KW == 1);
     constexpr int NW = SORT_THREADS / 64;
     __shared__ uint32_t whist[NW][256];   // per-wave digit counts, then per-wave offsets inside a digit run
@@ -152,7 +215,8 @@ __global__ __launch_bounds__(SORT_THREADS) void radix_scatter_kernel(
     __shared__ uint32_t scratch[17];
     __shared__ uint32_t st_key[SORT_TILE];                 // ONE_WORD: key, else: source slot in the tile
     __shared__ int32_t st_row[ONE_WORD ? SORT_TILE : 1];
-    const int tile = blockIdx.x, t = blockIdx.y;
+    const int tile = CHAINED ? static_cast<int>(blockIdx.x / T) : static_cast<int>(blockIdx.x);
+    const int t = CHAINED ? static_cast<int>(blockIdx.x - static_cast<unsigned>(tile) * T) : static_cast<int>(blockIdx.y);
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     for (int i = tid; i < NW * 256; i += SORT_THREADS) (&whist[0][0])[i] = 0;
     __syncthreads();
@@ -203,7 +267,39 @@ __global__ __launch_bounds__(SORT_THREADS) void radix_scatter_kernel(
         uint32_t tile_total;
         const uint32_t ds = block_exclusive_sum(tot, scratch, &tile_total);
         dstart[tid] = ds;
-        gbase[tid] = hist_scanned[(static_cast<size_t>(t) * 256 + tid) * tiles + tile] - ds;
+        if (CHAINED) {
+            // publish this tile's count of digit `tid`, then add up the tiles before it
+            uint32_t* st = state + static_cast<size_t>(t) * tiles * 256 + tid;  // entry of tile k: st[k * 256]
+            __hip_atomic_store(st + static_cast<size_t>(tile) * 256, (tile == 0 ? ST_SUM : ST_COUNT) | tot,
+                               __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            // start of the digit's range in the table: exclusive scan of the digit totals
+            uint32_t all;
+            const uint32_t dbase = block_exclusive_sum(dtot[t * 256 + tid], scratch, &all);
+            uint32_t before = 0;
+            int polls = 0;
+            for (int k = tile - 1; k >= 0;) {
+                const uint32_t v = __hip_atomic_load(st + static_cast<size_t>(k) * 256, __ATOMIC_RELAXED,
+                                                     __HIP_MEMORY_SCOPE_AGENT);
+                const uint32_t tag = v >> 30;
+                if (tag == 0u) {
+                    if (++polls > spin_limit) {  // give up: positions stay inside the digit's range
+                        atomicOr(err, 1u);
+                        break;
+                    }
+                    __builtin_amdgcn_s_sleep(1);
+                    continue;
+                }
+                before += v & ST_VALUE;
+                if (tag == 2u) break;
+                --k;
+            }
+            if (tile > 0)
+                __hip_atomic_store(st + static_cast<size_t>(tile) * 256, ST_SUM | (before + tot), __ATOMIC_RELAXED,
+                                   __HIP_MEMORY_SCOPE_AGENT);
+            gbase[tid] = dbase + before - ds;
+        } else {
+            gbase[tid] = hist_scanned[(static_cast<size_t>(t) * 256 + tid) * tiles + tile] - ds;
+        }
     }
     __syncthreads();
     // Stage the tile in digit order in LDS so that the global stores below walk
@@ -305,34 +401,81 @@ culsh_status sort_tables(culsh_ctx* ctx, uint32_t* keys_in, uint32_t* keys_tmp, 
         return CULSH_OK;
     }
 
-    uint32_t* hist = nullptr;
-    CULSH_TRY(arena_alloc_t(ctx, static_cast<size_t>(T) * 256 * tiles, &hist));
     uint32_t* kin = keys_in;
     uint32_t* kout = keys_tmp;
     const int np = static_cast<int>(passes.size());
-    uint32_t* dtot = nullptr;  // [pass][T][256] digit totals, accumulated by the histogram kernel
+    uint32_t* dtot = nullptr;  // [pass][T][256] digit totals
     CULSH_TRY(arena_alloc_t(ctx, static_cast<size_t>(np) * T * 256, &dtot));
     CULSH_HIP(hipMemsetAsync(dtot, 0, static_cast<size_t>(np) * T * 256 * sizeof(uint32_t), ctx->stream));
+
+    const char* env_unchained = std::getenv("CULSH_SORT_UNCHAINED");
+    const bool chained = !ctx->sort_unchained && n < (1 << 30) && !(env_unchained && *env_unchained == '1') &&
+                         static_cast<size_t>(tiles) * T < (1ull << 31);
+    uint32_t* hist = nullptr;   // unchained: [T][256][tiles]
+    uint32_t* state = nullptr;  // chained: [pass][T][tiles][256]
+    uint32_t* err = nullptr;
+    const size_t state_words = static_cast<size_t>(T) * tiles * 256;
+    ctx->sort_err_dev = nullptr;
+    if (chained) {
+        CULSH_TRY(arena_alloc_t(ctx, static_cast<size_t>(np) * state_words, &state));
+        CULSH_TRY(arena_alloc_t(ctx, 2, &err));
+        CULSH_HIP(hipMemsetAsync(state, 0, static_cast<size_t>(np) * state_words * sizeof(uint32_t), ctx->stream));
+        CULSH_HIP(hipMemsetAsync(err, 0, 2 * sizeof(uint32_t), ctx->stream));
+        ctx->sort_err_dev = err;
+        for (int p0 = 0; p0 < np; p0 += MAX_PASSES_PER_LAUNCH) {
+            PassList pl;
+            pl.count = std::min(MAX_PASSES_PER_LAUNCH, np - p0);
+            for (int i = 0; i < MAX_PASSES_PER_LAUNCH; ++i) {
+                pl.word[i] = i < pl.count ? passes[p0 + i].word : 0;
+                pl.shift[i] = i < pl.count ? passes[p0 + i].shift : 0;
+            }
+            CULSH_LAUNCH(ctx, radix_totals_kernel, dim3(tiles, T), dim3(SORT_THREADS), 0, ctx->stream, keys_in, n, W, pl,
+                         T, dtot + static_cast<size_t>(p0) * T * 256);
+            CULSH_LAUNCH_CHECK();
+        }
+    } else {
+        CULSH_TRY(arena_alloc_t(ctx, static_cast<size_t>(T) * 256 * tiles, &hist));
+    }
+    // polls of an unpublished predecessor before a workgroup gives up (CULSH_SORT_SPIN_LIMIT: tests
+    // set it to 0 to reach the give-up path while every kernel still runs to its end)
+    const char* env_spin = std::getenv("CULSH_SORT_SPIN_LIMIT");
+    const int spin_limit = (env_spin && *env_spin) ? std::atoi(env_spin) : (1 << 20);
     const int32_t* rin = nullptr;
     for (int p = 0; p < np; ++p) {
         // the last pass must land in rows_out
         int32_t* rout = ((np - 1 - p) % 2 == 0) ? rows_out : rows_tmp;
-        const dim3 grid(tiles, T);
-        CULSH_LAUNCH(ctx, radix_hist_kernel, grid, dim3(SORT_THREADS), 0, ctx->stream, kin, n, W,
-                           passes[p].word, passes[p].shift, tiles, hist, dtot + static_cast<size_t>(p) * T * 256);
-        CULSH_LAUNCH_CHECK();
-        CULSH_LAUNCH(ctx, radix_scan_kernel, dim3(T, SCAN_PARTS), dim3(256), 0, ctx->stream, hist,
-                     dtot + static_cast<size_t>(p) * T * 256, tiles);
-        CULSH_LAUNCH_CHECK();
+        uint32_t* pass_dtot = dtot + static_cast<size_t>(p) * T * 256;
         const bool aligned = reinterpret_cast<uintptr_t>(kin) % 16 == 0 && reinterpret_cast<uintptr_t>(kout) % 16 == 0;
-#define SCATTER(KW)                                                                                              \
-    CULSH_LAUNCH(ctx, radix_scatter_kernel<KW>, grid, dim3(SORT_THREADS), 0, ctx->stream, kin, rin, kout, rout, hist, \
-                 n, W, passes[p].word, passes[p].shift, tiles)
-        if (W == 1) SCATTER(1);
-        else if (W == 2 && aligned) SCATTER(2);
-        else if (W == 4 && aligned) SCATTER(4);
-        else SCATTER(0);
+        if (chained) {
+            const dim3 grid(static_cast<unsigned>(tiles) * T);
+            uint32_t* pass_state = state + static_cast<size_t>(p) * state_words;
+#define SCATTER(KW)                                                                                                  \
+    CULSH_LAUNCH(ctx, (radix_scatter_kernel<KW, true>), grid, dim3(SORT_THREADS), 0, ctx->stream, kin, rin, kout, rout, \
+                 static_cast<const uint32_t*>(nullptr), n, W, passes[p].word, passes[p].shift, tiles, T,              \
+                 static_cast<const uint32_t*>(pass_dtot), pass_state, err, spin_limit)
+            if (W == 1) SCATTER(1);
+            else if (W == 2 && aligned) SCATTER(2);
+            else if (W == 4 && aligned) SCATTER(4);
+            else SCATTER(0);
 #undef SCATTER
+        } else {
+            const dim3 grid(tiles, T);
+            CULSH_LAUNCH(ctx, radix_hist_kernel, grid, dim3(SORT_THREADS), 0, ctx->stream, kin, n, W,
+                         passes[p].word, passes[p].shift, tiles, hist, pass_dtot);
+            CULSH_LAUNCH_CHECK();
+            CULSH_LAUNCH(ctx, radix_scan_kernel, dim3(T, SCAN_PARTS), dim3(256), 0, ctx->stream, hist, pass_dtot, tiles);
+            CULSH_LAUNCH_CHECK();
+#define SCATTER(KW)                                                                                                   \
+    CULSH_LAUNCH(ctx, (radix_scatter_kernel<KW, false>), grid, dim3(SORT_THREADS), 0, ctx->stream, kin, rin, kout, rout, \
+                 static_cast<const uint32_t*>(hist), n, W, passes[p].word, passes[p].shift, tiles, T,                  \
+                 static_cast<const uint32_t*>(nullptr), static_cast<uint32_t*>(nullptr),                               \
+                 static_cast<uint32_t*>(nullptr), 0)
+            if (W == 1) SCATTER(1);
+            else if (W == 2 && aligned) SCATTER(2);
+            else if (W == 4 && aligned) SCATTER(4);
+            else SCATTER(0);
+#undef SCATTER
+        }
         CULSH_LAUNCH_CHECK();
         std::swap(kin, kout);
         rin = rout;

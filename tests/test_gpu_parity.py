@@ -141,6 +141,27 @@ def test_core_fit_index(ctx, kind, T, n, H):
     ctx.free_index(ih)
 
 
+@pytest.mark.parametrize("knob", ["CULSH_SORT_UNCHAINED=1", "CULSH_SORT_SPIN_LIMIT=0"])
+def test_core_fit_index_sort_fallbacks(ctx, c_oracle, monkeypatch, knob):
+    """The radix sort without the chained scan, and the repeat of a fit after the chained scan
+    gave up (forced by allowing no polls; every kernel still runs to its end)."""
+    _announce("sort_fallback", knob)
+    name, value = knob.split("=")
+    monkeypatch.setenv(name, value)
+    rng = np.random.default_rng(12)
+    T, n, H = 3, 70000, 2          # 18 tiles per table, two radix passes
+    sig = rng.integers(0, 256, size=(T, n, H), dtype=np.uint8)
+    from abi import Ctx, assert_index_matches
+
+    own = Ctx(0)                    # a give-up switches its context to unchained passes for good
+    try:
+        ih, _ = own.core_fit_index(sig, H)
+        assert_index_matches(own.index_arrays(ih), c_oracle.fit_index_c(sig, H).to_numpy(n))
+        own.free_index(ih)
+    finally:
+        own.close()
+
+
 def test_core_fit_index_single_bucket_per_table(ctx):
     """All signatures equal: no radix pass runs and rows stay in identity order."""
     sig = np.full((3, 1000, 4), 1, dtype=np.uint8)
