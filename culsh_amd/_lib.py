@@ -61,6 +61,7 @@ PROTOTYPES = {
     "culsh_ctx_synchronize": [_P],
     "culsh_profile_enable": [_P, _I],
     "culsh_profile_reset": [_P],
+    "culsh_profile_filter": [_P, C.c_char_p],
     "culsh_profile_get": [_P, _I, C.POINTER(C.c_char_p), C.POINTER(C.c_double), C.POINTER(C.c_int64)],
     "culsh_generate_projection_f32": [_U64, _I, _I, _P],
     "culsh_generate_projection_f64": [_U64, _I, _I, _P],

@@ -64,6 +64,7 @@ culsh_status arena_alloc(culsh_ctx* ctx, size_t bytes, void** out) {
 
 StageTimer::StageTimer(culsh_ctx* c, const char* name) : ctx(c) {
     if (!c->profiling) return;
+    if (!c->prof_filter.empty() && std::strstr(name, c->prof_filter.c_str()) == nullptr) return;
     int stage = -1;
     for (size_t i = 0; i < c->prof_stages.size(); ++i)
         if (c->prof_stages[i].name == name) { stage = static_cast<int>(i); break; }
@@ -247,6 +248,39 @@ static culsh_status upload(const T* host, size_t count, T** dev) {
     if (count == 0) return CULSH_OK;  // empty array -> nullptr (array_utils.cuh:34-36)
     CULSH_HIP(dev_malloc(dev, count * sizeof(T)));
     CULSH_HIP(hipMemcpy(*dev, host, count * sizeof(T), hipMemcpyHostToDevice));
+    return CULSH_OK;
+}
+
+// Hash parameters go through pinned staging and an asynchronous copy on the context's stream:
+// the kernels queued behind it see the data, and the host does not wait for the copy.
+template <typename T>
+static culsh_status upload_params(culsh_ctx* ctx, const T* host, size_t count, T** dev) {
+    *dev = nullptr;
+    if (count == 0) return CULSH_OK;
+    const size_t bytes = count * sizeof(T);
+    CULSH_HIP(dev_malloc(dev, bytes));
+    const size_t need = ctx->param_stage_off + align_up(bytes, 256);
+    if (need > ctx->param_stage_cap) {
+        if (ctx->param_stage_off != 0 || bytes > (size_t(64) << 20)) {  // staging in use or not worth pinning
+            CULSH_HIP(hipMemcpy(*dev, host, bytes, hipMemcpyHostToDevice));
+            return CULSH_OK;
+        }
+        if (ctx->param_stage) (void)hipHostFree(ctx->param_stage);
+        ctx->param_stage = nullptr;
+        ctx->param_stage_cap = 0;
+        const size_t cap = std::max<size_t>(size_t(1) << 20, 2 * align_up(bytes, 256));
+        if (hipHostMalloc(reinterpret_cast<void**>(&ctx->param_stage), cap, hipHostMallocDefault) != hipSuccess) {
+            (void)hipGetLastError();
+            ctx->param_stage = nullptr;
+            CULSH_HIP(hipMemcpy(*dev, host, bytes, hipMemcpyHostToDevice));
+            return CULSH_OK;
+        }
+        ctx->param_stage_cap = cap;
+    }
+    char* slot = ctx->param_stage + ctx->param_stage_off;
+    std::memcpy(slot, host, bytes);
+    ctx->param_stage_off += align_up(bytes, 256);
+    CULSH_HIP(hipMemcpyAsync(*dev, slot, bytes, hipMemcpyHostToDevice, ctx->stream));
     return CULSH_OK;
 }
 
@@ -445,23 +479,36 @@ static culsh_status dense_fit_once(culsh_ctx* ctx, Family fam, const T* X, int n
     ix->window_size = (fam == FAM_PSLSH) ? window : 0;
     const size_t TH = static_cast<size_t>(nT) * H;
     {
-        std::vector<T> hp, hb;
+        ctx->param_stage_off = 0;
         if (!P_host) {
-            hp.resize(TH * d);
-            gen_projection<T>(seed, TH * d, fam == FAM_PSLSH ? window : 0, hp.data());
-            P_host = hp.data();
-            if (fam == FAM_PSLSH) {
-                hb.resize(TH);
-                gen_bias<T>(seed, TH, hb.data());
-                b_host = hb.data();
+            culsh_ctx::GenCache& gc = ctx->gen_cache;
+            const int win = fam == FAM_PSLSH ? window : 0;
+            if (!(gc.family == static_cast<int>(fam) && gc.seed == seed && gc.rows == TH && gc.d == static_cast<size_t>(d) &&
+                  gc.window == win && gc.elem == static_cast<int>(sizeof(T)))) {
+                gc.family = -1;
+                gc.p.resize(TH * d * sizeof(T));
+                gen_projection<T>(seed, TH * d, win, reinterpret_cast<T*>(gc.p.data()));
+                gc.b.clear();
+                if (fam == FAM_PSLSH) {
+                    gc.b.resize(TH * sizeof(T));
+                    gen_bias<T>(seed, TH, reinterpret_cast<T*>(gc.b.data()));
+                }
+                gc.family = static_cast<int>(fam);
+                gc.seed = seed;
+                gc.rows = TH;
+                gc.d = static_cast<size_t>(d);
+                gc.window = win;
+                gc.elem = static_cast<int>(sizeof(T));
             }
+            P_host = reinterpret_cast<const T*>(gc.p.data());
+            if (fam == FAM_PSLSH) b_host = reinterpret_cast<const T*>(gc.b.data());
         }
         T* dP = nullptr;
-        CULSH_TRY(upload(P_host, TH * d, &dP));
+        CULSH_TRY(upload_params(ctx, P_host, TH * d, &dP));
         ix->P = dP;
         if (fam == FAM_PSLSH) {
             T* db = nullptr;
-            CULSH_TRY(upload(b_host, TH, &db));
+            CULSH_TRY(upload_params(ctx, b_host, TH, &db));
             ix->b = db;
         }
     }
@@ -498,16 +545,24 @@ static culsh_status minhash_fit_once(culsh_ctx* ctx, const int32_t* indices, con
     ix->kind = CULSH_KIND_MINHASH;
     const size_t TH = static_cast<size_t>(nT) * H;
     {
-        std::vector<uint32_t> ha, hb;
+        ctx->param_stage_off = 0;
         if (!A_host) {
-            ha.resize(TH);
-            hb.resize(TH);
-            gen_minhash(seed, TH, ha.data(), hb.data());
-            A_host = ha.data();
-            B_host = hb.data();
+            culsh_ctx::GenCache& gc = ctx->gen_cache;
+            constexpr int FAM_MINHASH_TAG = 100;
+            if (!(gc.family == FAM_MINHASH_TAG && gc.seed == seed && gc.rows == TH)) {
+                gc.family = -1;
+                gc.p.resize(TH * sizeof(uint32_t));
+                gc.b.resize(TH * sizeof(uint32_t));
+                gen_minhash(seed, TH, reinterpret_cast<uint32_t*>(gc.p.data()), reinterpret_cast<uint32_t*>(gc.b.data()));
+                gc.family = FAM_MINHASH_TAG;
+                gc.seed = seed;
+                gc.rows = TH;
+            }
+            A_host = reinterpret_cast<const uint32_t*>(gc.p.data());
+            B_host = reinterpret_cast<const uint32_t*>(gc.b.data());
         }
-        CULSH_TRY(upload(A_host, TH, &ix->A));
-        CULSH_TRY(upload(B_host, TH, &ix->B));
+        CULSH_TRY(upload_params(ctx, A_host, TH, &ix->A));
+        CULSH_TRY(upload_params(ctx, B_host, TH, &ix->B));
     }
     const size_t N = static_cast<size_t>(n) * nT;
     uint32_t* keys = nullptr;
@@ -649,6 +704,7 @@ void culsh_ctx_destroy(culsh_ctx* ctx) {
     for (void* p : ctx->overflow) (void)hipFree(p);
     if (ctx->arena) (void)hipFree(ctx->arena);
     if (ctx->pinned) (void)hipHostFree(ctx->pinned);
+    if (ctx->param_stage) (void)hipHostFree(ctx->param_stage);
     delete ctx;
 }
 
@@ -667,6 +723,11 @@ culsh_status culsh_profile_enable(culsh_ctx* ctx, int on) {
     CULSH_HIP(hipStreamSynchronize(ctx->stream));
     profile_collect(ctx);
     ctx->profiling = on != 0;
+    return CULSH_OK;
+}
+culsh_status culsh_profile_filter(culsh_ctx* ctx, const char* substring) {
+    CULSH_REQUIRE(ctx, CULSH_ERR_INVALID, "null argument");
+    ctx->prof_filter = substring ? substring : "";
     return CULSH_OK;
 }
 culsh_status culsh_profile_reset(culsh_ctx* ctx) {

@@ -85,6 +85,18 @@ struct culsh_ctx {
     size_t arena_want = 0;               // high-water mark incl. overflow blocks
     std::vector<void*> overflow;         // freed at the end of the call
     uint64_t* pinned = nullptr;          // 64 x u64 pinned host words for D2H scalars
+    // pinned staging for hash parameters on their way to the device (grown on demand); calls end
+    // with the stream idle, so a call may reuse it from the start
+    char* param_stage = nullptr;
+    size_t param_stage_cap = 0, param_stage_off = 0;
+    // the hash parameters last generated from a seed (a model that is fitted again with the same
+    // settings draws the same parameters; generating them on the host costs more than a fit)
+    struct GenCache {
+        int family = -1, window = 0, elem = 0;
+        uint64_t seed = 0;
+        size_t rows = 0, d = 0;
+        std::vector<char> p, b;  // P and b, or A and B
+    } gen_cache;
     // chained scan of the radix sort: give-up flag of the last sort (device, arena) and the
     // switch to the unchained passes after a give-up
     uint32_t* sort_err_dev = nullptr;
@@ -93,6 +105,7 @@ struct culsh_ctx {
     int n_cus = 0;
     // per-kernel timing with HIP events on `stream` (off unless enabled)
     bool profiling = false;
+    std::string prof_filter;             // when not empty: only kernels whose name contains it are timed
     struct ProfPending { int stage; hipEvent_t start, stop; };
     struct ProfStage { std::string name; double total_ms = 0.0; long launches = 0; };
     std::vector<ProfPending> prof_pending;

@@ -97,8 +97,12 @@ void* culsh_ctx_stream(culsh_ctx* ctx);
 /* ---- per-kernel timing ------------------------------------------------------------------
  * No counterpart in the reference (it has wall-clock timing only, cuda/benchmark/bench.cu:144-163).
  * When enabled, every kernel launch is bracketed by two HIP events on the context's stream;
- * totals per kernel name are available after the call that launched them has returned. */
+ * totals per kernel name are available after the call that launched them has returned.
+ * The events keep consecutive kernels about 10 us apart, so a caller that times whole calls
+ * restricts the timing to the kernel it needs with culsh_profile_filter (a substring of the
+ * kernel name; NULL or "" = every kernel). */
 culsh_status culsh_profile_enable(culsh_ctx* ctx, int on);
+culsh_status culsh_profile_filter(culsh_ctx* ctx, const char* substring);
 culsh_status culsh_profile_reset(culsh_ctx* ctx);
 int culsh_profile_count(const culsh_ctx* ctx);
 culsh_status culsh_profile_get(const culsh_ctx* ctx, int i, const char** name, double* total_ms, int64_t* launches);
