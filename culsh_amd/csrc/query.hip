@@ -149,6 +149,7 @@ struct DedupArgs {
     uint64_t* offsets;            // EMIT: per-query output offsets (read); FUSED: [n_queries+1] (written)
     unsigned long long* state;    // FUSED: [n_queries] published counts / running sums, zero before the launch
     unsigned int* err;            // FUSED: set when the look-back gave up or the output would overflow
+    unsigned int* ticket;         // FUSED: next query to hand out (workgroups stay and take queries in order)
     unsigned long long capacity;  // FUSED: elements available in `out`
     int T, n_queries;
     int wpt;       // bitmap words per thread (power of two); a pass covers DD_THREADS*wpt*32 rows
@@ -224,7 +225,8 @@ __global__ __launch_bounds__(DD_THREADS) void dedup_kernel(DedupArgs a) {
     const int chunk_words = DD_THREADS * a.wpt;                  // multiple of 1024
     uint32_t* bm = lds;                                          // [chunk_words]
     unsigned long long* sh_base = reinterpret_cast<unsigned long long*>(bm + chunk_words);  // [1]
-    int2* tab = reinterpret_cast<int2*>(sh_base + 1);            // [DD_THREADS]
+    int* sh_q = reinterpret_cast<int*>(sh_base + 1);             // [2] query handed to the workgroup
+    int2* tab = reinterpret_cast<int2*>(sh_base + 2);            // [DD_THREADS]
     int* s_start = reinterpret_cast<int*>(tab + DD_THREADS);     // [T]
     int* s_len = s_start + T;                                    // [T]
     uint32_t* s_ppref = reinterpret_cast<uint32_t*>(s_len + T);  // [T+1]
@@ -239,14 +241,28 @@ __global__ __launch_bounds__(DD_THREADS) void dedup_kernel(DedupArgs a) {
     }
     unsigned long long tick_ = a.ticks ? wall_clock64() : 0ull;
 
-    const int q = blockIdx.x;
-    uint32_t n_pieces;
-    {
-        int2 sp = make_int2(0, 0);
-        if (tid < T) sp = a.spans[static_cast<size_t>(q) * T + tid];
-        // the first pass's bitmap is cleared while that load is in flight
+    // COUNT, EMIT: one workgroup per query.  FUSED: workgroups stay resident and take queries in
+    // order from a ticket counter, so a query's predecessors in the chained scan have always been
+    // taken by a running workgroup; the next ticket and its spans are fetched under the current
+    // query's read-out.
+    int q = blockIdx.x;
+    if (MODE == DD_FUSED && tid == 0) *sh_q = static_cast<int>(atomicAdd(a.ticket, 1u));
+    {   // the bitmap is cleared while the first loads are in flight; FUSED keeps it clean afterwards
         uint4* bm4 = reinterpret_cast<uint4*>(bm);
         for (int i = tid; i < chunk_words / 4; i += DD_THREADS) bm4[i] = make_uint4(0u, 0u, 0u, 0u);
+    }
+    if (MODE == DD_FUSED) {
+        __syncthreads();
+        q = *sh_q;
+        if (q >= a.n_queries) return;
+    }
+    int2 sp = make_int2(0, 0);
+    if (tid < T) sp = a.spans[static_cast<size_t>(q) * T + tid];
+  for (;;) {  // the queries of this workgroup (a single one unless FUSED)
+    int q_next = a.n_queries;
+    int2 sp_next = make_int2(0, 0);
+    uint32_t n_pieces;
+    {
         if (tid < T) {
             s_start[tid] = sp.x;
             s_len[tid] = sp.y;
@@ -325,9 +341,13 @@ __global__ __launch_bounds__(DD_THREADS) void dedup_kernel(DedupArgs a) {
         }
         // FUSED: the first wavefront publishes the count before anything else, so that later
         // queries can go on, and looks back only after lining up its own rows.
-        if (MODE == DD_FUSED && wave == 0 && lane == 0)
+        DD_TICK(4)
+        unsigned int ticket_next = 0;
+        if (MODE == DD_FUSED && wave == 0 && lane == 0) {
             __hip_atomic_store(&a.state[q], TAG_COUNT | static_cast<unsigned long long>(chunk_total), __ATOMIC_RELAXED,
                                __HIP_MEMORY_SCOPE_AGENT);
+            ticket_next = atomicAdd(a.ticket, 1u);  // arrives while the rows are lined up
+        }
         // Line-up.  A step's words go to registers, which frees its part of the bitmap: the rows are
         // written there in list order, ready for full-width wavefront stores.  No step needs the
         // position of the query's list for this.  A dense step (more rows than slots) is left alone.
@@ -359,12 +379,17 @@ __global__ __launch_bounds__(DD_THREADS) void dedup_kernel(DedupArgs a) {
                 }
             }
         }
+        DD_TICK(5)
         uint64_t base = out_base + running;
         bool store = true;
         if (MODE == DD_FUSED) {
             if (wave == 0) {
+                const int qn = min(static_cast<int>(__shfl(ticket_next, 0, 64)), a.n_queries);
+                // spans of the next query (they all sit in this wavefront when T <= 64)
+                if (T <= 64 && qn < a.n_queries && lane < T) sp_next = a.spans[static_cast<size_t>(qn) * T + lane];
                 const unsigned long long excl = look_back(a.state, q, chunk_total, a.spin_limit, a.err);
                 if (lane == 0) {
+                    *sh_q = qn;
                     unsigned long long b = excl;
                     if (excl + chunk_total > a.capacity) {  // cannot happen with capacity = raw candidates
                         atomicOr(a.err, 2u);
@@ -376,9 +401,11 @@ __global__ __launch_bounds__(DD_THREADS) void dedup_kernel(DedupArgs a) {
                     if (q == a.n_queries - 1) a.offsets[a.n_queries] = excl + chunk_total;
                 }
             }
+            DD_TICK(6)
             __syncthreads();
             base = *sh_base;
             store = base != ~0ull;
+            q_next = *sh_q;
         }
         DD_TICK(2)  // count, line-up (+ look-back)
         if (store) {
@@ -412,11 +439,24 @@ __global__ __launch_bounds__(DD_THREADS) void dedup_kernel(DedupArgs a) {
                 dst += st_total[j];
             }
         }
+        if (MODE == DD_FUSED) {  // leave this wavefront's part of the bitmap clean for the next query
+            uint4* z = reinterpret_cast<uint4*>(wbm);
+            for (int i = lane; i < wpw / 4; i += 64) z[i] = make_uint4(0u, 0u, 0u, 0u);
+        }
         running += chunk_total;
         __syncthreads();  // bitmap and wtot are rewritten by the next pass
         DD_TICK(3)  // ordered store
     }
     if (MODE == DD_COUNT && tid == 0) a.counts[q] = running;
+    if (MODE != DD_FUSED || q_next >= a.n_queries) break;
+    q = q_next;
+    if (T <= 64) {
+        sp = sp_next;  // zero outside the first T lanes
+    } else {
+        sp = make_int2(0, 0);
+        if (tid < T) sp = a.spans[static_cast<size_t>(q) * T + tid];
+    }
+  }
 #undef DD_TICK
 }
 
@@ -452,7 +492,7 @@ culsh_status query_from_spans(culsh_ctx* ctx, const int2* spans, const unsigned 
     // Geometry of a pass: DD_THREADS * wpt bitmap words, wpt a power of two.  Debug knobs:
     // CULSH_DEDUP_WPT lowers the cap on wpt (more passes), CULSH_DEDUP_TWO_PASS=1 forces the
     // count / scan / emit path, CULSH_DEDUP_TRACE=1 prints phase timers.
-    const size_t fixed = (2 + static_cast<size_t>(3 * T) + 1 + 2 * DD_THREADS + 17 + (NWAVES + 1) + 8) * sizeof(uint32_t);
+    const size_t fixed = (4 + static_cast<size_t>(3 * T) + 1 + 2 * DD_THREADS + 17 + (NWAVES + 1) + 8) * sizeof(uint32_t);
     auto lds_need = [&](int w) { return static_cast<size_t>(DD_THREADS) * w * 4 + fixed; };
     int wpt_max = 1;
     const int wpt_limit = std::max(1, std::min(32, env_int("CULSH_DEDUP_WPT", 32)));
@@ -482,6 +522,7 @@ culsh_status query_from_spans(culsh_ctx* ctx, const int2* spans, const unsigned 
     a.offsets = out->query_candidate_offsets;
     a.state = nullptr;
     a.err = nullptr;
+    a.ticket = nullptr;
     a.capacity = 0;
     a.T = T;
     a.n_queries = n_queries;
@@ -506,16 +547,21 @@ culsh_status query_from_spans(culsh_ctx* ctx, const int2* spans, const unsigned 
         const uint64_t cap = std::min<uint64_t>(R, static_cast<uint64_t>(n_queries) * static_cast<uint64_t>(n));
         unsigned int* err = nullptr;
         CULSH_TRY(arena_alloc_t(ctx, static_cast<size_t>(n_queries), &a.state));
-        CULSH_TRY(arena_alloc_t(ctx, 1, &err));
+        CULSH_TRY(arena_alloc_t(ctx, 2, &err));  // [0] error flags, [1] ticket counter
         CULSH_HIP(hipMemsetAsync(a.state, 0, static_cast<size_t>(n_queries) * sizeof(unsigned long long), ctx->stream));
-        CULSH_HIP(hipMemsetAsync(err, 0, sizeof(unsigned int), ctx->stream));
+        CULSH_HIP(hipMemsetAsync(err, 0, 2 * sizeof(unsigned int), ctx->stream));
+        a.ticket = err + 1;
         CULSH_HIP(dev_malloc(&out->query_candidate_indices, cap * sizeof(int32_t)));
         a.out = out->query_candidate_indices;
         a.err = err;
         a.capacity = cap;
         CULSH_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(dedup_kernel<DD_FUSED>),
                                       hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes)));
-        CULSH_LAUNCH(ctx, dedup_kernel<DD_FUSED>, dim3(n_queries), dim3(DD_THREADS), lds_bytes, ctx->stream, a);
+        // as many workgroups as fit on the device at once (LDS and 2048 threads per CU bound it)
+        const int per_cu = static_cast<int>(std::max<size_t>(1, std::min<size_t>(2, static_cast<size_t>(ctx->lds_max) / lds_bytes)));
+        const int resident = std::max(1, ctx->n_cus * per_cu);
+        CULSH_LAUNCH(ctx, dedup_kernel<DD_FUSED>, dim3(std::min(n_queries, resident)), dim3(DD_THREADS), lds_bytes,
+                     ctx->stream, a);
         CULSH_LAUNCH_CHECK();
         CULSH_HIP(hipMemcpyAsync(&ctx->pinned[0], out->query_candidate_offsets + n_queries, sizeof(uint64_t),
                                  hipMemcpyDeviceToHost, ctx->stream));
@@ -566,9 +612,10 @@ culsh_status query_from_spans(culsh_ctx* ctx, const int2* spans, const unsigned 
         CULSH_HIP(hipMemcpy(all.data(), ticks_dev, all.size() * sizeof(uint64_t), hipMemcpyDeviceToHost));
         uint64_t tk[8] = {0, 0, 0, 0, 0, 0, 0, 0};
         for (size_t i = 0; i < all.size(); ++i) tk[i & 7] += all[i];
-        fprintf(stderr, "[dedup trace] wpt=%d chunks=%d fused=%d | setup %llu gather %llu count %llu store %llu (ticks)\n",
+        fprintf(stderr, "[dedup trace] wpt=%d chunks=%d fused=%d | setup %llu gather %llu count %llu store %llu (ticks) | popc %llu line-up %llu look-back %llu barrier %llu\n",
                 wpt, n_chunks, int(fused), (unsigned long long)tk[0], (unsigned long long)tk[1],
-                (unsigned long long)tk[2], (unsigned long long)tk[3]);
+                (unsigned long long)tk[2], (unsigned long long)tk[3], (unsigned long long)tk[4],
+                (unsigned long long)tk[5], (unsigned long long)tk[6], (unsigned long long)tk[2]);
     }
     return CULSH_OK;
 }
