@@ -312,10 +312,7 @@ static culsh_status hash_dense_to_keys(culsh_ctx* ctx, Family fam, const T* X, i
         if constexpr (std::is_same_v<T, float>) {
             CULSH_TRY(launch_project_f32(ctx, X, static_cast<const float*>(P), nullptr, rows, d, nT, H, EPI_SIGN_KEYS, keys));
         } else {
-            uint8_t* sig = nullptr;
-            CULSH_TRY(arena_alloc_t(ctx, N * H, &sig));
-            CULSH_TRY(launch_project_f64(ctx, X, static_cast<const double*>(P), nullptr, rows, d, nT, H, EPI_SIGN_BYTES, sig));
-            CULSH_TRY(launch_sig_to_keys(ctx, sig, N, H, ENC_BITS, W, keys));
+            CULSH_TRY(launch_project_f64(ctx, X, static_cast<const double*>(P), nullptr, rows, d, nT, H, EPI_SIGN_KEYS, keys));
         }
         *keys_out = keys;
         *W_out = W;

@@ -275,56 +275,211 @@ __global__ __launch_bounds__(NTHREADS) void project_f32_kernel(ProjArgs a) {
     }
 }
 
-// ---------------------------------------------------------------- fp64 (plain FMA tiles)
-constexpr int DT = 64;   // tile edge
-constexpr int DK = 16;   // features per stage
+// ---------------------------------------------------------------- fp64 (MFMA 16x16x4 tiles)
+// Same tiling as the fp32 kernel: 128 x 128 outputs per workgroup, 2 x 2 wavefronts of 64 x 64,
+// here as 4 x 4 MFMA tiles of 16 x 16 x 4.  Operand lane l supplies A[row l%16][k l/16] and
+// B[k l/16][col l%16]; the four lane groups walk four consecutive features each per stage
+// pair, so fragments are 16-byte LDS reads.  Accumulator register i of lane l holds
+// row 4*i + l/16, column l%16 of its tile.
+typedef double f64x4 __attribute__((ext_vector_type(4)));
 
-template <int EPI>
-__global__ __launch_bounds__(256) void project_f64_kernel(const double* __restrict__ X,
-                                                         const double* __restrict__ P,
-                                                         const double* __restrict__ b, void* out,
-                                                         int n, int d, int T, int H) {
-    __shared__ double Xs[DK][DT + 1];
-    __shared__ double Ps[DK][DT + 1];
-    const int tx = threadIdx.x & 15, ty = threadIdx.x >> 4;
-    const int row0 = blockIdx.x * DT, col0 = blockIdx.y * DT;
+struct ProjArgs64 {
+    const double* X;
+    const double* P;
+    const double* b;
+    void* out;
+    int n, d, T, H;
+    int n_row_tiles, n_col_tiles;
+};
+
+constexpr int DBK = 16;  // features per stage
+
+template <int EPI, bool VEC>
+__global__ __launch_bounds__(NTHREADS, 2) void project_f64_kernel(ProjArgs64 a) {
+    constexpr int PITCH = DBK + 2;  // LDS row pitch in doubles
+    constexpr int D2 = DBK / 2;     // double2 per tile row and stage
+    constexpr int NLD = BM * D2 / NTHREADS;
+    constexpr int RSTEP = NTHREADS / D2;
+    __shared__ __attribute__((aligned(16))) double As[BM * PITCH];
+    __shared__ __attribute__((aligned(16))) double Bs[BN * PITCH];
+    __shared__ uint32_t tw[(EPI == EPI_SIGN_KEYS) ? BM * (BN / 32) : 1];
+
+    // same workgroup -> (row tile, column tile) arrangement as the fp32 kernel
+    const int nct = a.n_col_tiles;
+    const int per_group = 8 * nct;
+    const int grp = blockIdx.x / per_group, rem = blockIdx.x - grp * per_group;
+    const int ct = rem >> 3, slot = rem & 7;
+    const int rt = grp * 8 + slot;
+    if (rt >= a.n_row_tiles) return;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int r16 = lane & 15, g = lane >> 4;
+    const int n = a.n, d = a.d, T = a.T, H = a.H;
     const int TH = T * H;
-    double acc[4][4] = {};
-    for (int k0 = 0; k0 < d; k0 += DK) {
-        for (int idx = threadIdx.x; idx < DT * DK; idx += 256) {
-            const int r = idx / DK, k = idx - r * DK;
-            const int gr = row0 + r, gc = col0 + r, gk = k0 + k;
-            Xs[k][r] = (gr < n && gk < d) ? X[static_cast<size_t>(gr) * d + gk] : 0.0;
-            Ps[k][r] = (gc < TH && gk < d) ? P[static_cast<size_t>(gc) * d + gk] : 0.0;
-        }
-        __syncthreads();
+
+    const int lrow = tid / D2, c2 = (tid % D2) * 2;
+    const double* xbase = a.X + static_cast<size_t>(rt) * BM * d;
+    uint32_t xoff[NLD], poff[NLD];
+    bool xok[NLD], pok[NLD];
 #pragma unroll
-        for (int k = 0; k < DK; ++k) {
-            double xa[4], pb[4];
-#pragma unroll
-            for (int i = 0; i < 4; ++i) { xa[i] = Xs[k][ty + 16 * i]; pb[i] = Ps[k][tx + 16 * i]; }
-#pragma unroll
-            for (int i = 0; i < 4; ++i)
-#pragma unroll
-                for (int j = 0; j < 4; ++j) acc[i][j] = fma(xa[i], pb[j], acc[i][j]);
-        }
-        __syncthreads();
+    for (int i = 0; i < NLD; ++i) {
+        const int lr = lrow + RSTEP * i;
+        xok[i] = rt * BM + lr < n;
+        xoff[i] = static_cast<uint32_t>(VEC ? min(lr, n - 1 - rt * BM) : lr) * static_cast<uint32_t>(d);
+        const int vc = ct * BN + lr;
+        const int prow = (EPI == EPI_SIGN_KEYS) ? sign_vcol_to_prow(vc, T, H) : (vc < TH ? vc : -1);
+        pok[i] = prow >= 0;
+        poff[i] = static_cast<uint32_t>(prow < 0 ? 0 : prow) * static_cast<uint32_t>(d);
     }
+    auto fetch = [&](int k, double2 (&ra)[NLD], double2 (&rb)[NLD]) {
+        if (VEC) {
+            const int kk = min(k, d - 2);
+            const bool inside = k < d;  // a double2 is entirely inside or entirely outside [0, d)
+#pragma unroll
+            for (int i = 0; i < NLD; ++i) {
+                const double2 va = *reinterpret_cast<const double2*>(xbase + (xoff[i] + static_cast<uint32_t>(kk)));
+                const double2 vb = *reinterpret_cast<const double2*>(a.P + (poff[i] + static_cast<uint32_t>(kk)));
+                ra[i] = inside ? make_double2(va.x, va.y) : make_double2(0.0, 0.0);
+                rb[i] = inside ? make_double2(vb.x, vb.y) : make_double2(0.0, 0.0);
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < NLD; ++i) {
+                double2 va = make_double2(0.0, 0.0), vb = make_double2(0.0, 0.0);
+                if (xok[i]) {
+                    if (k < d) va.x = xbase[xoff[i] + k];
+                    if (k + 1 < d) va.y = xbase[xoff[i] + k + 1];
+                }
+                if (pok[i]) {
+                    if (k < d) vb.x = a.P[poff[i] + k];
+                    if (k + 1 < d) vb.y = a.P[poff[i] + k + 1];
+                }
+                ra[i] = va;
+                rb[i] = vb;
+            }
+        }
+    };
+
+    f64x4 acc[4][4];
 #pragma unroll
     for (int i = 0; i < 4; ++i)
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const int row = row0 + ty + 16 * i, col = col0 + tx + 16 * j;
-            if (row >= n || col >= TH) continue;
-            const int t = col / H, h = col - t * H;
-            const size_t off = (static_cast<size_t>(t) * n + row) * H + h;
-            if (EPI == EPI_SIGN_BYTES) {
-                // narrowing to float keeps the sign (rplsh/hash.cuh:47)
-                static_cast<uint8_t*>(out)[off] = (__double_as_longlong(acc[i][j]) < 0) ? 0 : 1;
-            } else {
-                static_cast<int32_t*>(out)[off] = static_cast<int32_t>(floor(acc[i][j] + b[col]));
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int v = 0; v < 4; ++v) acc[i][j][v] = 0.0;
+
+    double2 ra[NLD], rb[NLD];
+    fetch(c2, ra, rb);
+    const int nk = (d + DBK - 1) / DBK;
+    for (int kt = 0; kt < nk; ++kt) {
+#pragma unroll
+        for (int i = 0; i < NLD; ++i) {
+            *reinterpret_cast<double2*>(&As[(lrow + RSTEP * i) * PITCH + c2]) = ra[i];
+            *reinterpret_cast<double2*>(&Bs[(lrow + RSTEP * i) * PITCH + c2]) = rb[i];
+        }
+        __syncthreads();
+        if (kt + 1 < nk) fetch((kt + 1) * DBK + c2, ra, rb);
+        // lane group g walks features 4g .. 4g+3 of the stage, two at a time
+#pragma unroll
+        for (int kk = 0; kk < 4; kk += 2) {
+            double2 af[4], bf[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                af[i] = *reinterpret_cast<const double2*>(&As[(wm * 64 + i * 16 + r16) * PITCH + g * 4 + kk]);
+                bf[i] = *reinterpret_cast<const double2*>(&Bs[(wn * 64 + i * 16 + r16) * PITCH + g * 4 + kk]);
+            }
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    acc[i][j] = __builtin_amdgcn_mfma_f64_16x16x4f64(af[i].x, bf[j].x, acc[i][j], 0, 0, 0);
+                    acc[i][j] = __builtin_amdgcn_mfma_f64_16x16x4f64(af[i].y, bf[j].y, acc[i][j], 0, 0, 0);
+                }
+        }
+        __syncthreads();
+    }
+
+    if (EPI == EPI_SIGN_KEYS) {
+#pragma unroll
+        for (int ti = 0; ti < 4; ++ti)
+#pragma unroll
+            for (int cp = 0; cp < 2; ++cp) {
+                int mine = 0;
+#pragma unroll
+                for (int v = 0; v < 4; ++v) {
+                    // hash bit = 1 iff the sign bit is clear (rplsh/hash.cuh:47; narrowing to float keeps it)
+                    const unsigned long long b0 =
+                        __builtin_amdgcn_ballot_w64(__double_as_longlong(acc[ti][2 * cp][v]) >= 0);
+                    const unsigned long long b1 =
+                        __builtin_amdgcn_ballot_w64(__double_as_longlong(acc[ti][2 * cp + 1][v]) >= 0);
+#pragma unroll
+                    for (int gg = 0; gg < 4; ++gg) {
+                        // lanes 16gg..16gg+15 of a ballot are columns 0..15 of row 4v + gg
+                        const uint32_t word = static_cast<uint32_t>((b0 >> (16 * gg)) & 0xFFFFull) |
+                                              (static_cast<uint32_t>((b1 >> (16 * gg)) & 0xFFFFull) << 16);
+                        asm("s_nop 1\n\tv_writelane_b32 %0, %1, %2" : "+v"(mine) : "s"(word), "n"(4 * v + gg));
+                    }
+                }
+                if (lane < 16) tw[(wm * 64 + ti * 16 + lane) * (BN / 32) + (wn * 2 + cp)] = static_cast<uint32_t>(mine);
+            }
+        __syncthreads();
+        uint32_t* keys = static_cast<uint32_t*>(a.out);
+        if (H <= 32) {
+            const int tpt = 32 / H;
+            const uint32_t mask = (H == 32) ? 0xFFFFFFFFu : ((1u << H) - 1u);
+            constexpr int TL_STEP = NTHREADS / BM;
+            const int row = tid % BM, grow = rt * BM + row;
+            int tl = tid / BM;
+            int tc = tl / tpt, sub = tl - tc * tpt;
+            for (; tl < (BN / 32) * tpt; tl += TL_STEP) {
+                const int table = (ct * (BN / 32) + tc) * tpt + sub;
+                if (table < T && grow < n) {
+                    const uint32_t field = (tw[row * (BN / 32) + tc] >> (sub * H)) & mask;
+                    keys[static_cast<size_t>(table) * n + grow] = field << (32 - H);
+                }
+                sub += TL_STEP;
+                while (sub >= tpt) { sub -= tpt; ++tc; }
+            }
+        } else {
+            const int wt = (H + 31) >> 5;
+            for (int idx = tid; idx < (BN / 32) * BM; idx += NTHREADS) {
+                const int tc = idx / BM, row = idx - tc * BM;
+                const int tile = ct * (BN / 32) + tc;
+                const int table = tile / wt, w = tile - table * wt;
+                const int grow = rt * BM + row;
+                if (table < T && grow < n) {
+                    const int nbits = min(32, H - 32 * w);
+                    const uint32_t mask = (nbits == 32) ? 0xFFFFFFFFu : (0xFFFFFFFFu << (32 - nbits));
+                    keys[(static_cast<size_t>(table) * n + grow) * wt + w] = tw[row * (BN / 32) + tc] & mask;
+                }
             }
         }
+    } else {
+#pragma unroll
+        for (int ti = 0; ti < 4; ++ti)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int col = ct * BN + wn * 64 + j * 16 + r16;
+                if (col >= TH) continue;
+                const int t = col / H, h = col - t * H;
+                const double bias = (EPI == EPI_FLOOR_I32) ? a.b[col] : 0.0;
+#pragma unroll
+                for (int v = 0; v < 4; ++v) {
+                    const int row = rt * BM + wm * 64 + ti * 16 + 4 * v + g;
+                    if (row >= n) continue;
+                    const size_t off = (static_cast<size_t>(t) * n + row) * H + h;
+                    const double x = acc[ti][j][v];
+                    if (EPI == EPI_SIGN_BYTES) {
+                        // narrowing to float keeps the sign (rplsh/hash.cuh:47)
+                        static_cast<uint8_t*>(a.out)[off] = (__double_as_longlong(x) < 0) ? 0 : 1;
+                    } else {
+                        static_cast<int32_t*>(a.out)[off] = static_cast<int32_t>(floor(x + bias));
+                    }
+                }
+            }
+    }
 }
 
 }  // namespace
@@ -378,17 +533,39 @@ culsh_status launch_project_f64(culsh_ctx* ctx, const double* X, const double* P
                                 int n, int d, int T, int H, ProjEpilogue epi, void* out) {
     CULSH_REQUIRE(X && P && out, CULSH_ERR_INVALID, "projection: null pointer");
     CULSH_REQUIRE(n > 0 && d > 0 && T > 0 && H > 0, CULSH_ERR_INVALID, "projection: sizes must be positive");
-    CULSH_REQUIRE(epi == EPI_SIGN_BYTES || epi == EPI_FLOOR_I32, CULSH_ERR_INTERNAL,
-                  "fp64 projection writes the reference layout only");
     CULSH_REQUIRE(epi != EPI_FLOOR_I32 || b, CULSH_ERR_INVALID, "projection: bias is required");
-    const long long TH = static_cast<long long>(T) * H;
-    const long long gy = (TH + DT - 1) / DT;
-    CULSH_REQUIRE(gy <= 65535, CULSH_ERR_LIMIT, "T*H too large for the fp64 projection grid");
-    dim3 grid((n + DT - 1) / DT, static_cast<unsigned>(gy)), block(256);
-    if (epi == EPI_SIGN_BYTES)
-        CULSH_LAUNCH(ctx, project_f64_kernel<EPI_SIGN_BYTES>, grid, block, 0, ctx->stream, X, P, b, out, n, d, T, H);
-    else
-        CULSH_LAUNCH(ctx, project_f64_kernel<EPI_FLOOR_I32>, grid, block, 0, ctx->stream, X, P, b, out, n, d, T, H);
+    CULSH_REQUIRE(static_cast<long long>(T) * H < (1ll << 30), CULSH_ERR_LIMIT, "T*H too large");
+    CULSH_REQUIRE(static_cast<long long>(T) * H * d < (1ll << 32) && static_cast<long long>(BM) * d < (1ll << 31),
+                  CULSH_ERR_LIMIT, "projection: T*H*n_features must be below 2^32");
+    long long n_vcols;
+    if (epi == EPI_SIGN_KEYS) {
+        const long long tiles = (H <= 32) ? (T + (32 / H) - 1) / (32 / H)
+                                          : static_cast<long long>(T) * ((H + 31) / 32);
+        n_vcols = tiles * 32;
+    } else {
+        n_vcols = static_cast<long long>(T) * H;
+    }
+    ProjArgs64 a;
+    a.X = X; a.P = P; a.b = b; a.out = out;
+    a.n = n; a.d = d; a.T = T; a.H = H;
+    a.n_row_tiles = (n + BM - 1) / BM;
+    a.n_col_tiles = static_cast<int>((n_vcols + BN - 1) / BN);
+    const bool vec = (d % 2 == 0) && (reinterpret_cast<uintptr_t>(X) % 16 == 0) && (reinterpret_cast<uintptr_t>(P) % 16 == 0);
+    const long long groups = (a.n_row_tiles + 7) / 8;
+    const long long blocks = groups * 8 * a.n_col_tiles;
+    CULSH_REQUIRE(blocks < (1ll << 31), CULSH_ERR_LIMIT, "projection grid too large");
+    dim3 grid(static_cast<unsigned>(blocks)), block(NTHREADS);
+#define PROJ_CASE64(E)                                                                                  \
+    case E:                                                                                             \
+        if (vec) CULSH_LAUNCH(ctx, (project_f64_kernel<E, true>), grid, block, 0, ctx->stream, a);      \
+        else CULSH_LAUNCH(ctx, (project_f64_kernel<E, false>), grid, block, 0, ctx->stream, a);         \
+        break;
+    switch (epi) {
+        PROJ_CASE64(EPI_SIGN_KEYS)
+        PROJ_CASE64(EPI_SIGN_BYTES)
+        PROJ_CASE64(EPI_FLOOR_I32)
+    }
+#undef PROJ_CASE64
     CULSH_LAUNCH_CHECK();
     return CULSH_OK;
 }
