@@ -522,3 +522,66 @@ def test_object_memory_is_reused_and_trimmed(ctx):
         ctx.free_index(ih)
         if round_ == 1:
             ctx.lib.culsh_memory_trim()
+
+
+def test_full_size_invariants(ctx):
+    """BASELINE config 2 at its real size (1M x 128, 32 tables x 16 hashes, 10k queries): properties
+    that hold for any correct index / candidate set, checked on everything, plus a brute-force
+    comparison for a sample of queries."""
+    _announce("full_size")
+    n, d, nq, T, H = 1_000_000, 128, 10_000, 32, 16
+    rng = np.random.default_rng(2024)
+    X = np.clip(np.floor(rng.gamma(0.5, 30.0, size=(n, d))), 0, 255).astype(np.float32)
+    rows = rng.integers(0, n, size=nq)
+    Q = np.clip(X[rows] + rng.normal(0.0, 3.0, size=(nq, d)), 0, 255).astype(np.float32)
+    P = rng.standard_normal((T * H, d)).astype(np.float32)
+    ih = ctx.rplsh_fit(X, T, H, P=P)
+    ix = ctx.index_arrays(ih)
+    N = n * T
+    tbo, bco = ix["table_bucket_offsets"].astype(np.int64), ix["bucket_candidate_offsets"].astype(np.int64)
+    B = int(ix["n_total_buckets"])
+    cand = ix["all_candidate_indices"]
+    assert tbo[0] == 0 and tbo[-1] == B and np.all(np.diff(tbo) > 0)
+    assert bco[0] == 0 and bco[-1] == N and np.all(np.diff(bco) > 0)
+    assert np.all(bco[tbo[:-1]] == np.arange(T) * n)            # a table's first bucket starts its segment
+    # every table holds every row exactly once
+    for t in range(T):
+        assert np.array_equal(np.bincount(cand[t * n:(t + 1) * n], minlength=n), np.ones(n, dtype=np.int64))
+    # rows ascend inside a bucket: the only descents of the candidate array are at bucket starts
+    descents = np.flatnonzero(np.diff(cand.astype(np.int64)) < 0) + 1
+    assert np.all(np.isin(descents, bco))
+    # bucket signatures strictly ascend (byte order) inside a table
+    sig = ix["all_bucket_signatures"].reshape(B, H)
+    keys = sig.astype(np.int64) @ (1 << np.arange(H - 1, -1, -1)).astype(np.int64)   # H = 16 sign bytes as a number
+    inc = np.diff(keys) > 0
+    inc[tbo[1:-1] - 1] = True                                    # table boundaries may descend
+    assert np.all(inc)
+    # signatures agree with the GPU's own hash of the rows they contain (first row of a sample of buckets)
+    gsig = ctx.rplsh_hash(X[:20000], P, T, H)                    # [T][20000][H]
+    bucket_of_pos = np.searchsorted(bco, np.arange(0, N, 997), side="right") - 1
+    for pos, b in zip(np.arange(0, N, 997)[:4000], bucket_of_pos[:4000]):
+        r, t = int(cand[pos]), int(pos // n)
+        if r < 20000:
+            assert np.array_equal(sig[b], gsig[t, r])
+    # queries
+    got = ctx.rplsh_query(Q, ih)
+    off, idx = got["offsets"].astype(np.int64), got["indices"]
+    assert off[0] == 0 and off[-1] == len(idx) and np.all(np.diff(off) >= 0)
+    assert np.array_equal(np.diff(off), got["counts"].astype(np.int64))
+    inside = np.ones(len(idx), dtype=bool)
+    inside[off[1:-1][off[1:-1] < len(idx)]] = False              # first element of the next query
+    assert np.all((np.diff(idx.astype(np.int64)) > 0) | ~inside[1:])   # ascending and duplicate-free per query
+    assert idx.min() >= 0 and idx.max() < n
+    # brute force for a sample: union over tables of the rows in the bucket that matches the query's signature
+    qsig = ctx.rplsh_hash(Q[:64], P, T, H)
+    for q in range(0, 64, 7):
+        exp = []
+        for t in range(T):
+            lo, hi = tbo[t], tbo[t + 1]
+            hit = np.flatnonzero((sig[lo:hi] == qsig[t, q]).all(axis=1))
+            if len(hit):
+                b = lo + hit[0]
+                exp.append(cand[bco[b]:bco[b + 1]])
+        exp = np.unique(np.concatenate(exp)) if exp else np.zeros(0, np.int32)
+        np.testing.assert_array_equal(idx[off[q]:off[q + 1]], exp)
+    ctx.free_index(ih)
