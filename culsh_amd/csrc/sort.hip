@@ -236,13 +236,19 @@ __global__ __launch_bounds__(SORT_THREADS) void radix_scatter_kernel(
         if (ONE_WORD) rw[j] = (valid && rows_in) ? rows_in[tbase + idx] : idx;
         const uint32_t d = (k >> shift) & 255u;
         // lanes holding the same digit
-        unsigned long long peers = __builtin_amdgcn_ballot_w64(valid);
+        const unsigned long long live = __builtin_amdgcn_ballot_w64(valid);
+        uint32_t peers_lo = static_cast<uint32_t>(live), peers_hi = static_cast<uint32_t>(live >> 32);
 #pragma unroll
         for (int b = 0; b < 8; ++b) {
-            const bool bit = (d >> b) & 1u;
-            const unsigned long long m = __builtin_amdgcn_ballot_w64(bit);
-            peers &= bit ? m : ~m;
+            // x = all ones if bit b of the digit is set, else zero; lanes agreeing with this one
+            // on that bit are m where x is ones and ~m where x is zero, i.e. ~(m ^ x)
+            const int xs = __builtin_amdgcn_sbfe(static_cast<int>(d), b, 1);  // sign-extended bit b
+            const uint32_t x = static_cast<uint32_t>(xs);
+            const unsigned long long m = __builtin_amdgcn_ballot_w64(xs != 0);
+            peers_lo &= ~(static_cast<uint32_t>(m) ^ x);
+            peers_hi &= ~(static_cast<uint32_t>(m >> 32) ^ x);
         }
+        const unsigned long long peers = (static_cast<unsigned long long>(peers_hi) << 32) | peers_lo;
         uint32_t old = 0;
         int leader = lane;
         if (valid) {
