@@ -528,7 +528,7 @@ culsh_status query_from_spans(culsh_ctx* ctx, const int2* spans, const unsigned 
     a.n_queries = n_queries;
     a.wpt = wpt;
     a.n_chunks = n_chunks;
-    a.spin_limit = 1 << 16;
+    a.spin_limit = env_int("CULSH_DEDUP_SPIN_LIMIT", 1 << 16);  // tests set 0 to reach the give-up path
     a.ticks = ticks_dev;
 
     bool fused = n_chunks == 1 && env_int("CULSH_DEDUP_TWO_PASS", 0) == 0;

@@ -269,6 +269,36 @@ def test_core_query_two_launch_path(ctx, monkeypatch):
     ctx.free_index(ih)
 
 
+def test_core_query_after_look_back_gives_up(ctx, monkeypatch):
+    """No polls allowed in the chained scan over the query counts: some workgroup gives up, the
+    kernel still runs to its end, and the call is redone with the count / scan / emit launches."""
+    _announce("dedup_give_up")
+    monkeypatch.setenv("CULSH_DEDUP_SPIN_LIMIT", "0")
+    rng = np.random.default_rng(5)
+    T, n, nq, H = 6, 5000, 3000, 2
+    sig = random_sigs(rng, T, n, H, "rplsh")
+    qsig = random_sigs(rng, T, nq, H, "rplsh")
+    ih, _ = ctx.core_fit_index(sig, H)
+    from abi import assert_candidates_match
+
+    assert_candidates_match(ctx.core_query_index(qsig, ih), o.query_index(qsig, o.fit_index(sig, H)))
+    ctx.free_index(ih)
+
+
+def test_core_query_more_than_64_tables(ctx):
+    """More tables than a wavefront has lanes (the spans of the next query are then not prefetched)."""
+    _announce("many_tables")
+    rng = np.random.default_rng(6)
+    T, n, nq, H = 90, 3000, 400, 3
+    sig = random_sigs(rng, T, n, H, "rplsh")
+    qsig = random_sigs(rng, T, nq, H, "rplsh")
+    ih, _ = ctx.core_fit_index(sig, H)
+    from abi import assert_candidates_match
+
+    assert_candidates_match(ctx.core_query_index(qsig, ih), o.query_index(qsig, o.fit_index(sig, H)))
+    ctx.free_index(ih)
+
+
 def test_core_query_tables_that_overlap_completely(ctx, c_oracle):
     """Identical tables: the raw candidates outnumber the distinct ones eightfold, so the result
     array is cut down from its upper bound to the exact size."""
