@@ -214,6 +214,7 @@ void free_index_arrays(culsh_index* ix) {
     dev_free(ix->A);
     dev_free(ix->B);
     free_ps_codec(ix);
+    free_mh_codec(ix);
     ix->all_candidate_indices = nullptr;
     ix->all_bucket_signatures = nullptr;
     ix->bucket_candidate_offsets = nullptr;
@@ -562,16 +563,33 @@ static culsh_status minhash_fit_once(culsh_ctx* ctx, const int32_t* indices, con
         CULSH_TRY(upload_params(ctx, B_host, TH, &ix->B));
     }
     const size_t N = static_cast<size_t>(n) * nT;
+    // rank codes instead of raw hash values where that shortens the keys (needs the row count of
+    // the CSR arrays: indptr[n], read back once)
+    bool ranked = false;
+    {
+        uint32_t nnz32 = 0;
+        CULSH_TRY(read_back_u32(ctx, reinterpret_cast<const uint32_t*>(indptr) + n, 1, &nnz32));
+        CULSH_TRY(mh_build_codec(ctx, indices, static_cast<size_t>(nnz32), nT, H, d, ix.get(), &ranked));
+    }
     uint32_t* keys = nullptr;
-    CULSH_TRY(arena_alloc_t(ctx, N * H, &keys));
-    CULSH_TRY(launch_minhash(ctx, indices, indptr, ix->A, ix->B, n, nT, H, true, keys));
+    KeyEnc enc = ENC_BE;
+    int W = H;
+    if (ranked) {
+        enc = ENC_MHR;
+        W = ix->key_w;
+        CULSH_TRY(arena_alloc_t(ctx, N * W, &keys));
+        CULSH_TRY(launch_minhash_rank(ctx, indices, indptr, n, nT, H, ix.get(), keys));
+    } else {
+        CULSH_TRY(arena_alloc_t(ctx, N * H, &keys));
+        CULSH_TRY(launch_minhash(ctx, indices, indptr, ix->A, ix->B, n, nT, H, true, keys));
+    }
     CandPtr cands;
     if (cands_out) {
         cands.reset(new (std::nothrow) culsh_candidates());
         CULSH_REQUIRE(cands, CULSH_ERR_NOMEM, "host allocation failed");
         cands->device = ctx->device;
     }
-    CULSH_TRY(finish_fit(ctx, keys, n, nT, H, 4 * H, ENC_BE, H, ix.get(), cands.get()));  // minhash.cu:37
+    CULSH_TRY(finish_fit(ctx, keys, n, nT, H, 4 * H, enc, W, ix.get(), cands.get()));  // minhash.cu:37
     ix->n_features = d;
     ix->seed = seed;
     CULSH_TRY(arena_end(ctx));
@@ -854,8 +872,13 @@ culsh_status culsh_minhash_query(culsh_ctx* ctx, const int32_t* indices, const i
     CULSH_TRY(scope.begin_status);
     const int T = ix->n_hash_tables, H = ix->n_hashes;
     uint32_t* keys = nullptr;
-    CULSH_TRY(arena_alloc_t(ctx, static_cast<size_t>(nq) * T * H, &keys));
-    CULSH_TRY(launch_minhash(ctx, indices, indptr, ix->A, ix->B, nq, T, H, true, keys));
+    if (ix->enc == ENC_MHR) {
+        CULSH_TRY(arena_alloc_t(ctx, static_cast<size_t>(nq) * T * ix->key_w, &keys));
+        CULSH_TRY(launch_minhash_rank(ctx, indices, indptr, nq, T, H, ix, keys));
+    } else {
+        CULSH_TRY(arena_alloc_t(ctx, static_cast<size_t>(nq) * T * H, &keys));
+        CULSH_TRY(launch_minhash(ctx, indices, indptr, ix->A, ix->B, nq, T, H, true, keys));
+    }
     CandPtr c(new (std::nothrow) culsh_candidates());
     CULSH_REQUIRE(c, CULSH_ERR_NOMEM, "host allocation failed");
     c->device = ctx->device;
@@ -937,6 +960,10 @@ static culsh_status sig_query_keys(culsh_ctx* ctx, const void* Q_sig, int nq, in
     if (ix->enc == ENC_PSC) {
         CULSH_REQUIRE(reinterpret_cast<uintptr_t>(Q_sig) % 4 == 0, CULSH_ERR_INVALID, "signatures must be 4-byte aligned");
         return launch_ps_compress(ctx, static_cast<const int32_t*>(Q_sig), nq, ix->n_hash_tables, ix->n_hashes, ix, *keys);
+    }
+    if (ix->enc == ENC_MHR) {
+        CULSH_REQUIRE(reinterpret_cast<uintptr_t>(Q_sig) % 4 == 0, CULSH_ERR_INVALID, "signatures must be 4-byte aligned");
+        return launch_mh_sig_to_keys(ctx, static_cast<const uint32_t*>(Q_sig), nq, ix, *keys);
     }
     return launch_sig_to_keys(ctx, static_cast<const uint8_t*>(Q_sig), static_cast<size_t>(nq) * ix->n_hash_tables,
                               S, ix->enc, ix->key_w, *keys);

@@ -56,7 +56,9 @@ struct Status {
 //   ENC_BITS (signatures made of 0/1 bytes) hash h -> bit (31 - h%32) of word h/32
 //   ENC_PSC  (p-stable int32 hashes) per-hash ranks in byte order, `bits` each, MSB first;
 //            the width comes from the index's codec (pscodec.hip)
-enum KeyEnc : int { ENC_BE = 0, ENC_BITS = 1, ENC_PSC = 2 };
+//   ENC_MHR  (MinHash uint32 hashes) per-hash rank of the minimising column among all columns,
+//            in byte order of the hash values, `bits` each, MSB first (mhcodec.hip)
+enum KeyEnc : int { ENC_BE = 0, ENC_BITS = 1, ENC_PSC = 2, ENC_MHR = 3 };
 
 inline int key_words(KeyEnc enc, int sig_nbytes) {
     return enc == ENC_BITS ? (sig_nbytes + 31) / 32 : (sig_nbytes + 3) / 4;
@@ -70,6 +72,14 @@ struct PsCodec {
     int32_t* range = nullptr; // [T*H] number of values in [vmin, vmax]
     uint32_t* fwd = nullptr;  // [T*H][rmax] value - vmin -> rank in byte order (0-based)
     int32_t* inv = nullptr;   // [T*H][rmax] rank -> value
+};
+
+// Rank tables of the MinHash key compression (device arrays, owned by the index).
+struct MhCodec {
+    int bits = 0;              // bits per hash in a compressed key
+    int d = 0;                 // n_features; codes: 0..d-1 ranks, d = empty row, d+1 = matches nothing
+    uint32_t* rank = nullptr;  // [T*H][d] column -> rank of its hash value (signature byte order)
+    uint32_t* inv = nullptr;   // [T*H][d] rank -> hash value
 };
 
 }  // namespace culsh_amd
@@ -127,6 +137,7 @@ struct culsh_index {
     culsh_amd::KeyEnc enc = culsh_amd::ENC_BE;
     int key_w = 0;
     culsh_amd::PsCodec psc;  // enc == ENC_PSC only
+    culsh_amd::MhCodec mhc;  // enc == ENC_MHR only
     // family parameters (device): rplsh/index.cuh, pslsh/index.cuh, minhash/index.cuh
     culsh_kind kind = CULSH_KIND_CORE;
     bool is_double = false;
@@ -249,6 +260,23 @@ culsh_status launch_ps_compress(culsh_ctx* ctx, const int32_t* sig, size_t rows,
 culsh_status launch_ps_keys_to_sig(culsh_ctx* ctx, const culsh_index* ix, size_t count, const uint64_t* count_dev,
                                    uint8_t* sig);
 void free_ps_codec(culsh_index* ix);
+
+// ---------------------------------------------------------------- MinHash key compression (mhcodec.hip)
+// Builds the rank tables from ix->A / ix->B when that shortens the keys and every column id in
+// `indices` is below n_features `d`; then fills ix->mhc, sets ix->enc = ENC_MHR and ix->key_w, and
+// reports used = true.  May return CULSH_RETRY_UNCHAINED (its column sort is a chained radix sort).
+culsh_status mh_build_codec(culsh_ctx* ctx, const int32_t* indices, size_t nnz, int T, int H, int d, culsh_index* ix,
+                            bool* used);
+// CSR rows -> packed rank codes [T][n][ix->key_w]
+culsh_status launch_minhash_rank(culsh_ctx* ctx, const int32_t* indices, const int32_t* indptr, int n, int T, int H,
+                                 const culsh_index* ix, uint32_t* keys);
+// uint32 signatures [T][rows][H] -> packed rank codes
+culsh_status launch_mh_sig_to_keys(culsh_ctx* ctx, const uint32_t* sig, size_t rows, const culsh_index* ix,
+                                   uint32_t* keys);
+// ix->bucket_keys -> little-endian uint32 signatures of the buckets (needs table_bucket_offsets)
+culsh_status launch_mh_keys_to_sig(culsh_ctx* ctx, const culsh_index* ix, size_t count, const uint64_t* count_dev,
+                                   uint8_t* sig);
+void free_mh_codec(culsh_index* ix);
 
 // ---------------------------------------------------------------- sort (sort.hip)
 // Stable sort of each table's n items by key words (word 0 most significant), starting

@@ -260,6 +260,8 @@ culsh_status build_index_from_sorted(culsh_ctx* ctx, const uint32_t* sorted_keys
     CULSH_LAUNCH_CHECK();
     if (enc == ENC_PSC)
         CULSH_TRY(launch_ps_keys_to_sig(ctx, index, B_bound, total_dev, index->all_bucket_signatures));
+    else if (enc == ENC_MHR)
+        CULSH_TRY(launch_mh_keys_to_sig(ctx, index, B_bound, total_dev, index->all_bucket_signatures));
     else
         CULSH_TRY(launch_keys_to_sig(ctx, index->bucket_keys, B_bound, total_dev, S, enc, W, index->all_bucket_signatures));
     // end-of-build read-back: the bucket count (unless fetched above) and the sort's give-up flag
@@ -290,8 +292,8 @@ culsh_status fit_index_from_keys(culsh_ctx* ctx, uint32_t* keys, int n, int T, i
     uint32_t* sorted = nullptr;
     uint32_t bits_vary[64];
     const uint32_t* known_vary = nullptr;
-    if (enc == ENC_PSC && W <= 64) {
-        const int nb = H * index->psc.bits;  // compressed keys occupy the top H*bits bits
+    if ((enc == ENC_PSC || enc == ENC_MHR) && W <= 64) {
+        const int nb = H * (enc == ENC_PSC ? index->psc.bits : index->mhc.bits);  // compressed keys occupy the top H*bits bits
         for (int w = 0; w < W; ++w) {
             const int nbits = std::min(32, nb - 32 * w);
             bits_vary[w] = nbits >= 32 ? 0xFFFFFFFFu : (0xFFFFFFFFu << (32 - nbits));

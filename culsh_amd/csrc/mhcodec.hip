@@ -1,0 +1,300 @@
+// Order-preserving key compression for MinHash signatures.
+//
+// A MinHash signature is H little-endian uint32 hashes, ordered by the raw bytes
+// (core/fit.cuh:265-272); as key words that is 4*H bytes in which every byte varies, i.e.
+// 4*H radix passes over 4*H-byte keys.  Every hash value is (a*f + b) mod p of one column id
+// f < n_features, and for a fixed hash function that map is one-to-one (0 < a < p), so a hash
+// value can be replaced by the rank of its column among all n_features columns under that hash
+// function, taken in the byte order of the hash values.  Ranks need ceil(log2(n_features + 2))
+// bits (two more codes stand for "empty row" = 0xFFFFFFFF, which sorts last, and for "the minimum
+// came from a column >= n_features", which no fitted row can produce and therefore matches
+// nothing); packed MSB first they keep the bucket order bit for bit.  For 50,000 columns and 4
+// hashes a key shrinks from 128 to 64 bits and the sort from 16 passes to 8.
+//
+// The rank tables are built on the device: hash all columns, sort every hash function's column
+// list with the table sort of sort.hip, invert the permutation.
+#include <algorithm>
+
+#include "common.hpp"
+
+namespace culsh_amd {
+namespace {
+
+constexpr uint32_t PRIME = 4294967291u;  // minhash/hash.cuh:17 (2^32 - 5)
+
+// (a*x + b) mod (2^32 - 5) for a, x, b < 2^32, using 2^32 = 5 (mod p) twice.
+__device__ __forceinline__ uint32_t hash_mod_p(uint32_t a, uint32_t x, uint32_t b) {
+    const uint64_t v = static_cast<uint64_t>(a) * x + b;
+    const uint64_t v1 = 5ull * (v >> 32) + (v & 0xFFFFFFFFull);
+    const uint64_t v2 = 5ull * (v1 >> 32) + (v1 & 0xFFFFFFFFull);
+    return static_cast<uint32_t>(v2 >= PRIME ? v2 - PRIME : v2);
+}
+
+__global__ __launch_bounds__(256) void mh_max_index_kernel(const int32_t* __restrict__ indices, size_t nnz,
+                                                          uint32_t* __restrict__ out_max) {
+    uint32_t m = 0;
+    for (size_t i = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x; i < nnz; i += static_cast<size_t>(gridDim.x) * 256)
+        m = max(m, static_cast<uint32_t>(indices[i]));  // negative ids read as huge: out of range
+#pragma unroll
+    for (int s = 32; s > 0; s >>= 1) m = max(m, static_cast<uint32_t>(__shfl_xor(m, s, 64)));
+    if ((threadIdx.x & 63) == 0 && m > 0) atomicMax(out_max, m);
+}
+
+// keys[c][f] = byte-order form of hash_c(f): the sort then ranks columns in signature byte order
+__global__ __launch_bounds__(256) void mh_hash_columns_kernel(const uint32_t* __restrict__ A,
+                                                             const uint32_t* __restrict__ B, int d,
+                                                             uint32_t* __restrict__ keys) {
+    const int c = blockIdx.y;
+    const int f = blockIdx.x * 256 + threadIdx.x;
+    if (f < d) keys[static_cast<size_t>(c) * d + f] = __builtin_bswap32(hash_mod_p(A[c], static_cast<uint32_t>(f), B[c]));
+}
+
+// sorted_cols[c][r] = column of rank r; sorted_keys[c][r] = its byte-swapped hash
+__global__ __launch_bounds__(256) void mh_invert_kernel(const int32_t* __restrict__ sorted_cols,
+                                                       const uint32_t* __restrict__ sorted_keys, size_t total, int d,
+                                                       uint32_t* __restrict__ rank, uint32_t* __restrict__ inv) {
+    const size_t i = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
+    if (i >= total) return;
+    const size_t c = i / d;
+    const uint32_t r = static_cast<uint32_t>(i - c * d);
+    rank[c * d + static_cast<uint32_t>(sorted_cols[i])] = r;
+    inv[i] = __builtin_bswap32(sorted_keys[i]);
+}
+
+constexpr int RB = 32;  // rows per workgroup
+constexpr int NTHREADS = 256;
+
+// MinHash of CSR rows written as packed rank codes (role of compute_minhash_kernel,
+// minhash/hash.cuh:69-128, plus the key packing).  Same work split as minhash_kernel: items are
+// (row, hash) pairs with hashes fastest; besides the running minimum a thread keeps the column
+// that produced it.
+__global__ __launch_bounds__(NTHREADS) void minhash_rank_kernel(const int32_t* __restrict__ indices,
+                                                               const int32_t* __restrict__ indptr,
+                                                               const uint32_t* __restrict__ A,
+                                                               const uint32_t* __restrict__ B,
+                                                               const uint32_t* __restrict__ rank, int n, int T, int H,
+                                                               int d, int bits, int W, int th_chunk,
+                                                               uint32_t* __restrict__ out) {
+    extern __shared__ uint32_t stage[];  // [th_chunk][RB] codes
+    const int TH = T * H;
+    const int row0 = blockIdx.x * RB;
+    const int rows = min(RB, n - row0);
+    for (int c0 = 0; c0 < TH; c0 += th_chunk) {
+        const int nc = min(th_chunk, TH - c0);
+        for (int item = threadIdx.x; item < rows * nc; item += NTHREADS) {
+            const int r = item / nc, c = item - r * nc;
+            const int s = indptr[row0 + r], e = indptr[row0 + r + 1];
+            const uint32_t a = A[c0 + c], b = B[c0 + c];
+            uint32_t m = 0xFFFFFFFFu, col = 0xFFFFFFFFu;
+            for (int j = s; j < e; ++j) {
+                const uint32_t f = static_cast<uint32_t>(indices[j]);
+                const uint32_t h = hash_mod_p(a, f, b);
+                const bool less = h < m;
+                m = less ? h : m;
+                col = less ? f : col;
+            }
+            uint32_t code = static_cast<uint32_t>(d);                      // empty row: sorts last
+            if (s < e) code = col < static_cast<uint32_t>(d) ? rank[static_cast<size_t>(c0 + c) * d + col]
+                                                              : static_cast<uint32_t>(d) + 1u;  // matches nothing
+            stage[c * RB + r] = code;
+        }
+        __syncthreads();
+        // one thread per (table, row): pack the H codes of the table MSB first
+        const int tables = nc / H;  // th_chunk is a whole number of tables
+        for (int item = threadIdx.x; item < tables * rows; item += NTHREADS) {
+            const int tl = item / rows, r = item - tl * rows;
+            const int t = c0 / H + tl;
+            uint32_t* k = out + (static_cast<size_t>(t) * n + row0 + r) * W;
+            unsigned long long acc = 0;
+            int nbits = 0, w = 0;
+            for (int h = 0; h < H; ++h) {
+                acc = (acc << bits) | stage[(tl * H + h) * RB + r];
+                nbits += bits;
+                if (nbits >= 32) {
+                    k[w++] = static_cast<uint32_t>(acc >> (nbits - 32));
+                    nbits -= 32;
+                    acc &= (1ull << nbits) - 1ull;
+                }
+            }
+            if (nbits > 0) k[w++] = static_cast<uint32_t>(acc << (32 - nbits));
+        }
+        __syncthreads();
+    }
+}
+
+// uint32 signatures [T][rows][H] (reference layout) -> packed rank codes.  A value is looked
+// up among the sorted hash values of its hash function (rank = position).
+__global__ __launch_bounds__(256) void mh_sig_to_keys_kernel(const uint32_t* __restrict__ sig, size_t rows, int T,
+                                                            int H, int d, int bits, int W,
+                                                            const uint32_t* __restrict__ inv,
+                                                            uint32_t* __restrict__ keys) {
+    const size_t item = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (item >= rows * T) return;
+    const int t = static_cast<int>(item / rows);
+    const uint32_t* s = sig + item * H;
+    uint32_t* k = keys + item * W;
+    unsigned long long acc = 0;
+    int nbits = 0, w = 0;
+    for (int h = 0; h < H; ++h) {
+        const uint32_t v = s[h];
+        uint32_t code = static_cast<uint32_t>(d) + 1u;
+        if (v == 0xFFFFFFFFu) {
+            code = static_cast<uint32_t>(d);
+        } else {
+            // inv holds hash values in the byte order of their little-endian form
+            const uint32_t* tab = inv + static_cast<size_t>(t * H + h) * d;
+            const uint32_t key = __builtin_bswap32(v);
+            int lo = 0, hi = d - 1;
+            while (lo <= hi) {
+                const int mid = lo + ((hi - lo) >> 1);
+                const uint32_t mk = __builtin_bswap32(tab[mid]);
+                if (mk == key) { code = static_cast<uint32_t>(mid); break; }
+                if (mk < key) lo = mid + 1; else hi = mid - 1;
+            }
+        }
+        acc = (acc << bits) | code;
+        nbits += bits;
+        if (nbits >= 32) {
+            k[w++] = static_cast<uint32_t>(acc >> (nbits - 32));
+            nbits -= 32;
+            acc &= (1ull << nbits) - 1ull;
+        }
+    }
+    if (nbits > 0) k[w++] = static_cast<uint32_t>(acc << (32 - nbits));
+}
+
+constexpr int MH_BPB = 256;  // buckets per workgroup
+__global__ __launch_bounds__(256) void mh_keys_to_sig_kernel(const uint32_t* __restrict__ keys, size_t count,
+                                                            const uint64_t* __restrict__ count_dev,
+                                                            const int32_t* __restrict__ table_bucket_offsets, int T,
+                                                            int H, int d, int bits, int W,
+                                                            const uint32_t* __restrict__ inv,
+                                                            uint32_t* __restrict__ sig) {
+    extern __shared__ uint32_t mh_lds[];  // [MH_BPB] table ids, then [MH_BPB][W] key words
+    uint32_t* tb = mh_lds;
+    uint32_t* kw = mh_lds + MH_BPB;
+    if (count_dev) count = min(count, static_cast<size_t>(*count_dev));
+    const size_t b0 = static_cast<size_t>(blockIdx.x) * MH_BPB;
+    if (b0 >= count) return;
+    const int nb = static_cast<int>(min(static_cast<size_t>(MH_BPB), count - b0));
+    if (static_cast<int>(threadIdx.x) < nb) {
+        const size_t bucket = b0 + threadIdx.x;
+        int lo = 0, hi = T;  // largest t with table_bucket_offsets[t] <= bucket
+        while (hi - lo > 1) {
+            const int mid = (lo + hi) >> 1;
+            if (static_cast<size_t>(table_bucket_offsets[mid]) <= bucket) lo = mid; else hi = mid;
+        }
+        tb[threadIdx.x] = static_cast<uint32_t>(lo);
+    }
+    for (int i = threadIdx.x; i < nb * W; i += 256) kw[i] = keys[b0 * W + i];
+    __syncthreads();
+    const uint32_t mask = (1u << bits) - 1u;
+    for (int i = threadIdx.x; i < nb * H; i += 256) {
+        const int bl = i / H, h = i - bl * H;
+        const uint32_t* k = kw + bl * W;
+        const int o = h * bits, w0 = o >> 5, sh = o & 31;
+        const unsigned long long two = (static_cast<unsigned long long>(k[w0]) << 32) | (w0 + 1 < W ? k[w0 + 1] : 0u);
+        const uint32_t code = static_cast<uint32_t>(two >> (64 - sh - bits)) & mask;
+        sig[b0 * H + i] = code < static_cast<uint32_t>(d) ? inv[static_cast<size_t>(tb[bl] * H + h) * d + code] : 0xFFFFFFFFu;
+    }
+}
+
+}  // namespace
+
+void free_mh_codec(culsh_index* ix) {
+    dev_free(ix->mhc.rank);
+    dev_free(ix->mhc.inv);
+    ix->mhc = MhCodec();
+}
+
+culsh_status mh_build_codec(culsh_ctx* ctx, const int32_t* indices, size_t nnz, int T, int H, int d, culsh_index* ix,
+                            bool* used) {
+    *used = false;
+    const size_t TH = static_cast<size_t>(T) * H;
+    if (d < 1 || TH * static_cast<size_t>(d) > (size_t(1) << 25) || TH > 65535) return CULSH_OK;
+    int bits = 1;
+    while ((1ll << bits) < static_cast<long long>(d) + 2) ++bits;
+    const int W = (H * bits + 31) / 32;
+    if (W >= H || W > 64) return CULSH_OK;  // nothing to gain
+    // rank codes stand for columns below n_features only
+    if (nnz > 0) {
+        uint32_t* mx = nullptr;
+        CULSH_TRY(arena_alloc_t(ctx, 1, &mx));
+        CULSH_HIP(hipMemsetAsync(mx, 0, sizeof(uint32_t), ctx->stream));
+        const unsigned blocks = std::max(1u, std::min(2048u, div_up(nnz, 256 * 8)));
+        CULSH_LAUNCH(ctx, mh_max_index_kernel, dim3(blocks), dim3(256), 0, ctx->stream, indices, nnz, mx);
+        CULSH_LAUNCH_CHECK();
+        uint32_t max_index = 0;
+        CULSH_TRY(read_back_u32(ctx, mx, 1, &max_index));
+        if (max_index >= static_cast<uint32_t>(d)) return CULSH_OK;  // plain keys hash any column id
+    }
+    const size_t total = TH * d;
+    uint32_t *keys = nullptr, *keys_tmp = nullptr, *sorted = nullptr;
+    int32_t *cols_tmp = nullptr, *cols = nullptr;
+    CULSH_TRY(arena_alloc_t(ctx, total, &keys));
+    CULSH_TRY(arena_alloc_t(ctx, total, &keys_tmp));
+    CULSH_TRY(arena_alloc_t(ctx, total, &cols_tmp));
+    CULSH_TRY(arena_alloc_t(ctx, total, &cols));
+    CULSH_LAUNCH(ctx, mh_hash_columns_kernel, dim3(div_up(d, 256), static_cast<unsigned>(TH)), dim3(256), 0, ctx->stream,
+                 ix->A, ix->B, d, keys);
+    CULSH_LAUNCH_CHECK();
+    const uint32_t all_bits = 0xFFFFFFFFu;
+    CULSH_TRY(sort_tables(ctx, keys, keys_tmp, cols_tmp, cols, d, static_cast<int>(TH), 1, &all_bits, &sorted));
+    MhCodec& mc = ix->mhc;
+    CULSH_HIP(dev_malloc(&mc.rank, total * sizeof(uint32_t)));
+    CULSH_HIP(dev_malloc(&mc.inv, total * sizeof(uint32_t)));
+    CULSH_LAUNCH(ctx, mh_invert_kernel, dim3(div_up(total, 256)), dim3(256), 0, ctx->stream, cols, sorted, total, d,
+                 mc.rank, mc.inv);
+    CULSH_LAUNCH_CHECK();
+    if (ctx->sort_err_dev) {  // the column sort used the chained scan: its flag is settled here
+        uint32_t gave_up = 0;
+        CULSH_TRY(read_back_u32(ctx, ctx->sort_err_dev, 1, &gave_up));
+        ctx->sort_err_dev = nullptr;
+        if (gave_up) return CULSH_RETRY_UNCHAINED;
+    }
+    mc.bits = bits;
+    mc.d = d;
+    ix->enc = ENC_MHR;
+    ix->key_w = W;
+    *used = true;
+    return CULSH_OK;
+}
+
+culsh_status launch_minhash_rank(culsh_ctx* ctx, const int32_t* indices, const int32_t* indptr, int n, int T, int H,
+                                 const culsh_index* ix, uint32_t* keys) {
+    CULSH_REQUIRE(indptr && keys && ix->mhc.rank, CULSH_ERR_INVALID, "minhash: null pointer");
+    CULSH_REQUIRE(n > 0, CULSH_ERR_INVALID, "minhash: sizes must be positive");
+    CULSH_REQUIRE(H <= 384, CULSH_ERR_LIMIT, "minhash: n_hashes > 384 is not supported");
+    int tables_per_chunk = static_cast<int>(std::min<long long>(T, std::max(1, (12288 / RB) / H)));
+    const int th_chunk = tables_per_chunk * H;
+    const size_t lds = static_cast<size_t>(th_chunk) * RB * sizeof(uint32_t);
+    CULSH_LAUNCH(ctx, minhash_rank_kernel, dim3((n + RB - 1) / RB), dim3(NTHREADS), lds, ctx->stream, indices, indptr,
+                 ix->A, ix->B, ix->mhc.rank, n, T, H, ix->mhc.d, ix->mhc.bits, ix->key_w, th_chunk, keys);
+    CULSH_LAUNCH_CHECK();
+    return CULSH_OK;
+}
+
+culsh_status launch_mh_sig_to_keys(culsh_ctx* ctx, const uint32_t* sig, size_t rows, const culsh_index* ix,
+                                   uint32_t* keys) {
+    const size_t items = rows * ix->n_hash_tables;
+    if (items == 0) return CULSH_OK;
+    CULSH_REQUIRE(items / 256 < (1ull << 31), CULSH_ERR_LIMIT, "too many items");
+    CULSH_LAUNCH(ctx, mh_sig_to_keys_kernel, dim3(div_up(items, 256)), dim3(256), 0, ctx->stream, sig, rows,
+                 ix->n_hash_tables, ix->n_hashes, ix->mhc.d, ix->mhc.bits, ix->key_w, ix->mhc.inv, keys);
+    CULSH_LAUNCH_CHECK();
+    return CULSH_OK;
+}
+
+culsh_status launch_mh_keys_to_sig(culsh_ctx* ctx, const culsh_index* ix, size_t count, const uint64_t* count_dev,
+                                   uint8_t* sig) {
+    if (count == 0) return CULSH_OK;
+    CULSH_REQUIRE(count / MH_BPB < (1ull << 31), CULSH_ERR_LIMIT, "too many buckets");
+    const size_t lds = static_cast<size_t>(MH_BPB) * (1 + ix->key_w) * sizeof(uint32_t);
+    CULSH_LAUNCH(ctx, mh_keys_to_sig_kernel, dim3(div_up(count, MH_BPB)), dim3(256), lds, ctx->stream, ix->bucket_keys,
+                 count, count_dev, ix->table_bucket_offsets, ix->n_hash_tables, ix->n_hashes, ix->mhc.d, ix->mhc.bits,
+                 ix->key_w, ix->mhc.inv, reinterpret_cast<uint32_t*>(sig));
+    CULSH_LAUNCH_CHECK();
+    return CULSH_OK;
+}
+
+}  // namespace culsh_amd
