@@ -32,12 +32,25 @@ __device__ __forceinline__ uint32_t hash_mod_p(uint32_t a, uint32_t x, uint32_t 
 
 __global__ __launch_bounds__(256) void mh_max_index_kernel(const int32_t* __restrict__ indices, size_t nnz,
                                                           uint32_t* __restrict__ out_max) {
-    uint32_t m = 0;
-    for (size_t i = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x; i < nnz; i += static_cast<size_t>(gridDim.x) * 256)
-        m = max(m, static_cast<uint32_t>(indices[i]));  // negative ids read as huge: out of range
+    uint32_t m = 0;  // negative ids read as huge values: out of range
+    const size_t stride = static_cast<size_t>(gridDim.x) * 256;
+    const size_t tid = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
+    const size_t head = std::min(nnz, (16 - reinterpret_cast<uintptr_t>(indices) % 16) % 16 / 4);  // up to alignment
+    const uint4* v = reinterpret_cast<const uint4*>(indices + head);
+    const size_t nvec = (nnz - head) / 4;
+#pragma unroll 4
+    for (size_t i = tid; i < nvec; i += stride) {
+        const uint4 q = v[i];
+        m = max(max(m, q.x), max(max(q.y, q.z), q.w));
+    }
+    if (tid < head) m = max(m, static_cast<uint32_t>(indices[tid]));
+    const size_t tail0 = head + nvec * 4;
+    if (tail0 + tid < nnz) m = max(m, static_cast<uint32_t>(indices[tail0 + tid]));  // fewer than 4 left
 #pragma unroll
     for (int s = 32; s > 0; s >>= 1) m = max(m, static_cast<uint32_t>(__shfl_xor(m, s, 64)));
-    if ((threadIdx.x & 63) == 0 && m > 0) atomicMax(out_max, m);
+    // atomics on one address are served one after the other: only wavefronts that would raise the
+    // maximum issue one
+    if ((threadIdx.x & 63) == 0 && m > __atomic_load_n(out_max, __ATOMIC_RELAXED)) atomicMax(out_max, m);
 }
 
 // keys[c][f] = byte-order form of hash_c(f): the sort then ranks columns in signature byte order
@@ -221,7 +234,7 @@ culsh_status mh_build_codec(culsh_ctx* ctx, const int32_t* indices, size_t nnz, 
         uint32_t* mx = nullptr;
         CULSH_TRY(arena_alloc_t(ctx, 1, &mx));
         CULSH_HIP(hipMemsetAsync(mx, 0, sizeof(uint32_t), ctx->stream));
-        const unsigned blocks = std::max(1u, std::min(2048u, div_up(nnz, 256 * 8)));
+        const unsigned blocks = std::max(1u, std::min(4096u, div_up(nnz, 256 * 16)));
         CULSH_LAUNCH(ctx, mh_max_index_kernel, dim3(blocks), dim3(256), 0, ctx->stream, indices, nnz, mx);
         CULSH_LAUNCH_CHECK();
         uint32_t max_index = 0;

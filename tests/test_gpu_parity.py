@@ -615,3 +615,46 @@ def test_full_size_invariants(ctx):
         exp = np.unique(np.concatenate(exp)) if exp else np.zeros(0, np.int32)
         np.testing.assert_array_equal(idx[off[q]:off[q + 1]], exp)
     ctx.free_index(ih)
+
+
+def test_minhash_rank_keys_edge_cases(ctx):
+    """MinHash keys are stored as column ranks when every fitted column id is below n_features.
+    Checked against the oracle: query rows whose minimum comes from a column >= n_features (they
+    can match nothing in that table), empty rows on both sides, queries given as raw signatures
+    through the stage-level call, and a fit that contains an out-of-range column (plain keys)."""
+    _announce("minhash_rank_edges")
+    rng = np.random.default_rng(31)
+    n, d, T, H, nq = 3000, 400, 6, 3, 200
+    indices, indptr = make_csr(rng, n, d, 6, empty_rows=(1, 2, 50))
+    A, B = o.generate_hash_integers(5, T * H)
+    qrows = []
+    for i in range(nq):
+        r = indices[indptr[i]:indptr[i + 1]].astype(np.int64)
+        if i % 5 == 0:
+            r = np.concatenate([r, rng.integers(d, d + 4000, size=2)])   # columns the fit never saw
+        if i % 17 == 0:
+            r = np.zeros(0, dtype=np.int64)
+        qrows.append(np.unique(r))
+    qindptr = np.concatenate([[0], np.cumsum([len(r) for r in qrows])]).astype(np.int32)
+    qindices = np.concatenate(qrows).astype(np.int32)
+    from abi import assert_candidates_match, assert_index_matches
+
+    sig = o.minhash_hash(indices, indptr, A, B, T, H)
+    qsig = o.minhash_hash(qindices, qindptr, A, B, T, H)
+    exp_ix = o.fit_index(sig, H)
+    exp = o.query_index(qsig, exp_ix)
+    ih = ctx.minhash_fit(indices, indptr, d, T, H, A=A, B=B)
+    assert_index_matches(ctx.index_arrays(ih), exp_ix)
+    assert_candidates_match(ctx.minhash_query(qindices, qindptr, ih), exp)
+    assert_candidates_match(ctx.core_query_index(qsig, ih), exp)          # raw signatures -> rank keys
+    np.testing.assert_array_equal(ctx.core_find_matching_buckets(qsig, ih), o.find_matching_buckets_fast(qsig, exp_ix))
+    ctx.free_index(ih)
+    # a fitted row with a column id >= n_features: every id is hashed as it is (minhash/hash.cuh:97-104)
+    bad = indices.copy()
+    bad[7] = d + 123
+    sig2 = o.minhash_hash(bad, indptr, A, B, T, H)
+    ih2 = ctx.minhash_fit(bad, indptr, d, T, H, A=A, B=B)
+    exp_ix2 = o.fit_index(sig2, H)
+    assert_index_matches(ctx.index_arrays(ih2), exp_ix2)
+    assert_candidates_match(ctx.minhash_query(qindices, qindptr, ih2), o.query_index(qsig, exp_ix2))
+    ctx.free_index(ih2)
