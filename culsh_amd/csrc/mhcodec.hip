@@ -99,13 +99,22 @@ __global__ __launch_bounds__(NTHREADS) void minhash_rank_kernel(const int32_t* _
             const int s = indptr[row0 + r], e = indptr[row0 + r + 1];
             const uint32_t a = A[c0 + c], b = B[c0 + c];
             uint32_t m = 0xFFFFFFFFu, col = 0xFFFFFFFFu;
-            for (int j = s; j < e; ++j) {
-                const uint32_t f = static_cast<uint32_t>(indices[j]);
+            auto take = [&](uint32_t f) {
                 const uint32_t h = hash_mod_p(a, f, b);
                 const bool less = h < m;
                 m = less ? h : m;
                 col = less ? f : col;
+            };
+            int j = s;
+            for (; j + 4 <= e; j += 4) {  // four loads in flight, then four hash chains
+                const uint32_t f0 = static_cast<uint32_t>(indices[j]), f1 = static_cast<uint32_t>(indices[j + 1]);
+                const uint32_t f2 = static_cast<uint32_t>(indices[j + 2]), f3 = static_cast<uint32_t>(indices[j + 3]);
+                take(f0);
+                take(f1);
+                take(f2);
+                take(f3);
             }
+            for (; j < e; ++j) take(static_cast<uint32_t>(indices[j]));
             uint32_t code = static_cast<uint32_t>(d);                      // empty row: sorts last
             if (s < e) code = col < static_cast<uint32_t>(d) ? rank[static_cast<size_t>(c0 + c) * d + col]
                                                               : static_cast<uint32_t>(d) + 1u;  // matches nothing

@@ -42,7 +42,14 @@ __global__ __launch_bounds__(NTHREADS) void minhash_kernel(const int32_t* __rest
             const int s = indptr[row0 + r], e = indptr[row0 + r + 1];
             const uint32_t a = A[c0 + c], b = B[c0 + c];
             uint32_t m = 0xFFFFFFFFu;  // empty row (minhash/hash.cuh:86-89)
-            for (int j = s; j < e; ++j) m = min(m, hash_mod_p(a, static_cast<uint32_t>(indices[j]), b));
+            int j = s;
+            for (; j + 4 <= e; j += 4) {  // four loads in flight, then four hash chains
+                const uint32_t f0 = static_cast<uint32_t>(indices[j]), f1 = static_cast<uint32_t>(indices[j + 1]);
+                const uint32_t f2 = static_cast<uint32_t>(indices[j + 2]), f3 = static_cast<uint32_t>(indices[j + 3]);
+                m = min(min(m, hash_mod_p(a, f0, b)), hash_mod_p(a, f1, b));
+                m = min(min(m, hash_mod_p(a, f2, b)), hash_mod_p(a, f3, b));
+            }
+            for (; j < e; ++j) m = min(m, hash_mod_p(a, static_cast<uint32_t>(indices[j]), b));
             stage[c * RB + r] = m;
         }
         __syncthreads();
