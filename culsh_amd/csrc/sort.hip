@@ -221,7 +221,14 @@ __global__ __launch_bounds__(SORT_THREADS) void radix_scatter_kernel(
     for (int i = tid; i < NW * 256; i += SORT_THREADS) (&whist[0][0])[i] = 0;
     __syncthreads();
 
+    // table bases are wavefront-uniform; inside a table 32-bit element offsets suffice for the
+    // fixed key widths (n < 2^30 there)
     const size_t tbase = static_cast<size_t>(t) * n;
+    const int Wc = KW > 0 ? KW : W;
+    const uint32_t* tkeys_in = keys_in + tbase * Wc;
+    const int32_t* trows_in = rows_in ? rows_in + tbase : nullptr;
+    uint32_t* tkeys_out = keys_out + tbase * Wc;
+    int32_t* trows_out = rows_out + tbase;
     const int tile0 = tile * SORT_TILE;
     const int base_idx = tile0 + wave * (SORT_ITEMS * 64);
     uint32_t kw[SORT_ITEMS], rank[SORT_ITEMS];
@@ -231,9 +238,11 @@ __global__ __launch_bounds__(SORT_THREADS) void radix_scatter_kernel(
     for (int j = 0; j < SORT_ITEMS; ++j) {
         const int idx = base_idx + j * 64 + lane;
         const bool valid = idx < n;
-        const uint32_t k = valid ? keys_in[(tbase + idx) * W + word] : 0u;
+        uint32_t k = 0u;
+        if (valid) k = KW > 0 ? tkeys_in[static_cast<uint32_t>(idx) * static_cast<uint32_t>(KW) + static_cast<uint32_t>(word)]
+                              : tkeys_in[static_cast<size_t>(idx) * W + word];
         kw[j] = k;
-        if (ONE_WORD) rw[j] = (valid && rows_in) ? rows_in[tbase + idx] : idx;
+        if (ONE_WORD) rw[j] = (valid && trows_in) ? trows_in[static_cast<uint32_t>(idx)] : idx;
         const uint32_t d = (k >> shift) & 255u;
         // lanes holding the same digit
         const unsigned long long live = __builtin_amdgcn_ballot_w64(valid);
@@ -329,28 +338,28 @@ __global__ __launch_bounds__(SORT_THREADS) void radix_scatter_kernel(
     for (int slot = tid; slot < cnt; slot += SORT_THREADS) {
         if (ONE_WORD) {
             const uint32_t k = st_key[slot];
-            const size_t dst = tbase + static_cast<uint32_t>(gbase[(k >> shift) & 255u] + slot);
-            keys_out[dst] = k;
-            rows_out[dst] = st_row[slot];
+            const uint32_t dst = gbase[(k >> shift) & 255u] + static_cast<uint32_t>(slot);
+            tkeys_out[dst] = k;
+            trows_out[dst] = st_row[slot];
         } else {
-            const int src = tile0 + static_cast<int>(st_key[slot]);
-            const uint32_t* ks = keys_in + (tbase + src) * W;
+            const uint32_t src = static_cast<uint32_t>(tile0) + st_key[slot];
             if (KW == 4) {
-                const uint4 v = *reinterpret_cast<const uint4*>(ks);
+                const uint4 v = *reinterpret_cast<const uint4*>(tkeys_in + src * 4u);
                 const uint32_t kd = word == 0 ? v.x : (word == 1 ? v.y : (word == 2 ? v.z : v.w));
-                const size_t dst = tbase + static_cast<uint32_t>(gbase[(kd >> shift) & 255u] + slot);
-                *reinterpret_cast<uint4*>(keys_out + dst * 4) = v;
-                rows_out[dst] = rows_in ? rows_in[tbase + src] : src;
+                const uint32_t dst = gbase[(kd >> shift) & 255u] + static_cast<uint32_t>(slot);
+                *reinterpret_cast<uint4*>(tkeys_out + dst * 4u) = v;
+                trows_out[dst] = trows_in ? trows_in[src] : static_cast<int32_t>(src);
             } else if (KW == 2) {
-                const uint2 v = *reinterpret_cast<const uint2*>(ks);
+                const uint2 v = *reinterpret_cast<const uint2*>(tkeys_in + src * 2u);
                 const uint32_t kd = word == 0 ? v.x : v.y;
-                const size_t dst = tbase + static_cast<uint32_t>(gbase[(kd >> shift) & 255u] + slot);
-                *reinterpret_cast<uint2*>(keys_out + dst * 2) = v;
-                rows_out[dst] = rows_in ? rows_in[tbase + src] : src;
+                const uint32_t dst = gbase[(kd >> shift) & 255u] + static_cast<uint32_t>(slot);
+                *reinterpret_cast<uint2*>(tkeys_out + dst * 2u) = v;
+                trows_out[dst] = trows_in ? trows_in[src] : static_cast<int32_t>(src);
             } else {
-                const size_t dst = tbase + static_cast<uint32_t>(gbase[(ks[word] >> shift) & 255u] + slot);
-                for (int w = 0; w < W; ++w) keys_out[dst * W + w] = ks[w];
-                rows_out[dst] = rows_in ? rows_in[tbase + src] : src;
+                const uint32_t* ks = tkeys_in + static_cast<size_t>(src) * W;
+                const uint32_t dst = gbase[(ks[word] >> shift) & 255u] + static_cast<uint32_t>(slot);
+                for (int w = 0; w < W; ++w) tkeys_out[static_cast<size_t>(dst) * W + w] = ks[w];
+                trows_out[dst] = trows_in ? trows_in[src] : static_cast<int32_t>(src);
             }
         }
     }
@@ -451,7 +460,8 @@ culsh_status sort_tables(culsh_ctx* ctx, uint32_t* keys_in, uint32_t* keys_tmp, 
         // the last pass must land in rows_out
         int32_t* rout = ((np - 1 - p) % 2 == 0) ? rows_out : rows_tmp;
         uint32_t* pass_dtot = dtot + static_cast<size_t>(p) * T * 256;
-        const bool aligned = reinterpret_cast<uintptr_t>(kin) % 16 == 0 && reinterpret_cast<uintptr_t>(kout) % 16 == 0;
+        // fixed-width variants use 32-bit element offsets inside a table
+        const bool aligned = reinterpret_cast<uintptr_t>(kin) % 16 == 0 && reinterpret_cast<uintptr_t>(kout) % 16 == 0 && n < (1 << 30);
         if (chained) {
             const dim3 grid(static_cast<unsigned>(tiles) * T);
             uint32_t* pass_state = state + static_cast<size_t>(p) * state_words;
@@ -459,7 +469,7 @@ culsh_status sort_tables(culsh_ctx* ctx, uint32_t* keys_in, uint32_t* keys_tmp, 
     CULSH_LAUNCH(ctx, (radix_scatter_kernel<KW, true>), grid, dim3(SORT_THREADS), 0, ctx->stream, kin, rin, kout, rout, \
                  static_cast<const uint32_t*>(nullptr), n, W, passes[p].word, passes[p].shift, tiles, T,              \
                  static_cast<const uint32_t*>(pass_dtot), pass_state, err, spin_limit)
-            if (W == 1) SCATTER(1);
+            if (W == 1 && n < (1 << 30)) SCATTER(1);
             else if (W == 2 && aligned) SCATTER(2);
             else if (W == 4 && aligned) SCATTER(4);
             else SCATTER(0);
@@ -476,7 +486,7 @@ culsh_status sort_tables(culsh_ctx* ctx, uint32_t* keys_in, uint32_t* keys_tmp, 
                  static_cast<const uint32_t*>(hist), n, W, passes[p].word, passes[p].shift, tiles, T,                  \
                  static_cast<const uint32_t*>(nullptr), static_cast<uint32_t*>(nullptr),                               \
                  static_cast<uint32_t*>(nullptr), 0)
-            if (W == 1) SCATTER(1);
+            if (W == 1 && n < (1 << 30)) SCATTER(1);
             else if (W == 2 && aligned) SCATTER(2);
             else if (W == 4 && aligned) SCATTER(4);
             else SCATTER(0);
