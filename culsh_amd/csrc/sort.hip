@@ -26,8 +26,8 @@ namespace culsh_amd {
 namespace {
 
 constexpr int SORT_THREADS = 256;
-constexpr int SORT_ITEMS = 16;
-constexpr int SORT_TILE = SORT_THREADS * SORT_ITEMS;  // 4096 items per workgroup
+constexpr int SORT_ITEMS = 8;
+constexpr int SORT_TILE = SORT_THREADS * SORT_ITEMS;  // 2048 items per workgroup (7-8 workgroups per CU; 16 items: 4)
 
 // vary[w] |= key[t][i][w] ^ key[t][0][w]
 __device__ __forceinline__ void publish_vary(uint32_t acc, uint32_t* __restrict__ slot) {
@@ -98,7 +98,10 @@ struct PassList {
     int shift[MAX_PASSES_PER_LAUNCH];
 };
 
-// Digit totals per (pass, table, digit) for up to 16 passes in one read of the keys.
+// Digit totals per (pass, table, digit) for up to 16 passes in one read of the keys (tiles of its
+// own size: the totals do not depend on how the scatter cuts a table).
+constexpr int TOT_ITEMS = 32;
+constexpr int TOT_TILE = SORT_THREADS * TOT_ITEMS;
 __global__ __launch_bounds__(SORT_THREADS) void radix_totals_kernel(const uint32_t* __restrict__ keys, int n, int W,
                                                                    PassList pl, int T,
                                                                    uint32_t* __restrict__ dtot /*[pass][T][256]*/) {
@@ -110,22 +113,22 @@ __global__ __launch_bounds__(SORT_THREADS) void radix_totals_kernel(const uint32
     for (int i = threadIdx.x; i < copies * pl.count * 256; i += SORT_THREADS) (&h[0][0])[i] = 0;
     __syncthreads();
     const uint32_t* tk = keys + static_cast<size_t>(t) * n * W;
-    uint32_t kw[SORT_ITEMS];
+    uint32_t kw[TOT_ITEMS];
     int last_word = -1;
     for (int p = 0; p < pl.count; ++p) {  // passes are ordered by word, so a word is fetched once
         if (pl.word[p] != last_word) {
             last_word = pl.word[p];
 #pragma unroll
-            for (int j = 0; j < SORT_ITEMS; ++j) {
-                const int idx = tile * SORT_TILE + j * SORT_THREADS + threadIdx.x;
+            for (int j = 0; j < TOT_ITEMS; ++j) {
+                const int idx = tile * TOT_TILE + j * SORT_THREADS + threadIdx.x;
                 kw[j] = (idx < n) ? tk[static_cast<size_t>(idx) * W + last_word] : 0u;
             }
         }
         uint32_t* hp = h[mine * pl.count + p];
         const int shift = pl.shift[p];
 #pragma unroll
-        for (int j = 0; j < SORT_ITEMS; ++j) {
-            const int idx = tile * SORT_TILE + j * SORT_THREADS + threadIdx.x;
+        for (int j = 0; j < TOT_ITEMS; ++j) {
+            const int idx = tile * TOT_TILE + j * SORT_THREADS + threadIdx.x;
             if (idx < n) atomicAdd(&hp[(kw[j] >> shift) & 255u], 1u);
         }
     }
@@ -444,7 +447,7 @@ culsh_status sort_tables(culsh_ctx* ctx, uint32_t* keys_in, uint32_t* keys_tmp, 
                 pl.word[i] = i < pl.count ? passes[p0 + i].word : 0;
                 pl.shift[i] = i < pl.count ? passes[p0 + i].shift : 0;
             }
-            CULSH_LAUNCH(ctx, radix_totals_kernel, dim3(tiles, T), dim3(SORT_THREADS), 0, ctx->stream, keys_in, n, W, pl,
+            CULSH_LAUNCH(ctx, radix_totals_kernel, dim3((n + TOT_TILE - 1) / TOT_TILE, T), dim3(SORT_THREADS), 0, ctx->stream, keys_in, n, W, pl,
                          T, dtot + static_cast<size_t>(p0) * T * 256);
             CULSH_LAUNCH_CHECK();
         }
