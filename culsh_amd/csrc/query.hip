@@ -482,7 +482,18 @@ int env_int(const char* name, int dflt) {
     return (v && *v) ? std::atoi(v) : dflt;
 }
 
-// `raw_total` (device) holds the number of raw candidates = sum of all span lengths.
+// The zero-initialised words a query needs, in one block cleared by one memset:
+// [0] raw candidate total, [1] error flags (low half) and ticket counter (high half),
+// [2 .. 2 + n_queries) the published words of the chained scan.
+culsh_status alloc_query_words(culsh_ctx* ctx, int n_queries, unsigned long long** words) {
+    const size_t count = 2 + static_cast<size_t>(n_queries);
+    CULSH_TRY(arena_alloc_t(ctx, count, words));
+    CULSH_HIP(hipMemsetAsync(*words, 0, count * sizeof(unsigned long long), ctx->stream));
+    return CULSH_OK;
+}
+
+// `raw_total` points at the block of alloc_query_words; its first word holds the number of raw
+// candidates = sum of all span lengths.
 culsh_status query_from_spans(culsh_ctx* ctx, const int2* spans, const unsigned long long* raw_total, int n_queries,
                               const culsh_index* index, culsh_candidates* out) {
     const int T = index->n_hash_tables;
@@ -545,11 +556,9 @@ culsh_status query_from_spans(culsh_ctx* ctx, const int2* spans, const unsigned 
         }
         // a query holds at most n distinct rows, which bounds the output when buckets overlap heavily
         const uint64_t cap = std::min<uint64_t>(R, static_cast<uint64_t>(n_queries) * static_cast<uint64_t>(n));
-        unsigned int* err = nullptr;
-        CULSH_TRY(arena_alloc_t(ctx, static_cast<size_t>(n_queries), &a.state));
-        CULSH_TRY(arena_alloc_t(ctx, 2, &err));  // [0] error flags, [1] ticket counter
-        CULSH_HIP(hipMemsetAsync(a.state, 0, static_cast<size_t>(n_queries) * sizeof(unsigned long long), ctx->stream));
-        CULSH_HIP(hipMemsetAsync(err, 0, 2 * sizeof(unsigned int), ctx->stream));
+        unsigned long long* words = const_cast<unsigned long long*>(raw_total);
+        unsigned int* err = reinterpret_cast<unsigned int*>(words + 1);  // [0] error flags, [1] ticket counter
+        a.state = words + 2;
         a.ticket = err + 1;
         CULSH_HIP(dev_malloc(&out->query_candidate_indices, cap * sizeof(int32_t)));
         a.out = out->query_candidate_indices;
@@ -637,8 +646,7 @@ culsh_status query_from_matched(culsh_ctx* ctx, const int32_t* matched, int n_qu
     int2* spans = nullptr;
     unsigned long long* raw_total = nullptr;
     CULSH_TRY(arena_alloc_t(ctx, pairs, &spans));
-    CULSH_TRY(arena_alloc_t(ctx, 1, &raw_total));
-    CULSH_HIP(hipMemsetAsync(raw_total, 0, sizeof(unsigned long long), ctx->stream));
+    CULSH_TRY(alloc_query_words(ctx, n_queries, &raw_total));
     CULSH_LAUNCH(ctx, span_kernel, dim3(div_up(pairs, 256)), dim3(256), 0, ctx->stream, matched,
                  index->bucket_candidate_offsets, pairs, spans, raw_total);
     CULSH_LAUNCH_CHECK();
@@ -651,8 +659,7 @@ culsh_status query_from_keys(culsh_ctx* ctx, const uint32_t* q_keys, int n_queri
     int2* spans = nullptr;
     unsigned long long* raw_total = nullptr;
     CULSH_TRY(arena_alloc_t(ctx, static_cast<size_t>(n_queries) * index->n_hash_tables, &spans));
-    CULSH_TRY(arena_alloc_t(ctx, 1, &raw_total));
-    CULSH_HIP(hipMemsetAsync(raw_total, 0, sizeof(unsigned long long), ctx->stream));
+    CULSH_TRY(alloc_query_words(ctx, n_queries, &raw_total));
     CULSH_TRY(launch_find_matching_buckets(ctx, q_keys, n_queries, index, nullptr, spans, raw_total));
     return query_from_spans(ctx, spans, raw_total, n_queries, index, out);
 }
