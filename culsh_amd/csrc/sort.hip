@@ -422,23 +422,24 @@ culsh_status sort_tables(culsh_ctx* ctx, uint32_t* keys_in, uint32_t* keys_tmp, 
     uint32_t* kin = keys_in;
     uint32_t* kout = keys_tmp;
     const int np = static_cast<int>(passes.size());
-    uint32_t* dtot = nullptr;  // [pass][T][256] digit totals
-    CULSH_TRY(arena_alloc_t(ctx, static_cast<size_t>(np) * T * 256, &dtot));
-    CULSH_HIP(hipMemsetAsync(dtot, 0, static_cast<size_t>(np) * T * 256 * sizeof(uint32_t), ctx->stream));
-
     const char* env_unchained = std::getenv("CULSH_SORT_UNCHAINED");
     const bool chained = !ctx->sort_unchained && n < (1 << 30) && !(env_unchained && *env_unchained == '1') &&
                          static_cast<size_t>(tiles) * T < (1ull << 31);
-    uint32_t* hist = nullptr;   // unchained: [T][256][tiles]
-    uint32_t* state = nullptr;  // chained: [pass][T][tiles][256]
-    uint32_t* err = nullptr;
+    // zero-initialised words in one block, cleared by one memset: [pass][T][256] digit totals, then
+    // (chained) the published words [pass][T][tiles][256] and 2 flag words
+    const size_t dtot_words = static_cast<size_t>(np) * T * 256;
     const size_t state_words = static_cast<size_t>(T) * tiles * 256;
+    const size_t zero_words = dtot_words + (chained ? 2 + static_cast<size_t>(np) * state_words : 0);
+    uint32_t* dtot = nullptr;
+    CULSH_TRY(arena_alloc_t(ctx, zero_words, &dtot));
+    CULSH_HIP(hipMemsetAsync(dtot, 0, zero_words * sizeof(uint32_t), ctx->stream));
+    uint32_t* hist = nullptr;   // unchained: [T][256][tiles]
+    uint32_t* state = nullptr;
+    uint32_t* err = nullptr;
     ctx->sort_err_dev = nullptr;
     if (chained) {
-        CULSH_TRY(arena_alloc_t(ctx, static_cast<size_t>(np) * state_words, &state));
-        CULSH_TRY(arena_alloc_t(ctx, 2, &err));
-        CULSH_HIP(hipMemsetAsync(state, 0, static_cast<size_t>(np) * state_words * sizeof(uint32_t), ctx->stream));
-        CULSH_HIP(hipMemsetAsync(err, 0, 2 * sizeof(uint32_t), ctx->stream));
+        state = dtot + dtot_words;  // rows of 256 words stay 1 KiB aligned
+        err = state + static_cast<size_t>(np) * state_words;
         ctx->sort_err_dev = err;
         for (int p0 = 0; p0 < np; p0 += MAX_PASSES_PER_LAUNCH) {
             PassList pl;
