@@ -216,8 +216,10 @@ __global__ __launch_bounds__(SORT_THREADS) void radix_scatter_kernel(
     __shared__ uint32_t dstart[256];      // start of each digit's run inside the sorted tile
     __shared__ uint32_t gbase[256];       // global position of the run minus dstart (wraps, used additively)
     __shared__ uint32_t scratch[17];
-    __shared__ uint32_t st_key[SORT_TILE];                 // ONE_WORD: key, else: source slot in the tile
-    __shared__ int32_t st_row[ONE_WORD ? SORT_TILE : 1];
+    constexpr bool TWO_WORDS = (KW == 2);                  // staged in full as well (8-byte keys)
+    constexpr bool STAGED = ONE_WORD || TWO_WORDS;
+    __shared__ __attribute__((aligned(8))) uint32_t st_key[SORT_TILE * (TWO_WORDS ? 2 : 1)];  // staged keys, else source slots
+    __shared__ int32_t st_row[STAGED ? SORT_TILE : 1];
     const int tile = CHAINED ? static_cast<int>(blockIdx.x / T) : static_cast<int>(blockIdx.x);
     const int t = CHAINED ? static_cast<int>(blockIdx.x - static_cast<unsigned>(tile) * T) : static_cast<int>(blockIdx.y);
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -235,17 +237,25 @@ __global__ __launch_bounds__(SORT_THREADS) void radix_scatter_kernel(
     const int tile0 = tile * SORT_TILE;
     const int base_idx = tile0 + wave * (SORT_ITEMS * 64);
     uint32_t kw[SORT_ITEMS], rank[SORT_ITEMS];
-    int32_t rw[ONE_WORD ? SORT_ITEMS : 1];
+    int32_t rw[STAGED ? SORT_ITEMS : 1];
+    uint32_t kw_other[TWO_WORDS ? SORT_ITEMS : 1];  // the word of a two-word key that is not the digit word
     const unsigned long long lt_mask = (1ull << lane) - 1ull;
 #pragma unroll
     for (int j = 0; j < SORT_ITEMS; ++j) {
         const int idx = base_idx + j * 64 + lane;
         const bool valid = idx < n;
         uint32_t k = 0u;
-        if (valid) k = KW > 0 ? tkeys_in[static_cast<uint32_t>(idx) * static_cast<uint32_t>(KW) + static_cast<uint32_t>(word)]
-                              : tkeys_in[static_cast<size_t>(idx) * W + word];
+        if (TWO_WORDS) {
+            uint2 kv = make_uint2(0u, 0u);
+            if (valid) kv = *reinterpret_cast<const uint2*>(tkeys_in + static_cast<uint32_t>(idx) * 2u);
+            k = word == 0 ? kv.x : kv.y;
+            kw_other[j] = word == 0 ? kv.y : kv.x;
+        } else if (valid) {
+            k = KW > 0 ? tkeys_in[static_cast<uint32_t>(idx) * static_cast<uint32_t>(KW) + static_cast<uint32_t>(word)]
+                       : tkeys_in[static_cast<size_t>(idx) * W + word];
+        }
         kw[j] = k;
-        if (ONE_WORD) rw[j] = (valid && trows_in) ? trows_in[static_cast<uint32_t>(idx)] : idx;
+        if (STAGED) rw[j] = (valid && trows_in) ? trows_in[static_cast<uint32_t>(idx)] : idx;
         const uint32_t d = (k >> shift) & 255u;
         // lanes holding the same digit
         const unsigned long long live = __builtin_amdgcn_ballot_w64(valid);
@@ -331,6 +341,10 @@ __global__ __launch_bounds__(SORT_THREADS) void radix_scatter_kernel(
             if (ONE_WORD) {
                 st_key[lp] = kw[j];
                 st_row[lp] = rw[j];
+            } else if (TWO_WORDS) {
+                *reinterpret_cast<uint2*>(&st_key[2 * lp]) =
+                    word == 0 ? make_uint2(kw[j], kw_other[j]) : make_uint2(kw_other[j], kw[j]);
+                st_row[lp] = rw[j];
             } else {
                 st_key[lp] = static_cast<uint32_t>(idx - tile0);
             }
@@ -343,6 +357,12 @@ __global__ __launch_bounds__(SORT_THREADS) void radix_scatter_kernel(
             const uint32_t k = st_key[slot];
             const uint32_t dst = gbase[(k >> shift) & 255u] + static_cast<uint32_t>(slot);
             tkeys_out[dst] = k;
+            trows_out[dst] = st_row[slot];
+        } else if (TWO_WORDS) {
+            const uint2 v = *reinterpret_cast<const uint2*>(&st_key[2 * slot]);
+            const uint32_t kd = word == 0 ? v.x : v.y;
+            const uint32_t dst = gbase[(kd >> shift) & 255u] + static_cast<uint32_t>(slot);
+            *reinterpret_cast<uint2*>(tkeys_out + dst * 2u) = v;
             trows_out[dst] = st_row[slot];
         } else {
             const uint32_t src = static_cast<uint32_t>(tile0) + st_key[slot];
