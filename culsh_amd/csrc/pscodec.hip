@@ -57,6 +57,8 @@ __global__ __launch_bounds__(256) void ps_minmax_kernel(const int32_t* __restric
     }
 }
 
+// VEC4: H is a multiple of 4 and sig is 16-byte aligned, so the hashes of an item come in 16-byte loads.
+template <bool VEC4>
 __global__ __launch_bounds__(256) void ps_compress_kernel(const int32_t* __restrict__ sig, size_t rows, int T, int H,
                                                          int bits, int rmax, int W,
                                                          const int32_t* __restrict__ vmin,
@@ -70,9 +72,9 @@ __global__ __launch_bounds__(256) void ps_compress_kernel(const int32_t* __restr
     uint32_t* k = keys + item * W;
     unsigned long long acc = 0;
     int nbits = 0, w = 0;
-    for (int h = 0; h < H; ++h) {
+    auto put = [&](int h, int32_t v) {
         const int c = t * H + h;
-        const long long idx = static_cast<long long>(s[h]) - vmin[c];
+        const long long idx = static_cast<long long>(v) - vmin[c];
         const uint32_t code = (idx >= 0 && idx < range[c]) ? fwd[static_cast<size_t>(c) * rmax + idx] + 1u : 0u;
         acc = (acc << bits) | code;
         nbits += bits;
@@ -81,6 +83,17 @@ __global__ __launch_bounds__(256) void ps_compress_kernel(const int32_t* __restr
             nbits -= 32;
             acc &= (1ull << nbits) - 1ull;
         }
+    };
+    if (VEC4) {
+        for (int h = 0; h < H; h += 4) {
+            const int4 v = *reinterpret_cast<const int4*>(s + h);
+            put(h, v.x);
+            put(h + 1, v.y);
+            put(h + 2, v.z);
+            put(h + 3, v.w);
+        }
+    } else {
+        for (int h = 0; h < H; ++h) put(h, s[h]);
     }
     if (nbits > 0) k[w++] = static_cast<uint32_t>(acc << (32 - nbits));
 }
@@ -198,8 +211,12 @@ culsh_status launch_ps_compress(culsh_ctx* ctx, const int32_t* sig, size_t rows,
     if (items == 0) return CULSH_OK;
     CULSH_REQUIRE(items / 256 < (1ull << 31), CULSH_ERR_LIMIT, "too many items");
     const PsCodec& pc = ix->psc;
-    CULSH_LAUNCH(ctx, ps_compress_kernel, dim3(div_up(items, 256)), dim3(256), 0, ctx->stream, sig, rows, T, H,
-                 pc.bits, pc.rmax, ix->key_w, pc.vmin, pc.range, pc.fwd, keys);
+    if (H % 4 == 0 && reinterpret_cast<uintptr_t>(sig) % 16 == 0)
+        CULSH_LAUNCH(ctx, ps_compress_kernel<true>, dim3(div_up(items, 256)), dim3(256), 0, ctx->stream, sig, rows, T, H,
+                     pc.bits, pc.rmax, ix->key_w, pc.vmin, pc.range, pc.fwd, keys);
+    else
+        CULSH_LAUNCH(ctx, ps_compress_kernel<false>, dim3(div_up(items, 256)), dim3(256), 0, ctx->stream, sig, rows, T, H,
+                     pc.bits, pc.rmax, ix->key_w, pc.vmin, pc.range, pc.fwd, keys);
     CULSH_LAUNCH_CHECK();
     return CULSH_OK;
 }
