@@ -57,25 +57,19 @@ __global__ __launch_bounds__(256) void ps_minmax_kernel(const int32_t* __restric
     }
 }
 
-// VEC4: H is a multiple of 4 and sig is 16-byte aligned, so the hashes of an item come in 16-byte loads.
-template <bool VEC4>
-__global__ __launch_bounds__(256) void ps_compress_kernel(const int32_t* __restrict__ sig, size_t rows, int T, int H,
-                                                         int bits, int rmax, int W,
-                                                         const int32_t* __restrict__ vmin,
-                                                         const int32_t* __restrict__ range,
-                                                         const uint32_t* __restrict__ fwd,
-                                                         uint32_t* __restrict__ keys) {
-    const size_t item = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
-    if (item >= rows * T) return;
-    const int t = static_cast<int>(item / rows);
-    const int32_t* s = sig + item * H;
-    uint32_t* k = keys + item * W;
+// Rank tables of one table's H hash functions fit in LDS when they have at most this many words.
+// Looking ranks up in global memory costs a 64-address gather per wave and hash, which keeps the
+// texture path busy for longer than everything else in these kernels together.
+constexpr int PS_LUT_WORDS = 8192;
+
+template <bool VEC4, typename F, typename V>
+__device__ __forceinline__ void ps_compress_item(const int32_t* __restrict__ s, uint32_t* __restrict__ k, int H,
+                                                 int bits, int rmax, F fwd, V vmin, V range) {
     unsigned long long acc = 0;
     int nbits = 0, w = 0;
     auto put = [&](int h, int32_t v) {
-        const int c = t * H + h;
-        const long long idx = static_cast<long long>(v) - vmin[c];
-        const uint32_t code = (idx >= 0 && idx < range[c]) ? fwd[static_cast<size_t>(c) * rmax + idx] + 1u : 0u;
+        const long long idx = static_cast<long long>(v) - vmin[h];
+        const uint32_t code = (idx >= 0 && idx < range[h]) ? fwd[h * rmax + static_cast<int>(idx)] + 1u : 0u;
         acc = (acc << bits) | code;
         nbits += bits;
         if (nbits >= 32) {
@@ -98,19 +92,62 @@ __global__ __launch_bounds__(256) void ps_compress_kernel(const int32_t* __restr
     if (nbits > 0) k[w++] = static_cast<uint32_t>(acc << (32 - nbits));
 }
 
+// VEC4: H is a multiple of 4 and sig is 16-byte aligned, so the hashes of an item come in 16-byte loads.
+// `use_lds`: the launch carries (H * rmax + 2 * H) words of LDS; a workgroup whose items all belong to
+// one table (all but T - 1 of them) looks ranks up there.
+template <bool VEC4>
+__global__ __launch_bounds__(256) void ps_compress_kernel(const int32_t* __restrict__ sig, size_t rows, int T, int H,
+                                                         int bits, int rmax, int W, int use_lds,
+                                                         const int32_t* __restrict__ vmin,
+                                                         const int32_t* __restrict__ range,
+                                                         const uint32_t* __restrict__ fwd,
+                                                         uint32_t* __restrict__ keys) {
+    extern __shared__ uint32_t ps_lut[];  // [H * rmax] ranks, [H] minima, [H] ranges
+    const size_t items = rows * T;
+    const size_t item0 = static_cast<size_t>(blockIdx.x) * 256;
+    const size_t item = item0 + threadIdx.x;
+    const int t_first = static_cast<int>(item0 / rows);
+    const int t_last = static_cast<int>(min(item0 + 255, items - 1) / rows);
+    const bool staged = use_lds && t_first == t_last;  // uniform over the workgroup
+    if (staged) {
+        const int lut = H * rmax;
+        const uint32_t* f = fwd + static_cast<size_t>(t_first) * lut;
+        for (int i = threadIdx.x; i < lut; i += 256) ps_lut[i] = f[i];
+        for (int h = threadIdx.x; h < H; h += 256) {
+            ps_lut[lut + h] = static_cast<uint32_t>(vmin[t_first * H + h]);
+            ps_lut[lut + H + h] = static_cast<uint32_t>(range[t_first * H + h]);
+        }
+        __syncthreads();
+    }
+    if (item >= items) return;
+    const int32_t* s = sig + item * H;
+    uint32_t* k = keys + item * W;
+    if (staged) {
+        const int32_t* lv = reinterpret_cast<const int32_t*>(ps_lut + H * rmax);
+        ps_compress_item<VEC4>(s, k, H, bits, rmax, ps_lut, lv, lv + H);
+    } else {
+        const int t = static_cast<int>(item / rows);
+        ps_compress_item<VEC4>(s, k, H, bits, rmax, fwd + static_cast<size_t>(t) * H * rmax, vmin + t * H,
+                               range + t * H);
+    }
+}
+
 // A workgroup restores the signatures of PS_BPB consecutive buckets: the table of each bucket
 // is searched once and kept in LDS with the bucket's key words, then (bucket, hash) pairs are
-// written by consecutive threads to consecutive addresses.
+// written by consecutive threads to consecutive addresses.  With `use_lds` the launch also carries
+// 2 * H * rmax words of LDS for the value tables of two neighbouring hash tables, which cover a
+// workgroup unless it meets three tables or more.
 constexpr int PS_BPB = 256;
 __global__ __launch_bounds__(256) void ps_keys_to_sig_kernel(const uint32_t* __restrict__ keys, size_t count,
                                                             const uint64_t* __restrict__ count_dev,
                                                             const int32_t* __restrict__ table_bucket_offsets, int T,
-                                                            int H, int bits, int rmax, int W,
+                                                            int H, int bits, int rmax, int W, int use_lds,
                                                             const int32_t* __restrict__ inv,
                                                             int32_t* __restrict__ sig) {
-    extern __shared__ uint32_t ps_lds[];  // [PS_BPB] table ids, then [PS_BPB][W] key words
+    extern __shared__ uint32_t ps_lds[];  // [PS_BPB] table ids, [PS_BPB][W] key words, then the value tables
     uint32_t* tb = ps_lds;
     uint32_t* kw = ps_lds + PS_BPB;
+    int32_t* lut = reinterpret_cast<int32_t*>(kw + PS_BPB * W);
     if (count_dev) count = min(count, static_cast<size_t>(*count_dev));
     const size_t b0 = static_cast<size_t>(blockIdx.x) * PS_BPB;
     if (b0 >= count) return;
@@ -126,14 +163,38 @@ __global__ __launch_bounds__(256) void ps_keys_to_sig_kernel(const uint32_t* __r
     }
     for (int i = threadIdx.x; i < nb * W; i += 256) kw[i] = keys[b0 * W + i];
     __syncthreads();
+    const int t_first = static_cast<int>(tb[0]);
+    const bool staged = use_lds && static_cast<int>(tb[nb - 1]) - t_first <= 1;  // uniform over the workgroup
+    if (staged) {
+        const int words = min(2, T - t_first) * H * rmax;
+        const int32_t* src = inv + static_cast<size_t>(t_first) * H * rmax;
+        for (int i = threadIdx.x; i < words; i += 256) lut[i] = src[i];
+        __syncthreads();
+    }
     const uint32_t mask = (1u << bits) - 1u;
-    for (int i = threadIdx.x; i < nb * H; i += 256) {
-        const int bl = i / H, h = i - bl * H;
+    auto value = [&](int bl, int h) -> int32_t {
         const uint32_t* k = kw + bl * W;
         const int o = h * bits, w0 = o >> 5, sh = o & 31;
         const unsigned long long two = (static_cast<unsigned long long>(k[w0]) << 32) | (w0 + 1 < W ? k[w0 + 1] : 0u);
         const uint32_t code = static_cast<uint32_t>(two >> (64 - sh - bits)) & mask;
-        sig[b0 * H + i] = code ? inv[static_cast<size_t>(tb[bl] * H + h) * rmax + (code - 1u)] : 0;
+        if (!code) return 0;
+        const int c = static_cast<int>(tb[bl]) * H + h;
+        return staged ? lut[(c - t_first * H) * rmax + static_cast<int>(code - 1u)]
+                      : inv[static_cast<size_t>(c) * rmax + (code - 1u)];
+    };
+    int32_t* out = sig + b0 * H;
+    if (H % 4 == 0 && reinterpret_cast<uintptr_t>(sig) % 16 == 0) {  // four hashes of a bucket per thread and store
+        const int qpb = H >> 2;
+        for (int q = threadIdx.x; q < nb * qpb; q += 256) {
+            const int bl = q / qpb, h = (q - bl * qpb) << 2;
+            *reinterpret_cast<int4*>(out + 4 * q) =
+                make_int4(value(bl, h), value(bl, h + 1), value(bl, h + 2), value(bl, h + 3));
+        }
+    } else {
+        for (int i = threadIdx.x; i < nb * H; i += 256) {
+            const int bl = i / H;
+            out[i] = value(bl, i - bl * H);
+        }
     }
 }
 
@@ -170,6 +231,7 @@ culsh_status ps_build_codec(culsh_ctx* ctx, const int32_t* sig, int n, int T, in
     while ((1ll << bits) < rmax + 1) ++bits;  // codes 1..range, 0 reserved
     const int W = (H * bits + 31) / 32;
     if (bits > 12 || W >= H) return CULSH_OK;  // wide value ranges: keep the plain byte order keys
+    if (W > 56) return CULSH_OK;               // the restore kernel keeps PS_BPB keys of W words in LDS
 
     std::vector<int32_t> vmin(TH), range(TH), inv(static_cast<size_t>(TH) * rmax, 0);
     std::vector<uint32_t> fwd(static_cast<size_t>(TH) * rmax, 0);
@@ -211,12 +273,15 @@ culsh_status launch_ps_compress(culsh_ctx* ctx, const int32_t* sig, size_t rows,
     if (items == 0) return CULSH_OK;
     CULSH_REQUIRE(items / 256 < (1ull << 31), CULSH_ERR_LIMIT, "too many items");
     const PsCodec& pc = ix->psc;
+    const size_t lut_words = static_cast<size_t>(H) * pc.rmax;
+    const int use_lds = lut_words <= PS_LUT_WORDS;
+    const size_t lds = use_lds ? (lut_words + 2 * static_cast<size_t>(H)) * sizeof(uint32_t) : 0;
     if (H % 4 == 0 && reinterpret_cast<uintptr_t>(sig) % 16 == 0)
-        CULSH_LAUNCH(ctx, ps_compress_kernel<true>, dim3(div_up(items, 256)), dim3(256), 0, ctx->stream, sig, rows, T, H,
-                     pc.bits, pc.rmax, ix->key_w, pc.vmin, pc.range, pc.fwd, keys);
+        CULSH_LAUNCH(ctx, ps_compress_kernel<true>, dim3(div_up(items, 256)), dim3(256), lds, ctx->stream, sig, rows, T,
+                     H, pc.bits, pc.rmax, ix->key_w, use_lds, pc.vmin, pc.range, pc.fwd, keys);
     else
-        CULSH_LAUNCH(ctx, ps_compress_kernel<false>, dim3(div_up(items, 256)), dim3(256), 0, ctx->stream, sig, rows, T, H,
-                     pc.bits, pc.rmax, ix->key_w, pc.vmin, pc.range, pc.fwd, keys);
+        CULSH_LAUNCH(ctx, ps_compress_kernel<false>, dim3(div_up(items, 256)), dim3(256), lds, ctx->stream, sig, rows, T,
+                     H, pc.bits, pc.rmax, ix->key_w, use_lds, pc.vmin, pc.range, pc.fwd, keys);
     CULSH_LAUNCH_CHECK();
     return CULSH_OK;
 }
@@ -226,10 +291,13 @@ culsh_status launch_ps_keys_to_sig(culsh_ctx* ctx, const culsh_index* ix, size_t
     if (count == 0) return CULSH_OK;
     CULSH_REQUIRE(count / PS_BPB < (1ull << 31), CULSH_ERR_LIMIT, "too many buckets");
     const PsCodec& pc = ix->psc;
-    const size_t lds = static_cast<size_t>(PS_BPB) * (1 + ix->key_w) * sizeof(uint32_t);
+    const size_t lut_words = 2 * static_cast<size_t>(ix->n_hashes) * pc.rmax;
+    const int use_lds = lut_words <= PS_LUT_WORDS;
+    const size_t lds = (static_cast<size_t>(PS_BPB) * (1 + ix->key_w) + (use_lds ? lut_words : 0)) * sizeof(uint32_t);
+    CULSH_REQUIRE(lds <= 64 * 1024, CULSH_ERR_LIMIT, "key width too large for the signature restore kernel");
     CULSH_LAUNCH(ctx, ps_keys_to_sig_kernel, dim3(div_up(count, PS_BPB)), dim3(256), lds, ctx->stream, ix->bucket_keys,
                  count, count_dev, ix->table_bucket_offsets, ix->n_hash_tables, ix->n_hashes, pc.bits, pc.rmax,
-                 ix->key_w, pc.inv, reinterpret_cast<int32_t*>(sig));
+                 ix->key_w, use_lds, pc.inv, reinterpret_cast<int32_t*>(sig));
     CULSH_LAUNCH_CHECK();
     return CULSH_OK;
 }
