@@ -187,12 +187,17 @@ __global__ __launch_bounds__(NTHREADS, (BK <= 8 ? 5 : (BK <= 16 ? 4 : 3))) void 
             for (int i = 0; i < 2; ++i)
 #pragma unroll
                 for (int j = 0; j < 2; ++j)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[i][k], bf[j][k], acc[i][j], 0, 0, 0);
+                    // The key epilogue wants a lane to hold one column of its tile, the others one row
+                    // (four neighbouring hashes per register quad): those swap the operands and get
+                    // the transposed tile.
+                    acc[i][j] = (EPI == EPI_SIGN_KEYS)
+                                    ? __builtin_amdgcn_mfma_f32_32x32x2f32(af[i][k], bf[j][k], acc[i][j], 0, 0, 0)
+                                    : __builtin_amdgcn_mfma_f32_32x32x2f32(bf[j][k], af[i][k], acc[i][j], 0, 0, 0);
         __syncthreads();
     }
 
     // Accumulator layout of the 32x32 tile: register v of lane l holds
-    // row 8*(v/4) + 4*(l/32) + v%4, column l%32.
+    // row 8*(v/4) + 4*(l/32) + v%4, column l%32 of (first operand) x (second operand).
     if (EPI == EPI_SIGN_KEYS) {
 #pragma unroll
         for (int i = 0; i < 2; ++i)
@@ -251,28 +256,71 @@ __global__ __launch_bounds__(NTHREADS, (BK <= 8 ? 5 : (BK <= 16 ? 4 : 3))) void 
             }
         }
     } else {
+        // Transposed tiles: registers 4g..4g+3 of lane l hold row l%32, columns 8g + 4*(l/32) + 0..3.
+        // When H is a multiple of 4 those are four neighbouring hashes of one table, stored at once;
+        // the 32 lanes of a half wave then cover 32 consecutive rows, H * 4 bytes apart.
+        const bool quad = (H & 3) == 0 && (reinterpret_cast<uintptr_t>(a.out) & 15) == 0 &&
+                          (EPI != EPI_FLOOR_I32 || (reinterpret_cast<uintptr_t>(a.b) & 15) == 0);
 #pragma unroll
-        for (int i = 0; i < 2; ++i)
+        for (int j = 0; j < 2; ++j) {
+            const int cb = ct * BN + wn * 64 + j * 32 + 4 * half;  // column of register 0
+            int t = cb / H, h = cb - t * H;
 #pragma unroll
-            for (int j = 0; j < 2; ++j) {
-                const int col = ct * BN + wn * 64 + j * 32 + r32;
-                if (col >= TH) continue;
-                const int t = col / H, h = col - t * H;
-                const float bias = (EPI == EPI_FLOOR_I32) ? a.b[col] : 0.f;
+            for (int g = 0; g < 4; ++g) {
+                const int c0 = cb + 8 * g;
+                if (quad) {
+                    if (c0 < TH) {
+                        float4 bias = make_float4(0.f, 0.f, 0.f, 0.f);
+                        if (EPI == EPI_FLOOR_I32) bias = *reinterpret_cast<const float4*>(a.b + c0);
 #pragma unroll
-                for (int v = 0; v < 16; ++v) {
-                    const int row = rt * BM + wm * 64 + i * 32 + 8 * (v >> 2) + 4 * half + (v & 3);
-                    if (row >= n) continue;
-                    const size_t off = (static_cast<size_t>(t) * n + row) * H + h;
-                    const float x = acc[i][j][v];
-                    if (EPI == EPI_SIGN_BYTES) {
-                        static_cast<uint8_t*>(a.out)[off] =
-                            static_cast<uint8_t>((__float_as_uint(x) >> 31) ^ 1u);
-                    } else {
-                        static_cast<int32_t*>(a.out)[off] = static_cast<int32_t>(floorf(x + bias));  // pslsh/hash.cuh:46
+                        for (int i = 0; i < 2; ++i) {
+                            const int row = rt * BM + wm * 64 + i * 32 + r32;
+                            if (row >= n) continue;
+                            const size_t off = (static_cast<size_t>(t) * n + row) * H + h;
+                            const float x0 = acc[i][j][4 * g], x1 = acc[i][j][4 * g + 1];
+                            const float x2 = acc[i][j][4 * g + 2], x3 = acc[i][j][4 * g + 3];
+                            if (EPI == EPI_SIGN_BYTES) {
+                                const uint32_t bytes = ((__float_as_uint(x0) >> 31) ^ 1u) |
+                                                       (((__float_as_uint(x1) >> 31) ^ 1u) << 8) |
+                                                       (((__float_as_uint(x2) >> 31) ^ 1u) << 16) |
+                                                       (((__float_as_uint(x3) >> 31) ^ 1u) << 24);
+                                *reinterpret_cast<uint32_t*>(static_cast<uint8_t*>(a.out) + off) = bytes;
+                            } else {  // pslsh/hash.cuh:46
+                                *reinterpret_cast<int4*>(static_cast<int32_t*>(a.out) + off) =
+                                    make_int4(static_cast<int32_t>(floorf(x0 + bias.x)),
+                                              static_cast<int32_t>(floorf(x1 + bias.y)),
+                                              static_cast<int32_t>(floorf(x2 + bias.z)),
+                                              static_cast<int32_t>(floorf(x3 + bias.w)));
+                            }
+                        }
+                    }
+                } else {
+                    int tq = t, hq = h;
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        if (c0 + q < TH) {
+                            const float bias = (EPI == EPI_FLOOR_I32) ? a.b[c0 + q] : 0.f;
+#pragma unroll
+                            for (int i = 0; i < 2; ++i) {
+                                const int row = rt * BM + wm * 64 + i * 32 + r32;
+                                if (row >= n) continue;
+                                const size_t off = (static_cast<size_t>(tq) * n + row) * H + hq;
+                                const float x = acc[i][j][4 * g + q];
+                                if (EPI == EPI_SIGN_BYTES) {
+                                    static_cast<uint8_t*>(a.out)[off] =
+                                        static_cast<uint8_t>((__float_as_uint(x) >> 31) ^ 1u);
+                                } else {
+                                    static_cast<int32_t*>(a.out)[off] = static_cast<int32_t>(floorf(x + bias));
+                                }
+                            }
+                        }
+                        if (++hq == H) { hq = 0; ++tq; }
                     }
                 }
+                h += 8;
+                while (h >= H) { h -= H; ++t; }
             }
+        }
     }
 }
 
