@@ -578,7 +578,7 @@ static culsh_status minhash_fit_once(culsh_ctx* ctx, const int32_t* indices, con
         enc = ENC_MHR;
         W = ix->key_w;
         CULSH_TRY(arena_alloc_t(ctx, N * W, &keys));
-        CULSH_TRY(launch_minhash_rank(ctx, indices, indptr, n, nT, H, ix.get(), keys));
+        CULSH_TRY(launch_minhash_rank(ctx, indices, indptr, n, nT, H, ix.get(), true, keys));
     } else {
         CULSH_TRY(arena_alloc_t(ctx, N * H, &keys));
         CULSH_TRY(launch_minhash(ctx, indices, indptr, ix->A, ix->B, n, nT, H, true, keys));
@@ -874,7 +874,7 @@ culsh_status culsh_minhash_query(culsh_ctx* ctx, const int32_t* indices, const i
     uint32_t* keys = nullptr;
     if (ix->enc == ENC_MHR) {
         CULSH_TRY(arena_alloc_t(ctx, static_cast<size_t>(nq) * T * ix->key_w, &keys));
-        CULSH_TRY(launch_minhash_rank(ctx, indices, indptr, nq, T, H, ix, keys));
+        CULSH_TRY(launch_minhash_rank(ctx, indices, indptr, nq, T, H, ix, false, keys));
     } else {
         CULSH_TRY(arena_alloc_t(ctx, static_cast<size_t>(nq) * T * H, &keys));
         CULSH_TRY(launch_minhash(ctx, indices, indptr, ix->A, ix->B, nq, T, H, true, keys));

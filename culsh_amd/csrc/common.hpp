@@ -267,9 +267,10 @@ void free_ps_codec(culsh_index* ix);
 // reports used = true.  May return CULSH_RETRY_UNCHAINED (its column sort is a chained radix sort).
 culsh_status mh_build_codec(culsh_ctx* ctx, const int32_t* indices, size_t nnz, int T, int H, int d, culsh_index* ix,
                             bool* used);
-// CSR rows -> packed rank codes [T][n][ix->key_w]
+// CSR rows -> packed rank codes [T][n][ix->key_w].  `ids_below_d`: the caller has checked that every
+// column id is below the codec's n_features (a cheaper hash applies to small ids).
 culsh_status launch_minhash_rank(culsh_ctx* ctx, const int32_t* indices, const int32_t* indptr, int n, int T, int H,
-                                 const culsh_index* ix, uint32_t* keys);
+                                 const culsh_index* ix, bool ids_below_d, uint32_t* keys);
 // uint32 signatures [T][rows][H] -> packed rank codes
 culsh_status launch_mh_sig_to_keys(culsh_ctx* ctx, const uint32_t* sig, size_t rows, const culsh_index* ix,
                                    uint32_t* keys);

@@ -30,6 +30,15 @@ __device__ __forceinline__ uint32_t hash_mod_p(uint32_t a, uint32_t x, uint32_t 
     return static_cast<uint32_t>(v2 >= PRIME ? v2 - PRIME : v2);
 }
 
+// The same for x < 2^25: a*x + b < 2^57, so the first fold leaves less than 2^32 + 5 * 2^25 and a
+// second fold could only add 5 once: it is merged with the final subtraction.
+__device__ __forceinline__ uint32_t hash_mod_p_small(uint32_t a, uint32_t x, uint32_t b) {
+    const uint64_t v = static_cast<uint64_t>(a) * x + b;
+    const uint64_t v1 = 5ull * (v >> 32) + (v & 0xFFFFFFFFull);
+    const uint32_t lo = static_cast<uint32_t>(v1);
+    return v1 >= PRIME ? lo + 5u : lo;
+}
+
 __global__ __launch_bounds__(256) void mh_max_index_kernel(const int32_t* __restrict__ indices, size_t nnz,
                                                           uint32_t* __restrict__ out_max) {
     uint32_t m = 0;  // negative ids read as huge values: out of range
@@ -80,7 +89,8 @@ constexpr int NTHREADS = 256;
 // MinHash of CSR rows written as packed rank codes (role of compute_minhash_kernel,
 // minhash/hash.cuh:69-128, plus the key packing).  Same work split as minhash_kernel: items are
 // (row, hash) pairs with hashes fastest; besides the running minimum a thread keeps the column
-// that produced it.
+// that produced it.  SMALL: every column id is below 2^25.
+template <bool SMALL>
 __global__ __launch_bounds__(NTHREADS) void minhash_rank_kernel(const int32_t* __restrict__ indices,
                                                                const int32_t* __restrict__ indptr,
                                                                const uint32_t* __restrict__ A,
@@ -94,13 +104,13 @@ __global__ __launch_bounds__(NTHREADS) void minhash_rank_kernel(const int32_t* _
     const int rows = min(RB, n - row0);
     for (int c0 = 0; c0 < TH; c0 += th_chunk) {
         const int nc = min(th_chunk, TH - c0);
-        for (int item = threadIdx.x; item < rows * nc; item += NTHREADS) {
-            const int r = item / nc, c = item - r * nc;
+        // (row r, hash c0 + c) -> stage[c][r]
+        auto one = [&](int r, int c) {
             const int s = indptr[row0 + r], e = indptr[row0 + r + 1];
             const uint32_t a = A[c0 + c], b = B[c0 + c];
             uint32_t m = 0xFFFFFFFFu, col = 0xFFFFFFFFu;
             auto take = [&](uint32_t f) {
-                const uint32_t h = hash_mod_p(a, f, b);
+                const uint32_t h = SMALL ? hash_mod_p_small(a, f, b) : hash_mod_p(a, f, b);
                 const bool less = h < m;
                 m = less ? h : m;
                 col = less ? f : col;
@@ -119,6 +129,19 @@ __global__ __launch_bounds__(NTHREADS) void minhash_rank_kernel(const int32_t* _
             if (s < e) code = col < static_cast<uint32_t>(d) ? rank[static_cast<size_t>(c0 + c) * d + col]
                                                               : static_cast<uint32_t>(d) + 1u;  // matches nothing
             stage[c * RB + r] = code;
+        };
+        if ((nc & 63) == 0) {
+            // every wavefront works on one row at a time: saying so lets the row's column ids be fetched
+            // once per wavefront, through the scalar unit
+            for (int item = threadIdx.x; item < rows * nc; item += NTHREADS) {
+                const int r = item / nc;
+                one(__builtin_amdgcn_readfirstlane(r), item - r * nc);
+            }
+        } else {
+            for (int item = threadIdx.x; item < rows * nc; item += NTHREADS) {
+                const int r = item / nc;
+                one(r, item - r * nc);
+            }
         }
         __syncthreads();
         // one thread per (table, row): pack the H codes of the table MSB first
@@ -283,15 +306,19 @@ culsh_status mh_build_codec(culsh_ctx* ctx, const int32_t* indices, size_t nnz, 
 }
 
 culsh_status launch_minhash_rank(culsh_ctx* ctx, const int32_t* indices, const int32_t* indptr, int n, int T, int H,
-                                 const culsh_index* ix, uint32_t* keys) {
+                                 const culsh_index* ix, bool ids_below_d, uint32_t* keys) {
     CULSH_REQUIRE(indptr && keys && ix->mhc.rank, CULSH_ERR_INVALID, "minhash: null pointer");
     CULSH_REQUIRE(n > 0, CULSH_ERR_INVALID, "minhash: sizes must be positive");
     CULSH_REQUIRE(H <= 384, CULSH_ERR_LIMIT, "minhash: n_hashes > 384 is not supported");
     int tables_per_chunk = static_cast<int>(std::min<long long>(T, std::max(1, (12288 / RB) / H)));
     const int th_chunk = tables_per_chunk * H;
     const size_t lds = static_cast<size_t>(th_chunk) * RB * sizeof(uint32_t);
-    CULSH_LAUNCH(ctx, minhash_rank_kernel, dim3((n + RB - 1) / RB), dim3(NTHREADS), lds, ctx->stream, indices, indptr,
-                 ix->A, ix->B, ix->mhc.rank, n, T, H, ix->mhc.d, ix->mhc.bits, ix->key_w, th_chunk, keys);
+    if (ids_below_d && ix->mhc.d <= (1 << 25))
+        CULSH_LAUNCH(ctx, minhash_rank_kernel<true>, dim3((n + RB - 1) / RB), dim3(NTHREADS), lds, ctx->stream, indices,
+                     indptr, ix->A, ix->B, ix->mhc.rank, n, T, H, ix->mhc.d, ix->mhc.bits, ix->key_w, th_chunk, keys);
+    else
+        CULSH_LAUNCH(ctx, minhash_rank_kernel<false>, dim3((n + RB - 1) / RB), dim3(NTHREADS), lds, ctx->stream, indices,
+                     indptr, ix->A, ix->B, ix->mhc.rank, n, T, H, ix->mhc.d, ix->mhc.bits, ix->key_w, th_chunk, keys);
     CULSH_LAUNCH_CHECK();
     return CULSH_OK;
 }
