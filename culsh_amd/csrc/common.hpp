@@ -80,6 +80,7 @@ struct MhCodec {
     int d = 0;                 // n_features; codes: 0..d-1 ranks, d = empty row, d+1 = matches nothing
     uint32_t* rank = nullptr;  // [T*H][d] column -> rank of its hash value (signature byte order)
     uint32_t* inv = nullptr;   // [T*H][d] rank -> hash value
+    uint32_t* ainv = nullptr;  // [T*H] inverse of the multiplier modulo the prime (0: multiplier is a multiple of it)
 };
 
 }  // namespace culsh_amd

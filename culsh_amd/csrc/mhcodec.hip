@@ -62,6 +62,20 @@ __global__ __launch_bounds__(256) void mh_max_index_kernel(const int32_t* __rest
     if ((threadIdx.x & 63) == 0 && m > __atomic_load_n(out_max, __ATOMIC_RELAXED)) atomicMax(out_max, m);
 }
 
+// ainv[c] = A[c]^(p-2) mod p: the inverse of the multiplier, with which the column that produced a
+// hash value is recovered from the value (the hash is a bijection of [0, p) unless A[c] = 0 mod p)
+__global__ __launch_bounds__(256) void mh_inverse_kernel(const uint32_t* __restrict__ A, int count,
+                                                        uint32_t* __restrict__ ainv) {
+    const int c = blockIdx.x * 256 + threadIdx.x;
+    if (c >= count) return;
+    uint32_t base = hash_mod_p(A[c], 1u, 0u), acc = 1u;
+    for (uint32_t e = PRIME - 2u; e; e >>= 1) {
+        if (e & 1u) acc = hash_mod_p(acc, base, 0u);
+        base = hash_mod_p(base, base, 0u);
+    }
+    ainv[c] = acc;  // 0 for a multiplier that is 0 mod p (p - 2 is odd, so the first step already gives 0)
+}
+
 // keys[c][f] = byte-order form of hash_c(f): the sort then ranks columns in signature byte order
 __global__ __launch_bounds__(256) void mh_hash_columns_kernel(const uint32_t* __restrict__ A,
                                                              const uint32_t* __restrict__ B, int d,
@@ -79,7 +93,9 @@ __global__ __launch_bounds__(256) void mh_invert_kernel(const int32_t* __restric
     if (i >= total) return;
     const size_t c = i / d;
     const uint32_t r = static_cast<uint32_t>(i - c * d);
-    rank[c * d + static_cast<uint32_t>(sorted_cols[i])] = r;
+    // A multiplier that is 0 mod p gives every column the same value, hence the same rank (0); any
+    // other multiplier gives d different values.
+    rank[c * d + static_cast<uint32_t>(sorted_cols[i])] = sorted_keys[i] == sorted_keys[c * d] ? 0u : r;
     inv[i] = __builtin_bswap32(sorted_keys[i]);
 }
 
@@ -89,12 +105,14 @@ constexpr int NTHREADS = 256;
 // MinHash of CSR rows written as packed rank codes (role of compute_minhash_kernel,
 // minhash/hash.cuh:69-128, plus the key packing).  Same work split as minhash_kernel: items are
 // (row, hash) pairs with hashes fastest; besides the running minimum a thread keeps the column
-// that produced it.  SMALL: every column id is below 2^25.
+// that produced it.  SMALL: every column id is below 2^25; then only the minimum is kept and
+// its column is computed from it at the end, ainv * (min - b) mod p.
 template <bool SMALL>
 __global__ __launch_bounds__(NTHREADS) void minhash_rank_kernel(const int32_t* __restrict__ indices,
                                                                const int32_t* __restrict__ indptr,
                                                                const uint32_t* __restrict__ A,
                                                                const uint32_t* __restrict__ B,
+                                                               const uint32_t* __restrict__ ainv,
                                                                const uint32_t* __restrict__ rank, int n, int T, int H,
                                                                int d, int bits, int W, int th_chunk,
                                                                uint32_t* __restrict__ out) {
@@ -110,10 +128,14 @@ __global__ __launch_bounds__(NTHREADS) void minhash_rank_kernel(const int32_t* _
             const uint32_t a = A[c0 + c], b = B[c0 + c];
             uint32_t m = 0xFFFFFFFFu, col = 0xFFFFFFFFu;
             auto take = [&](uint32_t f) {
-                const uint32_t h = SMALL ? hash_mod_p_small(a, f, b) : hash_mod_p(a, f, b);
-                const bool less = h < m;
-                m = less ? h : m;
-                col = less ? f : col;
+                if (SMALL) {
+                    m = min(m, hash_mod_p_small(a, f, b));
+                } else {
+                    const uint32_t h = hash_mod_p(a, f, b);
+                    const bool less = h < m;
+                    m = less ? h : m;
+                    col = less ? f : col;
+                }
             };
             int j = s;
             for (; j + 4 <= e; j += 4) {  // four loads in flight, then four hash chains
@@ -125,6 +147,12 @@ __global__ __launch_bounds__(NTHREADS) void minhash_rank_kernel(const int32_t* _
                 take(f3);
             }
             for (; j < e; ++j) take(static_cast<uint32_t>(indices[j]));
+            if (SMALL && s < e) {
+                const uint32_t ai = ainv[c0 + c];
+                const uint32_t bp = b >= PRIME ? b - PRIME : b;
+                const uint32_t x = m - bp + (m < bp ? PRIME : 0u);  // (m - b) mod p; wraps to the exact value
+                col = ai ? hash_mod_p(ai, x, 0u) : static_cast<uint32_t>(indices[s]);  // all hashes equal: the first stays
+            }
             uint32_t code = static_cast<uint32_t>(d);                      // empty row: sorts last
             if (s < e) code = col < static_cast<uint32_t>(d) ? rank[static_cast<size_t>(c0 + c) * d + col]
                                                               : static_cast<uint32_t>(d) + 1u;  // matches nothing
@@ -190,6 +218,7 @@ __global__ __launch_bounds__(256) void mh_sig_to_keys_kernel(const uint32_t* __r
             const uint32_t* tab = inv + static_cast<size_t>(t * H + h) * d;
             const uint32_t key = __builtin_bswap32(v);
             int lo = 0, hi = d - 1;
+            if (__builtin_bswap32(tab[0]) == key) { code = 0u; hi = -1; }  // also the rank of a constant hash
             while (lo <= hi) {
                 const int mid = lo + ((hi - lo) >> 1);
                 const uint32_t mk = __builtin_bswap32(tab[mid]);
@@ -249,6 +278,7 @@ __global__ __launch_bounds__(256) void mh_keys_to_sig_kernel(const uint32_t* __r
 void free_mh_codec(culsh_index* ix) {
     dev_free(ix->mhc.rank);
     dev_free(ix->mhc.inv);
+    dev_free(ix->mhc.ainv);
     ix->mhc = MhCodec();
 }
 
@@ -288,8 +318,12 @@ culsh_status mh_build_codec(culsh_ctx* ctx, const int32_t* indices, size_t nnz, 
     MhCodec& mc = ix->mhc;
     CULSH_HIP(dev_malloc(&mc.rank, total * sizeof(uint32_t)));
     CULSH_HIP(dev_malloc(&mc.inv, total * sizeof(uint32_t)));
+    CULSH_HIP(dev_malloc(&mc.ainv, TH * sizeof(uint32_t)));
     CULSH_LAUNCH(ctx, mh_invert_kernel, dim3(div_up(total, 256)), dim3(256), 0, ctx->stream, cols, sorted, total, d,
                  mc.rank, mc.inv);
+    CULSH_LAUNCH_CHECK();
+    CULSH_LAUNCH(ctx, mh_inverse_kernel, dim3(div_up(TH, 256)), dim3(256), 0, ctx->stream, ix->A, static_cast<int>(TH),
+                 mc.ainv);
     CULSH_LAUNCH_CHECK();
     if (ctx->sort_err_dev) {  // the column sort used the chained scan: its flag is settled here
         uint32_t gave_up = 0;
@@ -315,10 +349,10 @@ culsh_status launch_minhash_rank(culsh_ctx* ctx, const int32_t* indices, const i
     const size_t lds = static_cast<size_t>(th_chunk) * RB * sizeof(uint32_t);
     if (ids_below_d && ix->mhc.d <= (1 << 25))
         CULSH_LAUNCH(ctx, minhash_rank_kernel<true>, dim3((n + RB - 1) / RB), dim3(NTHREADS), lds, ctx->stream, indices,
-                     indptr, ix->A, ix->B, ix->mhc.rank, n, T, H, ix->mhc.d, ix->mhc.bits, ix->key_w, th_chunk, keys);
+                     indptr, ix->A, ix->B, ix->mhc.ainv, ix->mhc.rank, n, T, H, ix->mhc.d, ix->mhc.bits, ix->key_w, th_chunk, keys);
     else
         CULSH_LAUNCH(ctx, minhash_rank_kernel<false>, dim3((n + RB - 1) / RB), dim3(NTHREADS), lds, ctx->stream, indices,
-                     indptr, ix->A, ix->B, ix->mhc.rank, n, T, H, ix->mhc.d, ix->mhc.bits, ix->key_w, th_chunk, keys);
+                     indptr, ix->A, ix->B, ix->mhc.ainv, ix->mhc.rank, n, T, H, ix->mhc.d, ix->mhc.bits, ix->key_w, th_chunk, keys);
     CULSH_LAUNCH_CHECK();
     return CULSH_OK;
 }

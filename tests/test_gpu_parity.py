@@ -649,6 +649,18 @@ def test_minhash_rank_keys_edge_cases(ctx):
     assert_candidates_match(ctx.core_query_index(qsig, ih), exp)          # raw signatures -> rank keys
     np.testing.assert_array_equal(ctx.core_find_matching_buckets(qsig, ih), o.find_matching_buckets_fast(qsig, exp_ix))
     ctx.free_index(ih)
+    # multipliers that are 0 modulo the prime (every column hashes alike), at and above the prime, and
+    # offsets at and above it: the column of the minimum is still the one the reference's scan keeps
+    A3, B3 = A.copy(), B.copy()
+    A3[0], A3[1], A3[2], A3[3] = 0, 4294967291, 4294967295, 1
+    B3[0], B3[2], B3[4] = 4294967295, 4294967291, 0
+    sig3 = o.minhash_hash(indices, indptr, A3, B3, T, H)
+    ih3 = ctx.minhash_fit(indices, indptr, d, T, H, A=A3, B=B3)
+    exp_ix3 = o.fit_index(sig3, H)
+    assert_index_matches(ctx.index_arrays(ih3), exp_ix3)
+    qsig3 = o.minhash_hash(qindices, qindptr, A3, B3, T, H)
+    assert_candidates_match(ctx.minhash_query(qindices, qindptr, ih3), o.query_index(qsig3, exp_ix3))
+    ctx.free_index(ih3)
     # a fitted row with a column id >= n_features: every id is hashed as it is (minhash/hash.cuh:97-104)
     bad = indices.copy()
     bad[7] = d + 123
