@@ -14,7 +14,11 @@
 // workgroup publishes its count and obtains the sum of its predecessors' counts by
 // looking back over their published values (a chained scan), then stores its list.  The
 // output is allocated for the number of raw candidates, an upper bound of the result.
-// Larger row ranges take two launches (count, scan, emit) with several passes each.
+// Larger row ranges take several passes per query, in the same launch: a query's spans
+// shrink from pass to pass (rows ascend inside a bucket), its list is written where its raw
+// candidates would start (no workgroup waits for another), and a copy closes the gaps
+// between the lists afterwards.  A path of two launches (count, scan, emit) with no
+// cooperation between workgroups stands behind both.
 #include <algorithm>
 #include <cstdlib>
 #include <vector>
@@ -93,6 +97,30 @@ __global__ __launch_bounds__(256) void span_kernel(const int32_t* __restrict__ m
     if (threadIdx.x == 0 && block_raw) atomicAdd(raw_total, block_raw);
 }
 
+// Raw candidates per query: the sum of its span lengths.
+__global__ __launch_bounds__(256) void raw_counts_kernel(const int2* __restrict__ spans, int n_queries, int T,
+                                                        uint64_t* __restrict__ raw_counts) {
+    const int q = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+    if (q >= n_queries) return;
+    unsigned long long sum = 0;
+    for (int t = lane; t < T; t += 64) sum += static_cast<unsigned long long>(spans[static_cast<size_t>(q) * T + t].y);
+    sum = wave_sum(sum);
+    if (lane == 0) raw_counts[q] = sum;
+}
+
+// Closes the gaps between the queries' lists: list q moves from src_offsets[q] to dst_offsets[q].
+__global__ __launch_bounds__(256) void close_gaps_kernel(const int32_t* __restrict__ src,
+                                                        const uint64_t* __restrict__ src_offsets,
+                                                        const uint64_t* __restrict__ dst_offsets,
+                                                        const uint64_t* __restrict__ counts,
+                                                        int32_t* __restrict__ dst) {
+    const int q = blockIdx.x;
+    const int32_t* from = src + src_offsets[q];
+    int32_t* to = dst + dst_offsets[q];
+    const uint64_t count = counts[q];
+    for (uint64_t i = threadIdx.x; i < count; i += 256) to[i] = from[i];
+}
+
 constexpr int NWAVES = DD_THREADS / 64;
 constexpr int WALK_U = 16;  // pieces in flight per wavefront
 
@@ -102,10 +130,13 @@ constexpr int WALK_U = 16;  // pieces in flight per wavefront
 // starts is looked up once per piece (one binary search per thread over the spans'
 // piece counts, all pieces of a round in parallel) and kept in `tab`, so the per-lane
 // work is an add, a compare and the load.  Contains barriers: all threads must call it.
-template <typename F>
+// TALLY: also counts, per span, the visited rows below `row_end` into s_cnt (zero on entry); the
+// rows of a span ascend, so that count is how far the span's next pass may skip.
+template <bool TALLY, typename F>
 __device__ __forceinline__ void walk_candidates(const int32_t* __restrict__ cand, const int* s_start,
                                                 const int* s_len, const uint32_t* s_ppref, int T,
-                                                uint32_t n_pieces, int2* tab, F&& f) {
+                                                uint32_t n_pieces, int2* tab, uint32_t row_end, int* s_cnt,
+                                                F&& f) {
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     for (uint32_t r0 = 0; r0 < n_pieces; r0 += DD_THREADS) {
         const uint32_t pc = r0 + static_cast<uint32_t>(tid);
@@ -116,7 +147,8 @@ __device__ __forceinline__ void walk_candidates(const int32_t* __restrict__ cand
                 if (s_ppref[mid] <= pc) tl = mid; else th = mid;
             }
             const int first = static_cast<int>(pc - s_ppref[tl]) * 64;
-            tab[tid] = make_int2(s_start[tl] + first, min(64, s_len[tl] - first));
+            // (length, span) share a word: lengths are at most 64
+            tab[tid] = make_int2(s_start[tl] + first, min(64, s_len[tl] - first) | (tl << 8));
         }
         __syncthreads();
         const uint32_t here = min(static_cast<uint32_t>(DD_THREADS), n_pieces - r0);
@@ -128,18 +160,26 @@ __device__ __forceinline__ void walk_candidates(const int32_t* __restrict__ cand
                 rows[u] = -1;
                 if (pi < here) {  // uniform across the wavefront
                     const int2 e = tab[pi];
-                    if (lane < e.y) rows[u] = cand[e.x + lane];
+                    if (lane < (e.y & 255)) rows[u] = cand[e.x + lane];
                 }
             }
 #pragma unroll
-            for (int u = 0; u < WALK_U; ++u)
+            for (int u = 0; u < WALK_U; ++u) {
                 if (rows[u] >= 0) f(rows[u]);
+                if (TALLY) {
+                    const uint32_t pi = p0 + u * NWAVES;
+                    if (pi < here) {
+                        const unsigned long long below = __ballot(static_cast<uint32_t>(rows[u]) < row_end);  // -1 is not
+                        if (lane == 0 && below) atomicAdd(&s_cnt[tab[pi].y >> 8], __popcll(below));
+                    }
+                }
+            }
         }
         __syncthreads();  // tab is rewritten by the next round
     }
 }
 
-enum DedupMode { DD_COUNT = 0, DD_EMIT = 1, DD_FUSED = 2 };
+enum DedupMode { DD_COUNT = 0, DD_EMIT = 1, DD_FUSED = 2, DD_FUSED_PASSES = 3 };  // FUSED: one bitmap pass per query
 
 struct DedupArgs {
     const int2* spans;            // [n_queries][T] (start, length) in `cand`
@@ -147,13 +187,14 @@ struct DedupArgs {
     int32_t* out;                 // EMIT, FUSED: candidate indices
     uint64_t* counts;             // COUNT, FUSED: per-query unique counts (written)
     uint64_t* offsets;            // EMIT: per-query output offsets (read); FUSED: [n_queries+1] (written)
-    unsigned long long* state;    // FUSED: [n_queries] published counts / running sums, zero before the launch
+    unsigned long long* state;    // FUSED, one pass: [n_queries] published counts / running sums, zero before the launch
+    const uint64_t* raw_offsets;  // FUSED, several passes: [n_queries] where a query's list starts in `out` (spaced by raw counts)
     unsigned int* err;            // FUSED: set when the look-back gave up or the output would overflow
     unsigned int* ticket;         // FUSED: next query to hand out (workgroups stay and take queries in order)
     unsigned long long capacity;  // FUSED: elements available in `out`
     int T, n_queries;
     int wpt;       // bitmap words per thread (power of two); a pass covers DD_THREADS*wpt*32 rows
-    int n_chunks;  // passes over the row range (FUSED: 1)
+    int n_chunks;  // passes over the row range
     int spin_limit;  // FUSED: polls of an unpublished predecessor before giving up
     unsigned long long* ticks;  // optional [n_queries][8] phase timers (wall clock ticks of thread 0), or null
 };
@@ -220,6 +261,7 @@ __device__ __forceinline__ void load_step_words(const uint32_t* p, int ew, uint3
 // never reach memory.
 template <int MODE>
 __global__ __launch_bounds__(DD_THREADS) void dedup_kernel(DedupArgs a) {
+    constexpr bool FUSED = MODE == DD_FUSED || MODE == DD_FUSED_PASSES;
     extern __shared__ uint32_t lds[];
     const int T = a.T, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int chunk_words = DD_THREADS * a.wpt;                  // multiple of 1024
@@ -232,6 +274,7 @@ __global__ __launch_bounds__(DD_THREADS) void dedup_kernel(DedupArgs a) {
     uint32_t* s_ppref = reinterpret_cast<uint32_t*>(s_len + T);  // [T+1]
     uint32_t* scratch = s_ppref + T + 1;                         // [17]
     uint32_t* wtot = scratch + 17;                               // [NWAVES + 1]
+    int* s_cnt = reinterpret_cast<int*>(wtot + NWAVES + 1);      // [T] FUSED with several passes: rows of the pass, per span
 
 #define DD_TICK(k)                                                                      \
     if (a.ticks && tid == 0) {                                                          \
@@ -246,12 +289,12 @@ __global__ __launch_bounds__(DD_THREADS) void dedup_kernel(DedupArgs a) {
     // taken by a running workgroup; the next ticket and its spans are fetched under the current
     // query's read-out.
     int q = blockIdx.x;
-    if (MODE == DD_FUSED && tid == 0) *sh_q = static_cast<int>(atomicAdd(a.ticket, 1u));
+    if (FUSED && tid == 0) *sh_q = static_cast<int>(atomicAdd(a.ticket, 1u));
     {   // the bitmap is cleared while the first loads are in flight; FUSED keeps it clean afterwards
         uint4* bm4 = reinterpret_cast<uint4*>(bm);
         for (int i = tid; i < chunk_words / 4; i += DD_THREADS) bm4[i] = make_uint4(0u, 0u, 0u, 0u);
     }
-    if (MODE == DD_FUSED) {
+    if (FUSED) {
         __syncthreads();
         q = *sh_q;
         if (q >= a.n_queries) return;
@@ -275,19 +318,26 @@ __global__ __launch_bounds__(DD_THREADS) void dedup_kernel(DedupArgs a) {
     const uint64_t out_base = MODE == DD_EMIT ? a.offsets[q] : 0;
     const uint32_t chunk_rows = static_cast<uint32_t>(chunk_words) * 32u;
 
+    // FUSED with several passes: a query's list starts where its raw candidates would (no dependence
+    // on other queries, the host closes the gaps afterwards), and the spans shrink from pass to pass
+    // by the rows already written.
+    constexpr bool several = MODE == DD_FUSED_PASSES;
+    const unsigned long long raw_base = several ? a.raw_offsets[q] : 0ull;
     for (int chunk = 0; chunk < a.n_chunks; ++chunk) {
         const uint32_t lo = static_cast<uint32_t>(chunk) * chunk_rows;
-        if (chunk > 0) {
+        const bool last = MODE == DD_FUSED || chunk == a.n_chunks - 1;  // DD_FUSED is launched for one pass only
+        if (chunk > 0 && !FUSED) {  // FUSED leaves the bitmap clean after every read-out
             uint4* bm4 = reinterpret_cast<uint4*>(bm);
             for (int i = tid; i < chunk_words / 4; i += DD_THREADS) bm4[i] = make_uint4(0u, 0u, 0u, 0u);
         }
         if (tid <= NWAVES) wtot[tid] = 0;
+        if (several && tid < T) s_cnt[tid] = 0;
         __syncthreads();
         DD_TICK(0)  // setup + clear
         // Mark the rows of this pass (collect_candidates_kernel, core/query.cuh:199-237, but into
         // the bitmap instead of memory).  Rows outside [lo, lo + chunk_rows) belong to another pass.
         uint32_t fresh = 0;  // COUNT: bits this thread set first
-        walk_candidates(a.cand, s_start, s_len, s_ppref, T, n_pieces, tab, [&](int row) {
+        auto mark = [&](int row) {
             const uint32_t bit = static_cast<uint32_t>(row) - lo;
             if (bit < chunk_rows) {
                 const uint32_t m = 1u << (bit & 31u);
@@ -297,7 +347,23 @@ __global__ __launch_bounds__(DD_THREADS) void dedup_kernel(DedupArgs a) {
                     atomicOr(&bm[bit >> 5], m);
                 }
             }
-        });
+        };
+        if (several && !last) {
+            walk_candidates<true>(a.cand, s_start, s_len, s_ppref, T, n_pieces, tab, lo + chunk_rows, s_cnt, mark);
+            // the next pass starts behind the rows of this one (the walk ended with a barrier, or saw nothing)
+            uint32_t pieces = 0;
+            if (tid < T) {
+                const int c = s_cnt[tid];
+                s_start[tid] += c;
+                s_len[tid] -= c;
+                pieces = (static_cast<uint32_t>(s_len[tid]) + 63u) >> 6;
+            }
+            const uint32_t ex = block_exclusive_sum(pieces, scratch, &n_pieces);
+            if (tid < T) s_ppref[tid] = ex;
+            if (tid == 0) s_ppref[T] = n_pieces;
+        } else {
+            walk_candidates<false>(a.cand, s_start, s_len, s_ppref, T, n_pieces, tab, 0u, nullptr, mark);
+        }
         DD_TICK(1)  // gather
         if (MODE == DD_COUNT) {
             // a row is counted by whichever lane set its bit first
@@ -343,10 +409,11 @@ __global__ __launch_bounds__(DD_THREADS) void dedup_kernel(DedupArgs a) {
         // queries can go on, and looks back only after lining up its own rows.
         DD_TICK(4)
         unsigned int ticket_next = 0;
-        if (MODE == DD_FUSED && wave == 0 && lane == 0) {
-            __hip_atomic_store(&a.state[q], TAG_COUNT | static_cast<unsigned long long>(chunk_total), __ATOMIC_RELAXED,
-                               __HIP_MEMORY_SCOPE_AGENT);
-            ticket_next = atomicAdd(a.ticket, 1u);  // arrives while the rows are lined up
+        if (FUSED && wave == 0 && lane == 0) {
+            if (!several)
+                __hip_atomic_store(&a.state[q], TAG_COUNT | static_cast<unsigned long long>(chunk_total),
+                                   __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (last) ticket_next = atomicAdd(a.ticket, 1u);  // arrives while the rows are lined up
         }
         // Line-up.  A step's words go to registers, which frees its part of the bitmap: the rows are
         // written there in list order, ready for full-width wavefront stores.  No step needs the
@@ -382,30 +449,33 @@ __global__ __launch_bounds__(DD_THREADS) void dedup_kernel(DedupArgs a) {
         DD_TICK(5)
         uint64_t base = out_base + running;
         bool store = true;
-        if (MODE == DD_FUSED) {
+        if (FUSED) {
             if (wave == 0) {
                 const int qn = min(static_cast<int>(__shfl(ticket_next, 0, 64)), a.n_queries);
                 // spans of the next query (they all sit in this wavefront when T <= 64)
-                if (T <= 64 && qn < a.n_queries && lane < T) sp_next = a.spans[static_cast<size_t>(qn) * T + lane];
-                const unsigned long long excl = look_back(a.state, q, chunk_total, a.spin_limit, a.err);
+                if (last && T <= 64 && qn < a.n_queries && lane < T) sp_next = a.spans[static_cast<size_t>(qn) * T + lane];
+                const unsigned long long excl =
+                    several ? raw_base + running : look_back(a.state, q, chunk_total, a.spin_limit, a.err);
                 if (lane == 0) {
-                    *sh_q = qn;
+                    if (last) *sh_q = qn;
                     unsigned long long b = excl;
                     if (excl + chunk_total > a.capacity) {  // cannot happen with capacity = raw candidates
                         atomicOr(a.err, 2u);
                         b = ~0ull;
                     }
                     *sh_base = b;
-                    a.counts[q] = chunk_total;
-                    a.offsets[q] = excl;
-                    if (q == a.n_queries - 1) a.offsets[a.n_queries] = excl + chunk_total;
+                    if (last) a.counts[q] = running + chunk_total;
+                    if (!several) {
+                        a.offsets[q] = excl;
+                        if (q == a.n_queries - 1) a.offsets[a.n_queries] = excl + chunk_total;
+                    }
                 }
             }
             DD_TICK(6)
             __syncthreads();
             base = *sh_base;
             store = base != ~0ull;
-            q_next = *sh_q;
+            if (last) q_next = *sh_q;
         }
         DD_TICK(2)  // count, line-up (+ look-back)
         if (store) {
@@ -439,7 +509,7 @@ __global__ __launch_bounds__(DD_THREADS) void dedup_kernel(DedupArgs a) {
                 dst += st_total[j];
             }
         }
-        if (MODE == DD_FUSED) {  // leave this wavefront's part of the bitmap clean for the next query
+        if (FUSED) {  // leave this wavefront's part of the bitmap clean for the next query
             uint4* z = reinterpret_cast<uint4*>(wbm);
             for (int i = lane; i < wpw / 4; i += 64) z[i] = make_uint4(0u, 0u, 0u, 0u);
         }
@@ -448,7 +518,7 @@ __global__ __launch_bounds__(DD_THREADS) void dedup_kernel(DedupArgs a) {
         DD_TICK(3)  // ordered store
     }
     if (MODE == DD_COUNT && tid == 0) a.counts[q] = running;
-    if (MODE != DD_FUSED || q_next >= a.n_queries) break;
+    if (!FUSED || q_next >= a.n_queries) break;
     q = q_next;
     if (T <= 64) {
         sp = sp_next;  // zero outside the first T lanes
@@ -482,28 +552,17 @@ int env_int(const char* name, int dflt) {
     return (v && *v) ? std::atoi(v) : dflt;
 }
 
-// The zero-initialised words a query needs, in one block cleared by one memset:
-// [0] raw candidate total, [1] error flags (low half) and ticket counter (high half),
-// [2 .. 2 + n_queries) the published words of the chained scan.
-culsh_status alloc_query_words(culsh_ctx* ctx, int n_queries, unsigned long long** words) {
-    const size_t count = 2 + static_cast<size_t>(n_queries);
-    CULSH_TRY(arena_alloc_t(ctx, count, words));
-    CULSH_HIP(hipMemsetAsync(*words, 0, count * sizeof(unsigned long long), ctx->stream));
-    return CULSH_OK;
-}
+// Geometry of a de-duplication pass: DD_THREADS * wpt bitmap words, wpt a power of two; row ranges
+// beyond one bitmap take n_chunks passes.  Debug knob: CULSH_DEDUP_WPT lowers the cap on wpt (more passes).
+struct DedupGeometry {
+    int wpt = 1, n_chunks = 1;
+    size_t lds_bytes = 0;
+};
 
-// `raw_total` points at the block of alloc_query_words; its first word holds the number of raw
-// candidates = sum of all span lengths.
-culsh_status query_from_spans(culsh_ctx* ctx, const int2* spans, const unsigned long long* raw_total, int n_queries,
-                              const culsh_index* index, culsh_candidates* out) {
+culsh_status dedup_geometry(const culsh_ctx* ctx, const culsh_index* index, DedupGeometry* g) {
     const int T = index->n_hash_tables;
-    // rows addressed by the index: candidates are row ids < n = n_total_candidates / T
-    const int n = index->n_total_candidates / T;
-
-    // Geometry of a pass: DD_THREADS * wpt bitmap words, wpt a power of two.  Debug knobs:
-    // CULSH_DEDUP_WPT lowers the cap on wpt (more passes), CULSH_DEDUP_TWO_PASS=1 forces the
-    // count / scan / emit path, CULSH_DEDUP_TRACE=1 prints phase timers.
-    const size_t fixed = (4 + static_cast<size_t>(3 * T) + 1 + 2 * DD_THREADS + 17 + (NWAVES + 1) + 8) * sizeof(uint32_t);
+    const int n = index->n_total_candidates / T;  // candidates are row ids < n
+    const size_t fixed = (4 + static_cast<size_t>(4 * T) + 1 + 2 * DD_THREADS + 17 + (NWAVES + 1) + 8) * sizeof(uint32_t);
     auto lds_need = [&](int w) { return static_cast<size_t>(DD_THREADS) * w * 4 + fixed; };
     int wpt_max = 1;
     const int wpt_limit = std::max(1, std::min(32, env_int("CULSH_DEDUP_WPT", 32)));
@@ -511,9 +570,32 @@ culsh_status query_from_spans(culsh_ctx* ctx, const int2* spans, const unsigned 
     int wpt = 1;
     while (wpt < wpt_max && static_cast<long long>(DD_THREADS) * wpt * 32 < n) wpt *= 2;
     const long long chunk_rows = static_cast<long long>(DD_THREADS) * wpt * 32;
-    const int n_chunks = static_cast<int>((n + chunk_rows - 1) / chunk_rows);
-    const size_t lds_bytes = lds_need(wpt);
-    CULSH_REQUIRE(lds_bytes <= static_cast<size_t>(ctx->lds_max), CULSH_ERR_INTERNAL, "LDS budget exceeded");
+    g->wpt = wpt;
+    g->n_chunks = static_cast<int>((n + chunk_rows - 1) / chunk_rows);
+    g->lds_bytes = lds_need(wpt);
+    CULSH_REQUIRE(g->lds_bytes <= static_cast<size_t>(ctx->lds_max), CULSH_ERR_INTERNAL, "LDS budget exceeded");
+    return CULSH_OK;
+}
+
+// The zero-initialised words a query needs, in one block cleared by one memset:
+// [0] raw candidate total, [1] error flags (low half) and ticket counter (high half),
+// [2 .. 2 + n_queries) the published words of the chained scan (one pass only).
+culsh_status alloc_query_words(culsh_ctx* ctx, int n_queries, const DedupGeometry& g, unsigned long long** words) {
+    const size_t count = 2 + (g.n_chunks == 1 ? static_cast<size_t>(n_queries) : 0);
+    CULSH_TRY(arena_alloc_t(ctx, count, words));
+    CULSH_HIP(hipMemsetAsync(*words, 0, count * sizeof(unsigned long long), ctx->stream));
+    return CULSH_OK;
+}
+
+// `raw_total` points at the block of alloc_query_words; its first word holds the number of raw
+// candidates = sum of all span lengths.  Debug knobs: CULSH_DEDUP_TWO_PASS=1 forces the
+// count / scan / emit path, CULSH_DEDUP_TRACE=1 prints phase timers.
+culsh_status query_from_spans(culsh_ctx* ctx, const int2* spans, const unsigned long long* raw_total, int n_queries,
+                              const culsh_index* index, const DedupGeometry& g, culsh_candidates* out) {
+    const int T = index->n_hash_tables;
+    const int n = index->n_total_candidates / T;
+    const int wpt = g.wpt, n_chunks = g.n_chunks;
+    const size_t lds_bytes = g.lds_bytes;
     const bool trace = env_int("CULSH_DEDUP_TRACE", 0) != 0;
     unsigned long long* ticks_dev = nullptr;
     if (trace) {
@@ -532,6 +614,7 @@ culsh_status query_from_spans(culsh_ctx* ctx, const int2* spans, const unsigned 
     a.counts = out->query_candidate_counts;
     a.offsets = out->query_candidate_offsets;
     a.state = nullptr;
+    a.raw_offsets = nullptr;
     a.err = nullptr;
     a.ticket = nullptr;
     a.capacity = 0;
@@ -542,7 +625,8 @@ culsh_status query_from_spans(culsh_ctx* ctx, const int2* spans, const unsigned 
     a.spin_limit = env_int("CULSH_DEDUP_SPIN_LIMIT", 1 << 16);  // tests set 0 to reach the give-up path
     a.ticks = ticks_dev;
 
-    bool fused = n_chunks == 1 && env_int("CULSH_DEDUP_TWO_PASS", 0) == 0;
+    bool fused = env_int("CULSH_DEDUP_TWO_PASS", 0) == 0;
+    const bool several = n_chunks > 1;
     uint64_t U = 0;
     if (fused) {
         uint64_t R = 0;
@@ -554,45 +638,72 @@ culsh_status query_from_spans(culsh_ctx* ctx, const int2* spans, const unsigned 
             out->query_candidate_indices = nullptr;
             return CULSH_OK;
         }
-        // a query holds at most n distinct rows, which bounds the output when buckets overlap heavily
-        const uint64_t cap = std::min<uint64_t>(R, static_cast<uint64_t>(n_queries) * static_cast<uint64_t>(n));
+        // One pass: lists are packed by a chained scan over the queries; a query holds at most n
+        // distinct rows, which bounds the output when buckets overlap heavily.  Several passes: list q
+        // starts at the sum of the raw counts of the queries before it, and the gaps are closed below.
+        const uint64_t cap = several ? R : std::min<uint64_t>(R, static_cast<uint64_t>(n_queries) * static_cast<uint64_t>(n));
         unsigned long long* words = const_cast<unsigned long long*>(raw_total);
         unsigned int* err = reinterpret_cast<unsigned int*>(words + 1);  // [0] error flags, [1] ticket counter
         a.state = words + 2;
         a.ticket = err + 1;
-        CULSH_HIP(dev_malloc(&out->query_candidate_indices, cap * sizeof(int32_t)));
-        a.out = out->query_candidate_indices;
+        uint64_t* raw_offsets = nullptr;
+        if (several) {
+            uint64_t* raw_counts = nullptr;
+            CULSH_TRY(arena_alloc_t(ctx, static_cast<size_t>(n_queries), &raw_counts));
+            CULSH_TRY(arena_alloc_t(ctx, static_cast<size_t>(n_queries) + 1, &raw_offsets));
+            CULSH_LAUNCH(ctx, raw_counts_kernel, dim3(div_up(static_cast<size_t>(n_queries), 4)), dim3(256), 0, ctx->stream,
+                         spans, n_queries, T, raw_counts);
+            CULSH_LAUNCH_CHECK();
+            CULSH_TRY(exclusive_scan_u64(ctx, raw_counts, raw_offsets, n_queries));
+            a.raw_offsets = raw_offsets;
+            a.state = nullptr;
+        }
+        int32_t* lists = nullptr;
+        CULSH_HIP(dev_malloc(&lists, cap * sizeof(int32_t)));
+        a.out = lists;
         a.err = err;
         a.capacity = cap;
-        CULSH_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(dedup_kernel<DD_FUSED>),
-                                      hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes)));
+        const void* kernel = several ? reinterpret_cast<const void*>(dedup_kernel<DD_FUSED_PASSES>)
+                                     : reinterpret_cast<const void*>(dedup_kernel<DD_FUSED>);
+        CULSH_HIP(hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes)));
         // as many workgroups as fit on the device at once (LDS and 2048 threads per CU bound it)
         const int per_cu = static_cast<int>(std::max<size_t>(1, std::min<size_t>(2, static_cast<size_t>(ctx->lds_max) / lds_bytes)));
         const int resident = std::max(1, ctx->n_cus * per_cu);
-        CULSH_LAUNCH(ctx, dedup_kernel<DD_FUSED>, dim3(std::min(n_queries, resident)), dim3(DD_THREADS), lds_bytes,
-                     ctx->stream, a);
+        if (several)
+            CULSH_LAUNCH(ctx, dedup_kernel<DD_FUSED_PASSES>, dim3(std::min(n_queries, resident)), dim3(DD_THREADS),
+                         lds_bytes, ctx->stream, a);
+        else
+            CULSH_LAUNCH(ctx, dedup_kernel<DD_FUSED>, dim3(std::min(n_queries, resident)), dim3(DD_THREADS), lds_bytes,
+                         ctx->stream, a);
         CULSH_LAUNCH_CHECK();
+        if (several) CULSH_TRY(exclusive_scan_u64(ctx, out->query_candidate_counts, out->query_candidate_offsets, n_queries));
         CULSH_HIP(hipMemcpyAsync(&ctx->pinned[0], out->query_candidate_offsets + n_queries, sizeof(uint64_t),
                                  hipMemcpyDeviceToHost, ctx->stream));
         CULSH_HIP(hipMemcpyAsync(&ctx->pinned[1], err, sizeof(unsigned int), hipMemcpyDeviceToHost, ctx->stream));
         CULSH_HIP(hipStreamSynchronize(ctx->stream));  // host sync 2 of 2
         U = ctx->pinned[0];
         const unsigned int e = static_cast<unsigned int>(ctx->pinned[1] & 0xffffffffu);
+        out->query_candidate_indices = nullptr;
         if (e != 0) {  // never seen; the two-launch path below needs no cooperation between workgroups
-            dev_free(out->query_candidate_indices);
-            out->query_candidate_indices = nullptr;
+            dev_free(lists);
             fused = false;
         } else if (U == 0) {
-            dev_free(out->query_candidate_indices);
-            out->query_candidate_indices = nullptr;
+            dev_free(lists);
+        } else if (several) {
+            CULSH_HIP(dev_malloc(&out->query_candidate_indices, U * sizeof(int32_t)));
+            CULSH_LAUNCH(ctx, close_gaps_kernel, dim3(n_queries), dim3(256), 0, ctx->stream, lists, raw_offsets,
+                         out->query_candidate_offsets, out->query_candidate_counts, out->query_candidate_indices);
+            CULSH_LAUNCH_CHECK();
+            CULSH_HIP(hipStreamSynchronize(ctx->stream));
+            dev_free(lists);
         } else if (U <= cap / 2 && (cap - U) * sizeof(int32_t) > (size_t(16) << 20)) {
             // heavy overlap between tables: hand out an exact-size array instead of the bound
-            int32_t* exact = nullptr;
-            CULSH_HIP(dev_malloc(&exact, U * sizeof(int32_t)));
-            CULSH_HIP(hipMemcpyAsync(exact, out->query_candidate_indices, U * sizeof(int32_t), hipMemcpyDeviceToDevice, ctx->stream));
+            CULSH_HIP(dev_malloc(&out->query_candidate_indices, U * sizeof(int32_t)));
+            CULSH_HIP(hipMemcpyAsync(out->query_candidate_indices, lists, U * sizeof(int32_t), hipMemcpyDeviceToDevice, ctx->stream));
             CULSH_HIP(hipStreamSynchronize(ctx->stream));
-            dev_free(out->query_candidate_indices);
-            out->query_candidate_indices = exact;
+            dev_free(lists);
+        } else {
+            out->query_candidate_indices = lists;
         }
     }
     if (!fused) {
@@ -646,11 +757,13 @@ culsh_status query_from_matched(culsh_ctx* ctx, const int32_t* matched, int n_qu
     int2* spans = nullptr;
     unsigned long long* raw_total = nullptr;
     CULSH_TRY(arena_alloc_t(ctx, pairs, &spans));
-    CULSH_TRY(alloc_query_words(ctx, n_queries, &raw_total));
+    DedupGeometry g;
+    CULSH_TRY(dedup_geometry(ctx, index, &g));
+    CULSH_TRY(alloc_query_words(ctx, n_queries, g, &raw_total));
     CULSH_LAUNCH(ctx, span_kernel, dim3(div_up(pairs, 256)), dim3(256), 0, ctx->stream, matched,
                  index->bucket_candidate_offsets, pairs, spans, raw_total);
     CULSH_LAUNCH_CHECK();
-    return query_from_spans(ctx, spans, raw_total, n_queries, index, out);
+    return query_from_spans(ctx, spans, raw_total, n_queries, index, g, out);
 }
 
 culsh_status query_from_keys(culsh_ctx* ctx, const uint32_t* q_keys, int n_queries, const culsh_index* index,
@@ -659,9 +772,11 @@ culsh_status query_from_keys(culsh_ctx* ctx, const uint32_t* q_keys, int n_queri
     int2* spans = nullptr;
     unsigned long long* raw_total = nullptr;
     CULSH_TRY(arena_alloc_t(ctx, static_cast<size_t>(n_queries) * index->n_hash_tables, &spans));
-    CULSH_TRY(alloc_query_words(ctx, n_queries, &raw_total));
+    DedupGeometry g;
+    CULSH_TRY(dedup_geometry(ctx, index, &g));
+    CULSH_TRY(alloc_query_words(ctx, n_queries, g, &raw_total));
     CULSH_TRY(launch_find_matching_buckets(ctx, q_keys, n_queries, index, nullptr, spans, raw_total));
-    return query_from_spans(ctx, spans, raw_total, n_queries, index, out);
+    return query_from_spans(ctx, spans, raw_total, n_queries, index, g, out);
 }
 
 }  // namespace culsh_amd

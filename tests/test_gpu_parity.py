@@ -254,6 +254,30 @@ def test_core_query_wide_row_range(ctx, c_oracle, n):
     ctx.free_index(ih)
 
 
+@pytest.mark.parametrize("two_pass", [False, True])
+def test_core_query_many_bitmap_passes(ctx, monkeypatch, two_pass):
+    """A small bitmap (32768 rows per pass) makes a 150k-row index take five passes per query: in the
+    single launch every (query, pass) is a unit of the chained scan and spans shrink from pass to
+    pass; passes without any row and queries without candidates are among them.  Also through the
+    count / scan / emit launches."""
+    _announce("many_bitmap_passes", two_pass)
+    monkeypatch.setenv("CULSH_DEDUP_WPT", "1")
+    if two_pass:
+        monkeypatch.setenv("CULSH_DEDUP_TWO_PASS", "1")
+    rng = np.random.default_rng(77)
+    T, n, nq, H = 7, 150_000, 1500, 2
+    sig = rng.integers(0, 40, size=(T, n, H)).astype(np.uint8)           # ~94 rows per bucket
+    sig[:, 40_000:70_000, 0] = 200                                        # rows of the second pass keep to themselves
+    qsig = rng.integers(0, 40, size=(T, nq, H)).astype(np.uint8)
+    qsig[:, ::9, 0] = 200                                                 # candidates in one pass only
+    qsig[:, ::13, :] = 255                                                # no candidates at all
+    ih, _ = ctx.core_fit_index(sig, H)
+    from abi import assert_candidates_match
+
+    assert_candidates_match(ctx.core_query_index(qsig, ih), o.query_index(qsig, o.fit_index(sig, H)))
+    ctx.free_index(ih)
+
+
 def test_core_query_two_launch_path(ctx, monkeypatch):
     """The count / scan / emit path (taken for row ranges beyond one bitmap pass) on a small case."""
     _announce("two_launch_path")
