@@ -641,6 +641,96 @@ def test_full_size_invariants(ctx):
     ctx.free_index(ih)
 
 
+def test_config5_full_size_invariants(ctx):
+    """BASELINE config 5 at its real shape (4M x 768 rows of a 1000-component Gaussian mixture on the
+    unit sphere, 64 tables x 16 hashes), 20k queries in batches of 10k: the index takes 2^28 items, a
+    query four bitmap passes over the row range, and the batches are merged.  Data are made and the
+    properties checked on the device; a sample of buckets and of queries is compared with brute force."""
+    _announce("config5_full_size")
+    import ctypes as C
+
+    import torch
+    from abi import hp, ptr
+    from culsh_amd import _lib as L
+
+    n, d, nq, T, H, batch = 4_000_000, 768, 20_000, 64, 16, 10_000
+    g = torch.Generator(device="cuda")
+    g.manual_seed(7)
+    centres = torch.randn(1000, d, device="cuda", generator=g)
+
+    def mixture(rows):
+        out = torch.empty(rows, d, device="cuda", dtype=torch.float32)
+        for s0 in range(0, rows, 500_000):
+            m = min(500_000, rows - s0)
+            comp = torch.randint(0, 1000, (m,), device="cuda", generator=g)
+            x = centres[comp] + 0.3 * torch.randn(m, d, device="cuda", generator=g)
+            out[s0:s0 + m] = x / x.norm(dim=1, keepdim=True)
+        return out
+
+    X, Q = mixture(n), mixture(nq)
+    P = torch.randn(T * H, d, device="cuda", generator=g)
+    P_host = np.ascontiguousarray(P.cpu().numpy())
+    torch.cuda.synchronize()
+    ih = C.c_void_p()
+    L.check(ctx.lib.culsh_rplsh_fit_f32(ctx.h, ptr(X), n, d, T, H, 42, hp(P_host), C.byref(ih)))
+    ix = ctx.index_arrays(ih)
+    N = n * T
+    B = int(ix["n_total_buckets"])
+    tbo = torch.from_numpy(ix["table_bucket_offsets"].astype(np.int64)).cuda()
+    bco = torch.from_numpy(ix["bucket_candidate_offsets"].astype(np.int64)).cuda()
+    cand = torch.from_numpy(ix["all_candidate_indices"]).cuda()
+    assert tbo[0] == 0 and tbo[-1] == B and bool((tbo.diff() > 0).all())
+    assert bco[0] == 0 and bco[-1] == N and bool((bco.diff() > 0).all())
+    assert bool((bco[tbo[:-1]] == torch.arange(T, device="cuda") * n).all())   # a table's first bucket starts its segment
+    for t in range(T):                                                          # every table holds every row once
+        assert bool((torch.bincount(cand[t * n:(t + 1) * n], minlength=n) == 1).all()), t
+    descents = torch.nonzero(cand[1:] < cand[:-1]).flatten() + 1                # rows ascend inside a bucket
+    assert bool(torch.isin(descents, bco).all())
+    sig = torch.from_numpy(ix["all_bucket_signatures"].reshape(B, H)).cuda().to(torch.int64)
+    keys = (sig * (1 << torch.arange(H - 1, -1, -1, device="cuda"))).sum(1)     # 16 sign bytes as a number
+    inc = keys.diff() > 0
+    inc[tbo[1:-1] - 1] = True                                                   # table boundaries may descend
+    assert bool(inc.all())
+    # a bucket's signature is the sign pattern of the rows in it (float64 projection, outside the band)
+    pos = torch.arange(0, N, 100_003, device="cuda")
+    b = torch.searchsorted(bco, pos, right=True) - 1
+    rows, tt, k = cand[pos].long(), pos // n, torch.arange(len(pos), device="cuda")
+    proj = (X[rows].double() @ P.double().T).view(-1, T, H)[k, tt]
+    scale = (X[rows].abs().double() @ P.abs().double().T).view(-1, T, H)[k, tt]
+    assert int((((proj >= 0).to(torch.int64) != sig[b]) & (proj.abs() > TOL * scale)).sum()) == 0
+    # queries
+    ch = C.c_void_p()
+    L.check(ctx.lib.culsh_rplsh_query_f32(ctx.h, ptr(Q), nq, ih, batch, C.byref(ch)))
+    got = ctx.candidates_arrays(ch)
+    off = torch.from_numpy(got["offsets"].astype(np.int64)).cuda()
+    idx = torch.from_numpy(got["indices"]).cuda()
+    assert off[0] == 0 and int(off[-1]) == len(idx) and bool((off.diff() >= 0).all())
+    assert np.array_equal(np.diff(got["offsets"].astype(np.int64)), got["counts"].astype(np.int64))
+    inside = torch.ones(len(idx), dtype=torch.bool, device="cuda")
+    starts = off[1:-1]
+    inside[starts[starts < len(idx)]] = False                                   # first element of the next query
+    assert bool(((idx[1:] > idx[:-1]) | ~inside[1:]).all())                     # ascending, duplicate-free per query
+    assert int(idx.min()) >= 0 and int(idx.max()) < n
+    sample = [0, 9_999, 10_000, 14_321, 19_999]                                 # both batches and their edges
+    qsig = ctx.rplsh_hash(Q[sample].cpu().numpy(), P_host, T, H)                # [T][5][H]
+    sig_np = ix["all_bucket_signatures"].reshape(B, H)
+    tbo_np, bco_np, cand_np = ix["table_bucket_offsets"], ix["bucket_candidate_offsets"], ix["all_candidate_indices"]
+    for j, q in enumerate(sample):
+        exp = []
+        for t in range(T):
+            lo, hi = tbo_np[t], tbo_np[t + 1]
+            hit = np.flatnonzero((sig_np[lo:hi] == qsig[t, j]).all(axis=1))
+            if len(hit):
+                bb = lo + hit[0]
+                exp.append(cand_np[bco_np[bb]:bco_np[bb + 1]])
+        exp = np.unique(np.concatenate(exp)) if exp else np.zeros(0, np.int32)
+        np.testing.assert_array_equal(got["indices"][int(got["offsets"][q]):int(got["offsets"][q + 1])], exp)
+    ctx.free_index(ih)
+    del X, Q, cand, sig, idx
+    torch.cuda.empty_cache()
+    ctx.lib.culsh_memory_trim()
+
+
 def test_minhash_rank_keys_edge_cases(ctx):
     """MinHash keys are stored as column ranks when every fitted column id is below n_features.
     Checked against the oracle: query rows whose minimum comes from a column >= n_features (they
