@@ -240,22 +240,37 @@ __global__ __launch_bounds__(SORT_THREADS) void radix_scatter_kernel(
     int32_t rw[STAGED ? SORT_ITEMS : 1];
     uint32_t kw_other[TWO_WORDS ? SORT_ITEMS : 1];  // the word of a two-word key that is not the digit word
     const unsigned long long lt_mask = (1ull << lane) - 1ull;
+    // All loads of the tile are issued before the first is used: indices past the end are clamped
+    // instead of predicated, so nothing stands between the loads (a branch per load would make every
+    // item wait for its own round trip to memory).
+    const int last_idx = n - 1;
+#pragma unroll
+    for (int j = 0; j < SORT_ITEMS; ++j) {
+        const uint32_t idc = static_cast<uint32_t>(min(base_idx + j * 64 + lane, last_idx));
+        if (TWO_WORDS) {
+            const uint2 kv = *reinterpret_cast<const uint2*>(tkeys_in + idc * 2u);
+            kw[j] = word == 0 ? kv.x : kv.y;
+            kw_other[j] = word == 0 ? kv.y : kv.x;
+        } else {
+            kw[j] = KW > 0 ? tkeys_in[idc * static_cast<uint32_t>(KW) + static_cast<uint32_t>(word)]
+                           : tkeys_in[static_cast<size_t>(idc) * W + word];
+        }
+    }
+    if (STAGED) {
+        if (trows_in) {
+#pragma unroll
+            for (int j = 0; j < SORT_ITEMS; ++j)
+                rw[j] = trows_in[static_cast<uint32_t>(min(base_idx + j * 64 + lane, last_idx))];
+        } else {
+#pragma unroll
+            for (int j = 0; j < SORT_ITEMS; ++j) rw[j] = base_idx + j * 64 + lane;
+        }
+    }
 #pragma unroll
     for (int j = 0; j < SORT_ITEMS; ++j) {
         const int idx = base_idx + j * 64 + lane;
         const bool valid = idx < n;
-        uint32_t k = 0u;
-        if (TWO_WORDS) {
-            uint2 kv = make_uint2(0u, 0u);
-            if (valid) kv = *reinterpret_cast<const uint2*>(tkeys_in + static_cast<uint32_t>(idx) * 2u);
-            k = word == 0 ? kv.x : kv.y;
-            kw_other[j] = word == 0 ? kv.y : kv.x;
-        } else if (valid) {
-            k = KW > 0 ? tkeys_in[static_cast<uint32_t>(idx) * static_cast<uint32_t>(KW) + static_cast<uint32_t>(word)]
-                       : tkeys_in[static_cast<size_t>(idx) * W + word];
-        }
-        kw[j] = k;
-        if (STAGED) rw[j] = (valid && trows_in) ? trows_in[static_cast<uint32_t>(idx)] : idx;
+        const uint32_t k = kw[j];
         const uint32_t d = (k >> shift) & 255u;
         // lanes holding the same digit
         const unsigned long long live = __builtin_amdgcn_ballot_w64(valid);
