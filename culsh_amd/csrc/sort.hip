@@ -106,30 +106,36 @@ __global__ __launch_bounds__(SORT_THREADS) void radix_totals_kernel(const uint32
                                                                    PassList pl, int T,
                                                                    uint32_t* __restrict__ dtot /*[pass][T][256]*/) {
     __shared__ uint32_t h[MAX_PASSES_PER_LAUNCH][256];
-    const int tile = blockIdx.x, t = blockIdx.y;
+    const int t = blockIdx.y;
     // few passes leave room for one histogram copy per wavefront (fewer same-address atomics)
     const int copies = pl.count <= MAX_PASSES_PER_LAUNCH / 4 ? 4 : (pl.count <= MAX_PASSES_PER_LAUNCH / 2 ? 2 : 1);
     const int mine = (threadIdx.x >> 6) % copies;
     for (int i = threadIdx.x; i < copies * pl.count * 256; i += SORT_THREADS) (&h[0][0])[i] = 0;
     __syncthreads();
     const uint32_t* tk = keys + static_cast<size_t>(t) * n * W;
-    uint32_t kw[TOT_ITEMS];
-    int last_word = -1;
-    for (int p = 0; p < pl.count; ++p) {  // passes are ordered by word, so a word is fetched once
-        if (pl.word[p] != last_word) {
-            last_word = pl.word[p];
+    const int last_idx = n - 1;
+    // A workgroup takes every gridDim.x-th tile of its table: the atomics on the totals in memory at
+    // the end are what bounds this kernel, so there are few workgroups with many tiles each.
+    const int tiles = (n + TOT_TILE - 1) / TOT_TILE;
+    for (int tile = blockIdx.x; tile < tiles; tile += gridDim.x) {
+        uint32_t kw[TOT_ITEMS];
+        int last_word = -1;
+        for (int p = 0; p < pl.count; ++p) {  // passes are ordered by word, so a word is fetched once
+            if (pl.word[p] != last_word) {
+                last_word = pl.word[p];
+#pragma unroll
+                for (int j = 0; j < TOT_ITEMS; ++j) {  // clamped, not predicated: nothing stands between the loads
+                    const int idx = min(tile * TOT_TILE + j * SORT_THREADS + static_cast<int>(threadIdx.x), last_idx);
+                    kw[j] = tk[static_cast<size_t>(idx) * W + last_word];
+                }
+            }
+            uint32_t* hp = h[mine * pl.count + p];
+            const int shift = pl.shift[p];
 #pragma unroll
             for (int j = 0; j < TOT_ITEMS; ++j) {
                 const int idx = tile * TOT_TILE + j * SORT_THREADS + threadIdx.x;
-                kw[j] = (idx < n) ? tk[static_cast<size_t>(idx) * W + last_word] : 0u;
+                if (idx < n) atomicAdd(&hp[(kw[j] >> shift) & 255u], 1u);
             }
-        }
-        uint32_t* hp = h[mine * pl.count + p];
-        const int shift = pl.shift[p];
-#pragma unroll
-        for (int j = 0; j < TOT_ITEMS; ++j) {
-            const int idx = tile * TOT_TILE + j * SORT_THREADS + threadIdx.x;
-            if (idx < n) atomicAdd(&hp[(kw[j] >> shift) & 255u], 1u);
         }
     }
     __syncthreads();
@@ -483,7 +489,9 @@ culsh_status sort_tables(culsh_ctx* ctx, uint32_t* keys_in, uint32_t* keys_tmp, 
                 pl.word[i] = i < pl.count ? passes[p0 + i].word : 0;
                 pl.shift[i] = i < pl.count ? passes[p0 + i].shift : 0;
             }
-            CULSH_LAUNCH(ctx, radix_totals_kernel, dim3((n + TOT_TILE - 1) / TOT_TILE, T), dim3(SORT_THREADS), 0, ctx->stream, keys_in, n, W, pl,
+            // about four workgroups per CU over all tables
+            const int per_table = std::max(1, std::min((n + TOT_TILE - 1) / TOT_TILE, (4 * ctx->n_cus + T - 1) / T));
+            CULSH_LAUNCH(ctx, radix_totals_kernel, dim3(per_table, T), dim3(SORT_THREADS), 0, ctx->stream, keys_in, n, W, pl,
                          T, dtot + static_cast<size_t>(p0) * T * 256);
             CULSH_LAUNCH_CHECK();
         }
