@@ -25,9 +25,17 @@
 namespace culsh_amd {
 namespace {
 
-constexpr int SORT_THREADS = 256;
-constexpr int SORT_ITEMS = 8;
-constexpr int SORT_TILE = SORT_THREADS * SORT_ITEMS;  // 2048 items per workgroup (7-8 workgroups per CU; 16 items: 4)
+constexpr int SORT_THREADS = 256;  // histogram kernels; also the number of digits
+
+// Tile of a scatter pass: THREADS * ITEMS items per workgroup.  A tile leaves in 256 digit runs, so
+// bigger tiles mean longer runs of consecutive addresses per store (what the pass is bound by) and
+// fewer, larger workgroups per CU (LDS holds the whole tile).
+struct TileShape {
+    int threads, items;
+    constexpr int tile() const { return threads * items; }
+};
+constexpr TileShape SHAPE_W1{512, 16}, SHAPE_W2{512, 8}, SHAPE_ANY{256, 16};
+inline TileShape tile_shape(int W) { return W == 1 ? SHAPE_W1 : (W == 2 ? SHAPE_W2 : SHAPE_ANY); }
 
 // vary[w] |= key[t][i][w] ^ key[t][0][w]
 __device__ __forceinline__ void publish_vary(uint32_t acc, uint32_t* __restrict__ slot) {
@@ -151,24 +159,17 @@ constexpr uint32_t ST_COUNT = 1u << 30, ST_SUM = 2u << 30, ST_VALUE = ST_COUNT -
 
 __global__ __launch_bounds__(SORT_THREADS) void radix_hist_kernel(const uint32_t* __restrict__ keys, int n,
                                                                  int W, int word, int shift, int tiles,
-                                                                 uint32_t* __restrict__ hist,
+                                                                 int tile_items, uint32_t* __restrict__ hist,
                                                                  uint32_t* __restrict__ dtot) {
     __shared__ uint32_t h[SORT_THREADS / 64][256];  // one copy per wavefront: fewer same-bank atomics
     const int tile = blockIdx.x, t = blockIdx.y, wave = threadIdx.x >> 6;
     for (int i = threadIdx.x; i < (SORT_THREADS / 64) * 256; i += SORT_THREADS) (&h[0][0])[i] = 0;
     __syncthreads();
     const uint32_t* tk = keys + static_cast<size_t>(t) * n * W;
-    uint32_t k[SORT_ITEMS];
-#pragma unroll
-    for (int j = 0; j < SORT_ITEMS; ++j) {
-        const int idx = tile * SORT_TILE + j * SORT_THREADS + threadIdx.x;
-        k[j] = (idx < n) ? tk[static_cast<size_t>(idx) * W + word] : 0u;
-    }
-#pragma unroll
-    for (int j = 0; j < SORT_ITEMS; ++j) {
-        const int idx = tile * SORT_TILE + j * SORT_THREADS + threadIdx.x;
-        if (idx < n) atomicAdd(&h[wave][(k[j] >> shift) & 255u], 1u);
-    }
+    const int end = static_cast<int>(min(static_cast<long long>(n), static_cast<long long>(tile + 1) * tile_items));
+#pragma unroll 4
+    for (int idx = tile * tile_items + threadIdx.x; idx < end; idx += SORT_THREADS)
+        atomicAdd(&h[wave][(tk[static_cast<size_t>(idx) * W + word] >> shift) & 255u], 1u);
     __syncthreads();
     uint32_t c = 0;
 #pragma unroll
@@ -209,27 +210,36 @@ __global__ __launch_bounds__(256) void radix_scan_kernel(uint32_t* __restrict__ 
 // CHAINED: `hist_scanned` is null; `dtot` holds this pass's digit totals [T][256], `state`
 // the published words [T][tiles][256] (zero at launch), `err` the give-up flag; the grid is
 // one-dimensional and tile-major.
-template <int KW, bool CHAINED>
-__global__ __launch_bounds__(SORT_THREADS) void radix_scatter_kernel(
+// LDS bytes of a scatter workgroup (the kernel carves the same layout).
+constexpr size_t scatter_lds_bytes(int KW, TileShape sh) {
+    const size_t tile = static_cast<size_t>(sh.tile());
+    const size_t staged = (KW == 1 || KW == 2) ? tile * KW + tile : tile;  // keys + rows, else source slots
+    return ((sh.threads / 64) * 256 + 256 + 256 + 32 + staged) * sizeof(uint32_t);
+}
+
+template <int KW, bool CHAINED, int THREADS, int ITEMS>
+__global__ __launch_bounds__(THREADS) void radix_scatter_kernel(
     const uint32_t* __restrict__ keys_in, const int32_t* __restrict__ rows_in,
     uint32_t* __restrict__ keys_out, int32_t* __restrict__ rows_out,
     const uint32_t* __restrict__ hist_scanned, int n, int W, int word, int shift, int tiles, int T,
     const uint32_t* __restrict__ dtot, uint32_t* __restrict__ state, uint32_t* __restrict__ err,
     int spin_limit) {
     constexpr bool ONE_WORD = (KW == 1);
-    constexpr int NW = SORT_THREADS / 64;
-    __shared__ uint32_t whist[NW][256];   // per-wave digit counts, then per-wave offsets inside a digit run
-    __shared__ uint32_t dstart[256];      // start of each digit's run inside the sorted tile
-    __shared__ uint32_t gbase[256];       // global position of the run minus dstart (wraps, used additively)
-    __shared__ uint32_t scratch[17];
+    constexpr int NW = THREADS / 64;
+    constexpr int TILE = THREADS * ITEMS;
     constexpr bool TWO_WORDS = (KW == 2);                  // staged in full as well (8-byte keys)
     constexpr bool STAGED = ONE_WORD || TWO_WORDS;
-    __shared__ __attribute__((aligned(8))) uint32_t st_key[SORT_TILE * (TWO_WORDS ? 2 : 1)];  // staged keys, else source slots
-    __shared__ int32_t st_row[STAGED ? SORT_TILE : 1];
+    extern __shared__ __attribute__((aligned(16))) uint32_t scatter_lds[];
+    uint32_t (*whist)[256] = reinterpret_cast<uint32_t (*)[256]>(scatter_lds);  // [NW] per-wave digit counts, then per-wave offsets inside a digit run
+    uint32_t* dstart = scatter_lds + NW * 256;   // [256] start of each digit's run inside the sorted tile
+    uint32_t* gbase = dstart + 256;              // [256] global position of the run minus dstart (wraps, used additively)
+    uint32_t* scratch = gbase + 256;             // [32]
+    uint32_t* st_key = scratch + 32;             // [TILE * (1 or 2)] staged keys (8-byte aligned), else [TILE] source slots
+    int32_t* st_row = reinterpret_cast<int32_t*>(st_key + TILE * (TWO_WORDS ? 2 : 1));  // [TILE] when staged
     const int tile = CHAINED ? static_cast<int>(blockIdx.x / T) : static_cast<int>(blockIdx.x);
     const int t = CHAINED ? static_cast<int>(blockIdx.x - static_cast<unsigned>(tile) * T) : static_cast<int>(blockIdx.y);
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    for (int i = tid; i < NW * 256; i += SORT_THREADS) (&whist[0][0])[i] = 0;
+    for (int i = tid; i < NW * 256; i += THREADS) (&whist[0][0])[i] = 0;
     __syncthreads();
 
     // table bases are wavefront-uniform; inside a table 32-bit element offsets suffice for the
@@ -240,18 +250,17 @@ __global__ __launch_bounds__(SORT_THREADS) void radix_scatter_kernel(
     const int32_t* trows_in = rows_in ? rows_in + tbase : nullptr;
     uint32_t* tkeys_out = keys_out + tbase * Wc;
     int32_t* trows_out = rows_out + tbase;
-    const int tile0 = tile * SORT_TILE;
-    const int base_idx = tile0 + wave * (SORT_ITEMS * 64);
-    uint32_t kw[SORT_ITEMS], rank[SORT_ITEMS];
-    int32_t rw[STAGED ? SORT_ITEMS : 1];
-    uint32_t kw_other[TWO_WORDS ? SORT_ITEMS : 1];  // the word of a two-word key that is not the digit word
-    const unsigned long long lt_mask = (1ull << lane) - 1ull;
+    const int tile0 = tile * TILE;
+    const int base_idx = tile0 + wave * (ITEMS * 64);
+    uint32_t kw[ITEMS], rank[ITEMS];
+    int32_t rw[STAGED ? ITEMS : 1];
+    uint32_t kw_other[TWO_WORDS ? ITEMS : 1];  // the word of a two-word key that is not the digit word
     // All loads of the tile are issued before the first is used: indices past the end are clamped
     // instead of predicated, so nothing stands between the loads (a branch per load would make every
     // item wait for its own round trip to memory).
     const int last_idx = n - 1;
 #pragma unroll
-    for (int j = 0; j < SORT_ITEMS; ++j) {
+    for (int j = 0; j < ITEMS; ++j) {
         const uint32_t idc = static_cast<uint32_t>(min(base_idx + j * 64 + lane, last_idx));
         if (TWO_WORDS) {
             const uint2 kv = *reinterpret_cast<const uint2*>(tkeys_in + idc * 2u);
@@ -265,15 +274,15 @@ __global__ __launch_bounds__(SORT_THREADS) void radix_scatter_kernel(
     if (STAGED) {
         if (trows_in) {
 #pragma unroll
-            for (int j = 0; j < SORT_ITEMS; ++j)
+            for (int j = 0; j < ITEMS; ++j)
                 rw[j] = trows_in[static_cast<uint32_t>(min(base_idx + j * 64 + lane, last_idx))];
         } else {
 #pragma unroll
-            for (int j = 0; j < SORT_ITEMS; ++j) rw[j] = base_idx + j * 64 + lane;
+            for (int j = 0; j < ITEMS; ++j) rw[j] = base_idx + j * 64 + lane;
         }
     }
 #pragma unroll
-    for (int j = 0; j < SORT_ITEMS; ++j) {
+    for (int j = 0; j < ITEMS; ++j) {
         const int idx = base_idx + j * 64 + lane;
         const bool valid = idx < n;
         const uint32_t k = kw[j];
@@ -291,62 +300,63 @@ __global__ __launch_bounds__(SORT_THREADS) void radix_scatter_kernel(
             peers_lo &= ~(static_cast<uint32_t>(m) ^ x);
             peers_hi &= ~(static_cast<uint32_t>(m >> 32) ^ x);
         }
-        const unsigned long long peers = (static_cast<unsigned long long>(peers_hi) << 32) | peers_lo;
-        uint32_t old = 0;
-        int leader = lane;
-        if (valid) {
-            leader = __ffsll(static_cast<long long>(peers)) - 1;
-            if (lane == leader) {
-                old = whist[wave][d];
-                whist[wave][d] = old + static_cast<uint32_t>(__popcll(peers));
-            }
-        }
-        old = __shfl(old, leader, 64);
-        rank[j] = old + static_cast<uint32_t>(__popcll(peers & lt_mask));
+        // Every lane reads its digit's counter; then the lowest lane of each group of peers adds the
+        // group's size.  LDS accesses of one wavefront complete in order and the counters belong to
+        // this wavefront alone, so the reads see the value from before this step.
+        const uint32_t below = __builtin_amdgcn_mbcnt_hi(peers_hi, __builtin_amdgcn_mbcnt_lo(peers_lo, 0u));
+        const uint32_t old = whist[wave][d];
+        if (valid && below == 0u) whist[wave][d] = old + static_cast<uint32_t>(__popc(peers_lo) + __popc(peers_hi));
+        rank[j] = old + below;
     }
     __syncthreads();
-    {   // digit `tid`: exclusive over the waves, then over the digits of the tile
+    {   // digit `tid` (the first 256 threads have one): exclusive over the waves, then over the digits of the tile
+        const bool has_digit = THREADS == 256 || tid < 256;
         uint32_t tot = 0;
+        if (has_digit) {
 #pragma unroll
-        for (int w = 0; w < NW; ++w) {
-            const uint32_t c = whist[w][tid];
-            whist[w][tid] = tot;
-            tot += c;
+            for (int w = 0; w < NW; ++w) {
+                const uint32_t c = whist[w][tid];
+                whist[w][tid] = tot;
+                tot += c;
+            }
         }
         uint32_t tile_total;
         const uint32_t ds = block_exclusive_sum(tot, scratch, &tile_total);
-        dstart[tid] = ds;
+        if (has_digit) dstart[tid] = ds;
         if (CHAINED) {
             // publish this tile's count of digit `tid`, then add up the tiles before it
             uint32_t* st = state + static_cast<size_t>(t) * tiles * 256 + tid;  // entry of tile k: st[k * 256]
-            __hip_atomic_store(st + static_cast<size_t>(tile) * 256, (tile == 0 ? ST_SUM : ST_COUNT) | tot,
-                               __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (has_digit)
+                __hip_atomic_store(st + static_cast<size_t>(tile) * 256, (tile == 0 ? ST_SUM : ST_COUNT) | tot,
+                                   __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             // start of the digit's range in the table: exclusive scan of the digit totals
             uint32_t all;
-            const uint32_t dbase = block_exclusive_sum(dtot[t * 256 + tid], scratch, &all);
-            uint32_t before = 0;
-            int polls = 0;
-            for (int k = tile - 1; k >= 0;) {
-                const uint32_t v = __hip_atomic_load(st + static_cast<size_t>(k) * 256, __ATOMIC_RELAXED,
-                                                     __HIP_MEMORY_SCOPE_AGENT);
-                const uint32_t tag = v >> 30;
-                if (tag == 0u) {
-                    if (++polls > spin_limit) {  // give up: positions stay inside the digit's range
-                        atomicOr(err, 1u);
-                        break;
+            const uint32_t dbase = block_exclusive_sum(has_digit ? dtot[t * 256 + tid] : 0u, scratch, &all);
+            if (has_digit) {
+                uint32_t before = 0;
+                int polls = 0;
+                for (int k = tile - 1; k >= 0;) {
+                    const uint32_t v = __hip_atomic_load(st + static_cast<size_t>(k) * 256, __ATOMIC_RELAXED,
+                                                         __HIP_MEMORY_SCOPE_AGENT);
+                    const uint32_t tag = v >> 30;
+                    if (tag == 0u) {
+                        if (++polls > spin_limit) {  // give up: positions stay inside the digit's range
+                            atomicOr(err, 1u);
+                            break;
+                        }
+                        __builtin_amdgcn_s_sleep(1);
+                        continue;
                     }
-                    __builtin_amdgcn_s_sleep(1);
-                    continue;
+                    before += v & ST_VALUE;
+                    if (tag == 2u) break;
+                    --k;
                 }
-                before += v & ST_VALUE;
-                if (tag == 2u) break;
-                --k;
+                if (tile > 0)
+                    __hip_atomic_store(st + static_cast<size_t>(tile) * 256, ST_SUM | (before + tot), __ATOMIC_RELAXED,
+                                       __HIP_MEMORY_SCOPE_AGENT);
+                gbase[tid] = dbase + before - ds;
             }
-            if (tile > 0)
-                __hip_atomic_store(st + static_cast<size_t>(tile) * 256, ST_SUM | (before + tot), __ATOMIC_RELAXED,
-                                   __HIP_MEMORY_SCOPE_AGENT);
-            gbase[tid] = dbase + before - ds;
-        } else {
+        } else if (has_digit) {
             gbase[tid] = hist_scanned[(static_cast<size_t>(t) * 256 + tid) * tiles + tile] - ds;
         }
     }
@@ -354,7 +364,7 @@ __global__ __launch_bounds__(SORT_THREADS) void radix_scatter_kernel(
     // Stage the tile in digit order in LDS so that the global stores below walk
     // consecutive addresses inside every digit run (full-line writes instead of 4-byte ones).
 #pragma unroll
-    for (int j = 0; j < SORT_ITEMS; ++j) {
+    for (int j = 0; j < ITEMS; ++j) {
         const int idx = base_idx + j * 64 + lane;
         if (idx < n) {
             const uint32_t d = (kw[j] >> shift) & 255u;
@@ -372,8 +382,8 @@ __global__ __launch_bounds__(SORT_THREADS) void radix_scatter_kernel(
         }
     }
     __syncthreads();
-    const int cnt = min(SORT_TILE, n - tile0);
-    for (int slot = tid; slot < cnt; slot += SORT_THREADS) {
+    const int cnt = min(TILE, n - tile0);
+    for (int slot = tid; slot < cnt; slot += THREADS) {
         if (ONE_WORD) {
             const uint32_t k = st_key[slot];
             const uint32_t dst = gbase[(k >> shift) & 255u] + static_cast<uint32_t>(slot);
@@ -411,8 +421,47 @@ __global__ __launch_bounds__(SORT_THREADS) void radix_scatter_kernel(
 
 }  // namespace
 
+namespace {
+
+// One scatter pass with the tile shape of its key width.
+template <int KW, bool CHAINED, int THREADS, int ITEMS, typename... Args>
+culsh_status launch_scatter(culsh_ctx* ctx, dim3 grid, Args... args) {
+    constexpr size_t lds = scatter_lds_bytes(KW, TileShape{THREADS, ITEMS});
+    static bool configured[64] = {};  // per device: more LDS than a launch may ask for by default
+    if (lds > 48 * 1024 && !configured[ctx->device & 63]) {
+        CULSH_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(radix_scatter_kernel<KW, CHAINED, THREADS, ITEMS>),
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)));
+        configured[ctx->device & 63] = true;
+    }
+    {
+        static const char* const names[2][5] = {
+            {"radix_scatter_kernel<0, false>", "radix_scatter_kernel<1, false>", "radix_scatter_kernel<2, false>", "",
+             "radix_scatter_kernel<4, false>"},
+            {"radix_scatter_kernel<0, true>", "radix_scatter_kernel<1, true>", "radix_scatter_kernel<2, true>", "",
+             "radix_scatter_kernel<4, true>"}};
+        StageTimer st(ctx, names[CHAINED ? 1 : 0][KW]);
+        hipLaunchKernelGGL((radix_scatter_kernel<KW, CHAINED, THREADS, ITEMS>), grid, dim3(THREADS), lds, ctx->stream, args...);
+    }
+    CULSH_LAUNCH_CHECK();
+    return CULSH_OK;
+}
+
+template <bool CHAINED, typename... Args>
+culsh_status scatter_pass(culsh_ctx* ctx, dim3 grid, int W, bool fixed_width, Args... args) {
+    if (W == 1)
+        return fixed_width ? launch_scatter<1, CHAINED, SHAPE_W1.threads, SHAPE_W1.items>(ctx, grid, args...)
+                           : launch_scatter<0, CHAINED, SHAPE_W1.threads, SHAPE_W1.items>(ctx, grid, args...);
+    if (W == 2)
+        return fixed_width ? launch_scatter<2, CHAINED, SHAPE_W2.threads, SHAPE_W2.items>(ctx, grid, args...)
+                           : launch_scatter<0, CHAINED, SHAPE_W2.threads, SHAPE_W2.items>(ctx, grid, args...);
+    return (W == 4 && fixed_width) ? launch_scatter<4, CHAINED, SHAPE_ANY.threads, SHAPE_ANY.items>(ctx, grid, args...)
+                                   : launch_scatter<0, CHAINED, SHAPE_ANY.threads, SHAPE_ANY.items>(ctx, grid, args...);
+}
+
+}  // namespace
+
 size_t sort_scratch_bytes(int n, int T, int W) {
-    const size_t tiles = (static_cast<size_t>(n) + SORT_TILE - 1) / SORT_TILE;
+    const size_t tiles = (static_cast<size_t>(n) + tile_shape(W).tile() - 1) / tile_shape(W).tile();
     return align_up(static_cast<size_t>(T) * 256 * tiles * sizeof(uint32_t), 256) +
            align_up(static_cast<size_t>(W) * sizeof(uint32_t), 256) + 512;
 }
@@ -422,7 +471,8 @@ culsh_status sort_tables(culsh_ctx* ctx, uint32_t* keys_in, uint32_t* keys_tmp, 
                          uint32_t** sorted_keys) {
     CULSH_REQUIRE(n > 0 && T > 0 && W > 0 && W <= 64, CULSH_ERR_INVALID, "sort: bad sizes (W must be <= 64 words)");
     CULSH_REQUIRE(T <= 65535, CULSH_ERR_LIMIT, "n_hash_tables > 65535 is not supported");
-    const int tiles = (n + SORT_TILE - 1) / SORT_TILE;
+    const int tile_items = tile_shape(W).tile();
+    const int tiles = (n + tile_items - 1) / tile_items;
     const size_t N = static_cast<size_t>(n) * T;
 
     // which byte positions differ anywhere (given by the caller, or measured on the keys)
@@ -507,39 +557,27 @@ culsh_status sort_tables(culsh_ctx* ctx, uint32_t* keys_in, uint32_t* keys_tmp, 
         // the last pass must land in rows_out
         int32_t* rout = ((np - 1 - p) % 2 == 0) ? rows_out : rows_tmp;
         uint32_t* pass_dtot = dtot + static_cast<size_t>(p) * T * 256;
-        // fixed-width variants use 32-bit element offsets inside a table
-        const bool aligned = reinterpret_cast<uintptr_t>(kin) % 16 == 0 && reinterpret_cast<uintptr_t>(kout) % 16 == 0 && n < (1 << 30);
+        // fixed-width variants use 32-bit element offsets inside a table and vector accesses
+        const bool fixed_width = n < (1 << 30) && (W == 1 || (reinterpret_cast<uintptr_t>(kin) % 16 == 0 &&
+                                                               reinterpret_cast<uintptr_t>(kout) % 16 == 0));
         if (chained) {
             const dim3 grid(static_cast<unsigned>(tiles) * T);
             uint32_t* pass_state = state + static_cast<size_t>(p) * state_words;
-#define SCATTER(KW)                                                                                                  \
-    CULSH_LAUNCH(ctx, (radix_scatter_kernel<KW, true>), grid, dim3(SORT_THREADS), 0, ctx->stream, kin, rin, kout, rout, \
-                 static_cast<const uint32_t*>(nullptr), n, W, passes[p].word, passes[p].shift, tiles, T,              \
-                 static_cast<const uint32_t*>(pass_dtot), pass_state, err, spin_limit)
-            if (W == 1 && n < (1 << 30)) SCATTER(1);
-            else if (W == 2 && aligned) SCATTER(2);
-            else if (W == 4 && aligned) SCATTER(4);
-            else SCATTER(0);
-#undef SCATTER
+            CULSH_TRY(scatter_pass<true>(ctx, grid, W, fixed_width, static_cast<const uint32_t*>(kin), rin, kout, rout,
+                                         static_cast<const uint32_t*>(nullptr), n, W, passes[p].word, passes[p].shift,
+                                         tiles, T, static_cast<const uint32_t*>(pass_dtot), pass_state, err, spin_limit));
         } else {
             const dim3 grid(tiles, T);
             CULSH_LAUNCH(ctx, radix_hist_kernel, grid, dim3(SORT_THREADS), 0, ctx->stream, kin, n, W,
-                         passes[p].word, passes[p].shift, tiles, hist, pass_dtot);
+                         passes[p].word, passes[p].shift, tiles, tile_items, hist, pass_dtot);
             CULSH_LAUNCH_CHECK();
             CULSH_LAUNCH(ctx, radix_scan_kernel, dim3(T, SCAN_PARTS), dim3(256), 0, ctx->stream, hist, pass_dtot, tiles);
             CULSH_LAUNCH_CHECK();
-#define SCATTER(KW)                                                                                                   \
-    CULSH_LAUNCH(ctx, (radix_scatter_kernel<KW, false>), grid, dim3(SORT_THREADS), 0, ctx->stream, kin, rin, kout, rout, \
-                 static_cast<const uint32_t*>(hist), n, W, passes[p].word, passes[p].shift, tiles, T,                  \
-                 static_cast<const uint32_t*>(nullptr), static_cast<uint32_t*>(nullptr),                               \
-                 static_cast<uint32_t*>(nullptr), 0)
-            if (W == 1 && n < (1 << 30)) SCATTER(1);
-            else if (W == 2 && aligned) SCATTER(2);
-            else if (W == 4 && aligned) SCATTER(4);
-            else SCATTER(0);
-#undef SCATTER
+            CULSH_TRY(scatter_pass<false>(ctx, grid, W, fixed_width, static_cast<const uint32_t*>(kin), rin, kout, rout,
+                                          static_cast<const uint32_t*>(hist), n, W, passes[p].word, passes[p].shift,
+                                          tiles, T, static_cast<const uint32_t*>(nullptr),
+                                          static_cast<uint32_t*>(nullptr), static_cast<uint32_t*>(nullptr), 0));
         }
-        CULSH_LAUNCH_CHECK();
         std::swap(kin, kout);
         rin = rout;
     }
