@@ -290,15 +290,24 @@ __global__ __launch_bounds__(THREADS) void radix_scatter_kernel(
         // lanes holding the same digit
         const unsigned long long live = __builtin_amdgcn_ballot_w64(valid);
         uint32_t peers_lo = static_cast<uint32_t>(live), peers_hi = static_cast<uint32_t>(live >> 32);
+        // Per digit bit b: x = all ones if the bit is set in this lane, else zero, and m = the lanes where
+        // it is set.  Lanes agreeing with this one on the bit are m where x is ones and ~m where x is
+        // zero, i.e. ~(m ^ x); peers &= ~(m ^ x) is one three-input bit operation per half.  Written out
+        // by hand: eight compares first, then the sixteen bit operations, which keeps every vector read
+        // of a compare's scalar result at least two instructions behind the compare (gfx950 needs that
+        // distance and nothing pads inline assembly).
+        uint32_t x[8];
+        unsigned long long m[8];
+#pragma unroll
+        for (int b = 0; b < 8; ++b) x[b] = static_cast<uint32_t>(__builtin_amdgcn_sbfe(static_cast<int>(d), b, 1));
+#pragma unroll
+        for (int b = 0; b < 8; ++b) asm volatile("v_cmp_ne_u32_e64 %0, 0, %1" : "=s"(m[b]) : "v"(x[b]));
 #pragma unroll
         for (int b = 0; b < 8; ++b) {
-            // x = all ones if bit b of the digit is set, else zero; lanes agreeing with this one
-            // on that bit are m where x is ones and ~m where x is zero, i.e. ~(m ^ x)
-            const int xs = __builtin_amdgcn_sbfe(static_cast<int>(d), b, 1);  // sign-extended bit b
-            const uint32_t x = static_cast<uint32_t>(xs);
-            const unsigned long long m = __builtin_amdgcn_ballot_w64(xs != 0);
-            peers_lo &= ~(static_cast<uint32_t>(m) ^ x);
-            peers_hi &= ~(static_cast<uint32_t>(m >> 32) ^ x);
+            asm volatile("v_bitop3_b32 %0, %0, %1, %2 bitop3:0x90"
+                         : "+v"(peers_lo) : "s"(static_cast<uint32_t>(m[b])), "v"(x[b]));
+            asm volatile("v_bitop3_b32 %0, %0, %1, %2 bitop3:0x90"
+                         : "+v"(peers_hi) : "s"(static_cast<uint32_t>(m[b] >> 32)), "v"(x[b]));
         }
         // Every lane reads its digit's counter; then the lowest lane of each group of peers adds the
         // group's size.  LDS accesses of one wavefront complete in order and the counters belong to
