@@ -660,6 +660,7 @@ culsh_status query_from_spans(culsh_ctx* ctx, const int2* spans, const unsigned 
         }
         int32_t* lists = nullptr;
         CULSH_HIP(dev_malloc(&lists, cap * sizeof(int32_t)));
+        out->query_candidate_indices = lists;  // owned by `out` from here on, also if a later step fails
         a.out = lists;
         a.err = err;
         a.capacity = cap;
@@ -683,27 +684,36 @@ culsh_status query_from_spans(culsh_ctx* ctx, const int2* spans, const unsigned 
         CULSH_HIP(hipStreamSynchronize(ctx->stream));  // host sync 2 of 2
         U = ctx->pinned[0];
         const unsigned int e = static_cast<unsigned int>(ctx->pinned[1] & 0xffffffffu);
-        out->query_candidate_indices = nullptr;
         if (e != 0) {  // never seen; the two-launch path below needs no cooperation between workgroups
             dev_free(lists);
+            out->query_candidate_indices = nullptr;
             fused = false;
         } else if (U == 0) {
             dev_free(lists);
+            out->query_candidate_indices = nullptr;
         } else if (several) {
-            CULSH_HIP(dev_malloc(&out->query_candidate_indices, U * sizeof(int32_t)));
-            CULSH_LAUNCH(ctx, close_gaps_kernel, dim3(n_queries), dim3(256), 0, ctx->stream, lists, raw_offsets,
-                         out->query_candidate_offsets, out->query_candidate_counts, out->query_candidate_indices);
-            CULSH_LAUNCH_CHECK();
-            CULSH_HIP(hipStreamSynchronize(ctx->stream));
+            int32_t* packed = nullptr;
+            CULSH_HIP(dev_malloc(&packed, U * sizeof(int32_t)));
+            out->query_candidate_indices = packed;
+            hipError_t err_copy = hipSuccess;
+            {
+                StageTimer st(ctx, "close_gaps_kernel");
+                hipLaunchKernelGGL(close_gaps_kernel, dim3(n_queries), dim3(256), 0, ctx->stream, lists, raw_offsets,
+                                   out->query_candidate_offsets, out->query_candidate_counts, packed);
+                err_copy = hipGetLastError();
+            }
+            if (err_copy == hipSuccess) err_copy = hipStreamSynchronize(ctx->stream);
             dev_free(lists);
+            CULSH_HIP(err_copy);
         } else if (U <= cap / 2 && (cap - U) * sizeof(int32_t) > (size_t(16) << 20)) {
             // heavy overlap between tables: hand out an exact-size array instead of the bound
-            CULSH_HIP(dev_malloc(&out->query_candidate_indices, U * sizeof(int32_t)));
-            CULSH_HIP(hipMemcpyAsync(out->query_candidate_indices, lists, U * sizeof(int32_t), hipMemcpyDeviceToDevice, ctx->stream));
-            CULSH_HIP(hipStreamSynchronize(ctx->stream));
+            int32_t* exact = nullptr;
+            CULSH_HIP(dev_malloc(&exact, U * sizeof(int32_t)));
+            out->query_candidate_indices = exact;
+            hipError_t err_copy = hipMemcpyAsync(exact, lists, U * sizeof(int32_t), hipMemcpyDeviceToDevice, ctx->stream);
+            if (err_copy == hipSuccess) err_copy = hipStreamSynchronize(ctx->stream);
             dev_free(lists);
-        } else {
-            out->query_candidate_indices = lists;
+            CULSH_HIP(err_copy);
         }
     }
     if (!fused) {
