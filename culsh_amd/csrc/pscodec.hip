@@ -18,6 +18,9 @@
 namespace culsh_amd {
 namespace {
 
+// VEC4: H divides 1024 and is a multiple of 4, sig is 16-byte aligned: a thread reads 16 bytes at a time and
+// always meets the same four hash positions.
+template <bool VEC4>
 __global__ __launch_bounds__(256) void ps_minmax_kernel(const int32_t* __restrict__ sig, int n, int H,
                                                        int32_t* __restrict__ mm /*[T*H][2]*/) {
     __shared__ int32_t smin[1024], smax[1024];
@@ -28,7 +31,24 @@ __global__ __launch_bounds__(256) void ps_minmax_kernel(const int32_t* __restric
     const size_t total = static_cast<size_t>(n) * H;
     const size_t stride = static_cast<size_t>(gridDim.x) * 256;
     size_t e = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
-    if (256 % H == 0) {  // the thread always meets the same hash position
+    if (VEC4) {
+        const int4* t4 = reinterpret_cast<const int4*>(ts);  // table bases stay 16-byte aligned: n * H * 4 bytes each
+        const size_t quads = total / 4;
+        int4 lo = make_int4(INT_MAX, INT_MAX, INT_MAX, INT_MAX), hi = make_int4(INT_MIN, INT_MIN, INT_MIN, INT_MIN);
+#pragma unroll 4
+        for (; e < quads; e += stride) {
+            const int4 v = t4[e];
+            lo.x = min(lo.x, v.x); lo.y = min(lo.y, v.y); lo.z = min(lo.z, v.z); lo.w = min(lo.w, v.w);
+            hi.x = max(hi.x, v.x); hi.y = max(hi.y, v.y); hi.z = max(hi.z, v.z); hi.w = max(hi.w, v.w);
+        }
+        const int h0 = static_cast<int>((4 * (static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x)) % H);  // 4 * stride is a multiple of H
+        if (lo.x <= hi.x) {
+            atomicMin(&smin[h0], lo.x); atomicMax(&smax[h0], hi.x);
+            atomicMin(&smin[h0 + 1], lo.y); atomicMax(&smax[h0 + 1], hi.y);
+            atomicMin(&smin[h0 + 2], lo.z); atomicMax(&smax[h0 + 2], hi.z);
+            atomicMin(&smin[h0 + 3], lo.w); atomicMax(&smax[h0 + 3], hi.w);
+        }
+    } else if (256 % H == 0) {  // the thread always meets the same hash position
         int32_t lo = INT_MAX, hi = INT_MIN;
 #pragma unroll 4
         for (; e < total; e += stride) {
@@ -54,6 +74,14 @@ __global__ __launch_bounds__(256) void ps_minmax_kernel(const int32_t* __restric
             atomicMin(&mm[(t * H + h) * 2 + 0], smin[h]);
             atomicMax(&mm[(t * H + h) * 2 + 1], smax[h]);
         }
+    }
+}
+
+__global__ __launch_bounds__(256) void ps_minmax_reset_kernel(int32_t* __restrict__ mm, int columns) {
+    const int c = blockIdx.x * 256 + threadIdx.x;
+    if (c < columns) {
+        mm[2 * c] = INT_MAX;
+        mm[2 * c + 1] = INT_MIN;
     }
 }
 
@@ -201,10 +229,7 @@ __global__ __launch_bounds__(256) void ps_keys_to_sig_kernel(const uint32_t* __r
 }  // namespace
 
 void free_ps_codec(culsh_index* ix) {
-    dev_free(ix->psc.vmin);
-    dev_free(ix->psc.range);
-    dev_free(ix->psc.fwd);
-    dev_free(ix->psc.inv);
+    dev_free(ix->psc.vmin);  // one block: vmin | range | fwd | inv
     ix->psc = PsCodec();
 }
 
@@ -213,15 +238,22 @@ culsh_status ps_build_codec(culsh_ctx* ctx, const int32_t* sig, int n, int T, in
     *compressed = false;
     const int TH = T * H;
     if (H > 1024) return CULSH_OK;
-    std::vector<int32_t> mm(static_cast<size_t>(TH) * 2);
-    for (int c = 0; c < TH; ++c) { mm[2 * c] = INT_MAX; mm[2 * c + 1] = INT_MIN; }
     int32_t* mm_dev = nullptr;
-    CULSH_TRY(arena_alloc_t(ctx, mm.size(), &mm_dev));
-    CULSH_HIP(hipMemcpyAsync(mm_dev, mm.data(), mm.size() * sizeof(int32_t), hipMemcpyHostToDevice, ctx->stream));
-    CULSH_HIP(hipStreamSynchronize(ctx->stream));  // `mm` is pageable: the copy must not outlive this scope's reuse
-    const unsigned bx = std::max(1u, std::min(256u, div_up(static_cast<size_t>(n) * H, 256 * 16)));
-    CULSH_LAUNCH(ctx, ps_minmax_kernel, dim3(bx, T), dim3(256), 0, ctx->stream, sig, n, H, mm_dev);
+    CULSH_TRY(arena_alloc_t(ctx, static_cast<size_t>(TH) * 2, &mm_dev));
+    CULSH_LAUNCH(ctx, ps_minmax_reset_kernel, dim3(div_up(static_cast<size_t>(TH), 256)), dim3(256), 0, ctx->stream,
+                 mm_dev, TH);
     CULSH_LAUNCH_CHECK();
+    {
+        const size_t per_table = static_cast<size_t>(n) * H;
+        const bool vec4 = H % 4 == 0 && 1024 % H == 0 && reinterpret_cast<uintptr_t>(sig) % 16 == 0;
+        const unsigned bx = std::max(1u, std::min(256u, div_up(per_table, 256 * (vec4 ? 64 : 16))));
+        if (vec4)
+            CULSH_LAUNCH(ctx, ps_minmax_kernel<true>, dim3(bx, T), dim3(256), 0, ctx->stream, sig, n, H, mm_dev);
+        else
+            CULSH_LAUNCH(ctx, ps_minmax_kernel<false>, dim3(bx, T), dim3(256), 0, ctx->stream, sig, n, H, mm_dev);
+        CULSH_LAUNCH_CHECK();
+    }
+    std::vector<int32_t> mm(static_cast<size_t>(TH) * 2);
     CULSH_HIP(hipMemcpyAsync(mm.data(), mm_dev, mm.size() * sizeof(int32_t), hipMemcpyDeviceToHost, ctx->stream));
     CULSH_HIP(hipStreamSynchronize(ctx->stream));
 
@@ -233,8 +265,13 @@ culsh_status ps_build_codec(culsh_ctx* ctx, const int32_t* sig, int n, int T, in
     if (bits > 12 || W >= H) return CULSH_OK;  // wide value ranges: keep the plain byte order keys
     if (W > 56) return CULSH_OK;               // the restore kernel keeps PS_BPB keys of W words in LDS
 
-    std::vector<int32_t> vmin(TH), range(TH), inv(static_cast<size_t>(TH) * rmax, 0);
-    std::vector<uint32_t> fwd(static_cast<size_t>(TH) * rmax, 0);
+    // one host block, one device block, one copy: vmin[TH] | range[TH] | fwd[TH][rmax] | inv[TH][rmax]
+    const size_t lut = static_cast<size_t>(TH) * rmax;
+    std::vector<int32_t> host(2 * static_cast<size_t>(TH) + 2 * lut, 0);
+    int32_t* vmin = host.data();
+    int32_t* range = vmin + TH;
+    uint32_t* fwd = reinterpret_cast<uint32_t*>(range + TH);
+    int32_t* inv = reinterpret_cast<int32_t*>(fwd + lut);
     std::vector<std::pair<uint32_t, int32_t>> order;
     for (int c = 0; c < TH; ++c) {
         vmin[c] = mm[2 * c];
@@ -253,14 +290,13 @@ culsh_status ps_build_codec(culsh_ctx* ctx, const int32_t* sig, int n, int T, in
     PsCodec& pc = ix->psc;
     pc.bits = bits;
     pc.rmax = static_cast<int>(rmax);
-    CULSH_HIP(dev_malloc(&pc.vmin, TH * sizeof(int32_t)));
-    CULSH_HIP(dev_malloc(&pc.range, TH * sizeof(int32_t)));
-    CULSH_HIP(dev_malloc(&pc.fwd, fwd.size() * sizeof(uint32_t)));
-    CULSH_HIP(dev_malloc(&pc.inv, inv.size() * sizeof(int32_t)));
-    CULSH_HIP(hipMemcpy(pc.vmin, vmin.data(), TH * sizeof(int32_t), hipMemcpyHostToDevice));
-    CULSH_HIP(hipMemcpy(pc.range, range.data(), TH * sizeof(int32_t), hipMemcpyHostToDevice));
-    CULSH_HIP(hipMemcpy(pc.fwd, fwd.data(), fwd.size() * sizeof(uint32_t), hipMemcpyHostToDevice));
-    CULSH_HIP(hipMemcpy(pc.inv, inv.data(), inv.size() * sizeof(int32_t), hipMemcpyHostToDevice));
+    int32_t* block = nullptr;
+    CULSH_HIP(dev_malloc(&block, host.size() * sizeof(int32_t)));
+    pc.vmin = block;
+    pc.range = block + TH;
+    pc.fwd = reinterpret_cast<uint32_t*>(block + 2 * static_cast<size_t>(TH));
+    pc.inv = block + 2 * static_cast<size_t>(TH) + lut;
+    CULSH_HIP(hipMemcpy(block, host.data(), host.size() * sizeof(int32_t), hipMemcpyHostToDevice));
     ix->enc = ENC_PSC;
     ix->key_w = W;
     *compressed = true;
