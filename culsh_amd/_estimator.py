@@ -108,10 +108,16 @@ class LSHEstimator:
         return {}
 
     def _core_for(self, rows: _Rows):
+        """The core for this input.  An estimator keeps its last core: fitting again with the same
+        settings then reuses the core's stream, scratch memory and seeded hash parameters (the
+        reference builds a new core per fit, python/culsh/rp_lsh.py:119-121; the result is the same)."""
         hyper = self._hyper_values(rows)
-        core = self._family.core_cls(self._n_hash_tables, self._n_hashes,
-                                     *(hyper[k] for k in self._family.hyper), self._seed)
-        return core, hyper
+        key = (self._n_hash_tables, self._n_hashes, tuple(hyper[k] for k in self._family.hyper), self._seed)
+        kept = getattr(self, "_kept_core", None)
+        if kept is None or kept[0] != key:
+            kept = (key, self._family.core_cls(self._n_hash_tables, self._n_hashes, *key[2], self._seed))
+            self._kept_core = kept
+        return kept[1], hyper
 
     def _fit(self, X):
         rows = _Rows(X, self._family.dense)

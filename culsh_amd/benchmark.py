@@ -1,0 +1,302 @@
+"""
+Synthetic-data benchmark of the public API: fit / query (or fit_query) timing and recall@k
+against brute-force neighbours, one JSON report per run.
+
+Plays the part of the reference's python/benchmark/bench_base.py + bench_{rplsh,pslsh,minhash}.py
+(fit/query timing around the estimator calls, recall@k for the first `--n-eval-queries`
+queries, report with `runtimes` and `recall_evaluation`).  The reference loads SIFT / GloVe /
+a sparse text corpus from disk; there is no dataset here, so every workload is generated
+from a seed, on the device:
+
+  c1  RPLSH     10,000 x 128 N(0,1) rows, 100 queries, 16 tables x 8 hashes
+  c2  RPLSH     1,000,000 x 128 integers in [0,255] (clipped Gamma(0.5, 30)), 10,000 queries
+                = rows + N(0, 3^2), 32 x 16
+  c3  PStable   1,000,000 x 128 N(0,1), 10,000 queries, 16 x 8, window 4
+  c4  MinHash   1,000,000 rows over 50,000 columns, ~Poisson(50) distinct columns per row
+                drawn Zipf(1.1), 10,000 queries, 32 x 4
+  c5  RPLSH     4,000,000 x 768 rows of a 1000-component Gaussian mixture on the unit sphere,
+                100,000 queries, 64 x 16, batch size 10,000
+
+    python -m culsh_amd.benchmark --config c2
+    python -m culsh_amd.benchmark --config c3 -nt 32 -nh 4 -ne 20 -k 10,100 -r results/
+    python -m culsh_amd.benchmark --config c1 --fit-query --host-inputs
+
+Inputs are resident on the GPU when the timed calls start unless `--host-inputs` is given
+(then the calls receive numpy / scipy objects and their time includes the copy, which is
+how the reference's own benchmark measures).
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+from dataclasses import dataclass
+from typing import Callable, Optional
+
+import numpy as np
+
+from .minhash_lsh import MinHashLSH
+from .pstable_lsh import PStableLSH
+from .rp_lsh import RPLSH
+from .utils import DeviceCSR, compute_recall
+
+
+@dataclass(frozen=True)
+class Workload:
+    family: str              # "rplsh" | "pslsh" | "minhash"
+    n: int
+    d: int
+    n_queries: int
+    n_hash_tables: int
+    n_hashes: int
+    make: Callable           # (torch, n, d, n_queries, generator) -> (X, Q) on the device
+    metric: str              # ground truth: "cosine" | "euclidean" | "jaccard"
+    window_size: Optional[int] = None
+    batch_size: Optional[int] = None
+    describe: str = ""
+
+
+def _normal(torch, n, d, nq, g):
+    return (torch.randn(n, d, device="cuda", generator=g), torch.randn(nq, d, device="cuda", generator=g))
+
+
+def _gamma_ints(torch, n, d, nq, g):
+    # Gamma(k, theta) through the standard sampler, seeded by a state drawn from `g`
+    state = int(torch.randint(0, 2**31 - 1, (1,), device="cuda", generator=g).item())
+    prev = torch.cuda.get_rng_state()
+    torch.cuda.manual_seed(state)
+    conc = torch.full((n, d), 0.5, device="cuda")
+    X = torch._standard_gamma(conc).mul_(30.0).floor_().clamp_(0, 255)
+    torch.cuda.set_rng_state(prev)
+    rows = torch.randint(0, n, (nq,), device="cuda", generator=g)
+    Q = (X[rows] + 3.0 * torch.randn(nq, d, device="cuda", generator=g)).clamp_(0, 255)
+    return X, Q
+
+
+def _mixture(torch, n, d, nq, g):
+    centres = torch.randn(1000, d, device="cuda", generator=g)
+
+    def rows(count):
+        out = torch.empty(count, d, device="cuda", dtype=torch.float32)
+        for s in range(0, count, 500_000):
+            m = min(500_000, count - s)
+            comp = torch.randint(0, 1000, (m,), device="cuda", generator=g)
+            x = centres[comp] + 0.3 * torch.randn(m, d, device="cuda", generator=g)
+            out[s:s + m] = x / x.norm(dim=1, keepdim=True)
+        return out
+
+    return rows(n), rows(nq)
+
+
+def _zipf_sets(torch, n, d, nq, g):
+    """CSR rows of distinct column ids: Poisson(50) draws per row (at least one) from a Zipf(1.1) law
+    over d columns, duplicates inside a row removed."""
+    p = 1.0 / torch.arange(1, d + 1, device="cuda", dtype=torch.float64) ** 1.1
+    cdf = torch.cumsum(p, 0) / p.sum()
+
+    def rows(count):
+        nnz = torch.poisson(torch.full((count,), 50.0, device="cuda"), generator=g).clamp_(min=1).long()
+        owner = torch.repeat_interleave(torch.arange(count, device="cuda"), nnz)
+        cols = torch.searchsorted(cdf, torch.rand(int(nnz.sum()), device="cuda", generator=g, dtype=torch.float64))
+        cols.clamp_(max=d - 1)
+        pairs = torch.unique(owner * d + cols)  # sorted: rows ascending, columns ascending inside a row
+        owner, cols = pairs // d, pairs % d
+        indptr = torch.zeros(count + 1, device="cuda", dtype=torch.int64)
+        indptr[1:] = torch.cumsum(torch.bincount(owner, minlength=count), 0)
+        return DeviceCSR(cols.to(torch.int32), indptr.to(torch.int32), (count, d))
+
+    return rows(n), rows(nq)
+
+
+WORKLOADS = {
+    "c1": Workload("rplsh", 10_000, 128, 100, 16, 8, _normal, "cosine", describe="N(0,1) rows"),
+    "c2": Workload("rplsh", 1_000_000, 128, 10_000, 32, 16, _gamma_ints, "cosine",
+                   describe="integers in [0,255] from a clipped Gamma(0.5, 30); queries = rows + N(0, 3^2)"),
+    "c3": Workload("pslsh", 1_000_000, 128, 10_000, 16, 8, _normal, "euclidean", window_size=4,
+                   describe="N(0,1) rows"),
+    "c4": Workload("minhash", 1_000_000, 50_000, 10_000, 32, 4, _zipf_sets, "jaccard",
+                   describe="~Poisson(50) distinct columns per row, Zipf(1.1) over 50,000 columns"),
+    "c5": Workload("rplsh", 4_000_000, 768, 100_000, 64, 16, _mixture, "cosine", batch_size=10_000,
+                   describe="1000-component Gaussian mixture (sigma 0.3) on the unit sphere"),
+}
+
+
+# --------------------------------------------------------------------------------------
+# brute-force neighbours of one query (the reference's get_ground_truth_top_k)
+# --------------------------------------------------------------------------------------
+def _top_k(torch, metric: str, X, Q, qi: int, k: int, cache: dict):
+    if metric == "jaccard":
+        q_cols = Q.indices[int(Q.indptr[qi]):int(Q.indptr[qi + 1])].long()
+        member = torch.zeros(X.shape[1], device="cuda", dtype=torch.float32)
+        member[q_cols] = 1.0
+        hits = torch.cumsum(member[X.indices.long()].double(), 0)
+        hits = torch.cat([hits.new_zeros(1), hits])
+        ptr = X.indptr.long()
+        inter = hits[ptr[1:]] - hits[ptr[:-1]]
+        sizes = (ptr[1:] - ptr[:-1]).double()
+        union = sizes + float(len(q_cols)) - inter
+        score = torch.where(union > 0, inter / union, torch.zeros_like(union))
+    elif metric == "cosine":
+        if "xn" not in cache:
+            cache["xn"] = X.norm(dim=1).clamp_min(1e-30)
+        q = Q[qi]
+        score = (X @ q) / (cache["xn"] * q.norm().clamp_min(1e-30))
+    else:  # euclidean: smallest distance = largest negative squared distance
+        if "x2" not in cache:
+            cache["x2"] = (X * X).sum(1)
+        q = Q[qi]
+        score = -(cache["x2"] - 2.0 * (X @ q) + (q * q).sum())
+    return torch.topk(score, min(k, score.numel())).indices
+
+
+def evaluate_recall(torch, metric: str, X, Q, candidates, n_eval: int, ks: list[int]) -> dict:
+    offsets = candidates.get_offsets().astype(np.int64)
+    indices = candidates.get_indices(as_torch=True)
+    n_eval = min(n_eval, candidates.n_queries)
+    per_k = {k: [] for k in ks}
+    counts, with_candidates, cache = [], 0, {}
+    for i in range(n_eval):
+        mine = indices[int(offsets[i]):int(offsets[i + 1])]
+        counts.append(int(mine.numel()))
+        if mine.numel() == 0:
+            for k in ks:
+                per_k[k].append(0.0)
+            continue
+        with_candidates += 1
+        for k in ks:
+            per_k[k].append(compute_recall(mine, _top_k(torch, metric, X, Q, i, k, cache)))
+    return {"n_eval_queries": n_eval, "queries_with_candidates": with_candidates,
+            "recall_at_k": {str(k): float(np.mean(v)) if v else 0.0 for k, v in per_k.items()},
+            "mean_candidates": float(np.mean(counts)) if counts else 0.0,
+            "per_query_recall_at_k": {str(k): [float(x) for x in v] for k, v in per_k.items()}}
+
+
+# --------------------------------------------------------------------------------------
+def _to_host(torch, A):
+    if isinstance(A, DeviceCSR):
+        import scipy.sparse as sp
+
+        ind, ptr = A.indices.cpu().numpy(), A.indptr.cpu().numpy()
+        return sp.csr_matrix((np.ones(len(ind), dtype=np.float32), ind, ptr), shape=A.shape)
+    return A.cpu().numpy()
+
+
+def _slice_rows(A, count: int):
+    if isinstance(A, DeviceCSR):
+        end = int(A.indptr[count])
+        return DeviceCSR(A.indices[:end].contiguous(), A.indptr[:count + 1].contiguous(), (count, A.shape[1]))
+    return A[:count].contiguous()
+
+
+def make_estimator(w: Workload, args):
+    T = args.n_hash_tables or w.n_hash_tables
+    H = args.n_hashes or w.n_hashes
+    if w.family == "rplsh":
+        return RPLSH(n_hash_tables=T, n_hashes=H, seed=args.seed), {}
+    if w.family == "pslsh":
+        ws = args.window_size if args.window_size is not None else w.window_size
+        ws = "auto" if ws in (None, 0) else ws
+        return PStableLSH(n_hash_tables=T, n_hashes=H, window_size=ws, seed=args.seed), {"window_size": ws}
+    return MinHashLSH(n_hash_tables=T, n_hashes=H, seed=args.seed), {}
+
+
+def run(args) -> dict:
+    import torch
+
+    w = WORKLOADS[args.config]
+    n = args.n_samples or w.n
+    nq = args.n_queries or w.n_queries
+    batch = args.batch_size if args.batch_size is not None else w.batch_size
+    g = torch.Generator(device="cuda")
+    g.manual_seed(args.data_seed)
+    X, Q = w.make(torch, n, w.d, nq, g)
+    torch.cuda.synchronize()
+    est, extra = make_estimator(w, args)
+    fit_in, query_in = X, Q
+    if args.fit_query:
+        fit_in = query_in = _slice_rows(X, min(nq, n))  # the reference's -fq: the first n_queries rows
+    if args.host_inputs:
+        fit_in = _to_host(torch, fit_in)
+        query_in = fit_in if args.fit_query else _to_host(torch, Q)
+
+    def timed(fn):
+        best, out = float("inf"), None
+        for rep in range(args.repeats + 1):  # the first call also pays one-off costs (library load, arena growth)
+            out = None
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            out = fn()
+            dt = time.perf_counter() - t0
+            if rep > 0 or args.repeats == 0:
+                best = min(best, dt)
+        return best, out
+
+    runtimes, throughput, index_info = {}, {}, {}
+    if args.fit_query:
+        kw = {"batch_size": batch} if batch else {}
+        t, cands = timed(lambda: est.fit_query(fit_in, **kw))
+        runtimes["fit_query_time"] = t
+        X_eval = Q_eval = _slice_rows(X, min(nq, n))
+    else:
+        t_fit, model = timed(lambda: est.fit(fit_in))
+        kw = {"batch_size": batch} if batch else {}
+        t_query, cands = timed(lambda: model.query(query_in, **kw))
+        runtimes.update(fit_time=t_fit, query_time=t_query)
+        throughput.update(fit_mvec_per_s=n / t_fit / 1e6, query_per_s=nq / t_query)
+        index_info = {"n_total_buckets": int(model.index.n_total_buckets), "size_bytes": int(model.index.size_bytes())}
+        X_eval, Q_eval = X, Q
+    ks = [int(k) for k in args.recall_k.split(",") if k.strip()]
+    recall = evaluate_recall(torch, w.metric, X_eval, Q_eval, cands, args.n_eval_queries, ks)
+    return {
+        "algorithm": {"rplsh": "RPLSH", "pslsh": "PStableLSH", "minhash": "MinHashLSH"}[w.family],
+        "config": args.config,
+        "data": {"kind": "synthetic", "description": w.describe, "seed": args.data_seed, "n_samples": n,
+                 "n_features": w.d, "inputs": "host (copy inside the timed calls)" if args.host_inputs else "resident on the GPU"},
+        "params": dict({"n_hash_tables": args.n_hash_tables or w.n_hash_tables, "n_hashes": args.n_hashes or w.n_hashes,
+                        "seed": args.seed, "n_queries": nq, "recall_k": ks, "batch_size": batch,
+                        "mode": "fit_query" if args.fit_query else "fit+query"}, **extra),
+        "runtimes": runtimes,
+        "throughput": throughput,
+        "index": index_info,
+        "candidates": {"n_total_candidates": int(cands.n_total_candidates)},
+        "recall_evaluation": recall,
+    }
+
+
+def main(argv=None) -> int:
+    ap = argparse.ArgumentParser(description="Benchmark the LSH estimators on a synthetic workload")
+    ap.add_argument("-c", "--config", choices=sorted(WORKLOADS), default="c2")
+    ap.add_argument("-n", "--n-samples", type=int, default=None, help="override the number of rows")
+    ap.add_argument("-nt", "--n-hash-tables", type=int, default=None)
+    ap.add_argument("-nh", "--n-hashes", type=int, default=None)
+    ap.add_argument("-w", "--window-size", type=int, default=None, help="p-stable window (0 = 'auto')")
+    ap.add_argument("-s", "--seed", type=int, default=42, help="seed of the hash parameters")
+    ap.add_argument("--data-seed", type=int, default=1234)
+    ap.add_argument("-nq", "--n-queries", type=int, default=None)
+    ap.add_argument("-ne", "--n-eval-queries", type=int, default=10)
+    ap.add_argument("-k", "--recall-k", type=str, default="10,100")
+    ap.add_argument("-bs", "--batch-size", type=int, default=None)
+    ap.add_argument("-fq", "--fit-query", action="store_true", help="fit_query on the first n_queries rows")
+    ap.add_argument("--host-inputs", action="store_true", help="hand numpy / scipy inputs to the estimator")
+    ap.add_argument("--repeats", type=int, default=3, help="timed repetitions after one untimed call (best is kept)")
+    ap.add_argument("-r", "--results-dir", type=str, default=None)
+    args = ap.parse_args(argv)
+    report = run(args)
+    text = json.dumps(report, indent=2)
+    if args.results_dir:
+        os.makedirs(args.results_dir, exist_ok=True)
+        path = os.path.join(args.results_dir, f"report_{report['algorithm'].lower()}_{args.config}_"
+                                              f"{time.strftime('%Y%m%d_%H%M%S')}.json")
+        with open(path, "w") as f:
+            f.write(text + "\n")
+        print(path)
+    else:
+        print(text)
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -7,6 +7,8 @@
 #include <cstring>
 #include <memory>
 #include <new>
+#include <thread>
+#include <vector>
 
 #include "common.hpp"
 
@@ -162,15 +164,37 @@ void gen_raw_u64(uint64_t seed, int stream, size_t n, uint64_t* out) {
 }
 
 // Box-Muller: z = sqrt(-2 ln u1) cos(2 pi u2), u1 in (0,1], u2 in [0,1), 53-bit uniforms.
+// Element i depends on (key, i) alone, so large requests are cut into ranges for a few host threads.
 void gen_normals_f64(uint64_t seed, int stream, size_t n, double* out) {
     const uint64_t key = sm64(sm64(seed) ^ sm64(static_cast<uint64_t>(stream)));
-    const double inv = 1.0 / 9007199254740992.0;
-    const double two_pi = 6.283185307179586476925286766559;
-    for (size_t i = 0; i < n; ++i) {
-        const double u1 = static_cast<double>((sm64(key + 2 * i) >> 11) + 1) * inv;
-        const double u2 = static_cast<double>(sm64(key + 2 * i + 1) >> 11) * inv;
-        out[i] = std::sqrt(-2.0 * std::log(u1)) * std::cos(two_pi * u2);
+    auto range = [key, out](size_t lo, size_t hi) {
+        const double inv = 1.0 / 9007199254740992.0;
+        const double two_pi = 6.283185307179586476925286766559;
+        for (size_t i = lo; i < hi; ++i) {
+            const double u1 = static_cast<double>((sm64(key + 2 * i) >> 11) + 1) * inv;
+            const double u2 = static_cast<double>(sm64(key + 2 * i + 1) >> 11) * inv;
+            out[i] = std::sqrt(-2.0 * std::log(u1)) * std::cos(two_pi * u2);
+        }
+    };
+    const size_t per_thread = 8192;
+    const unsigned hw = std::max(1u, std::thread::hardware_concurrency());
+    const size_t want = std::min<size_t>({static_cast<size_t>(16), static_cast<size_t>(hw), n / per_thread});
+    if (want < 2) {
+        range(0, n);
+        return;
     }
+    std::vector<std::thread> workers;
+    const size_t chunk = (n + want - 1) / want;
+    for (size_t w = 1; w < want; ++w) {
+        const size_t lo = std::min(n, w * chunk), hi = std::min(n, lo + chunk);
+        try {
+            workers.emplace_back(range, lo, hi);
+        } catch (...) {  // no thread to be had: this one does the range itself
+            range(lo, hi);
+        }
+    }
+    range(0, std::min(n, chunk));
+    for (std::thread& t : workers) t.join();
 }
 
 template <typename T>
