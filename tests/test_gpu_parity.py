@@ -731,6 +731,58 @@ def test_config5_full_size_invariants(ctx):
     ctx.lib.culsh_memory_trim()
 
 
+@pytest.mark.parametrize("first_seed", [0, 12, 24])
+def test_random_shapes_all_families(ctx, first_seed):
+    """Twelve seeded draws per case of (family, rows, queries, tables, hashes, features, dtype, batch
+    size) from lists that sit on and around the tile sizes of the kernels: index, candidates (batched
+    or not) and fit_query against the oracle given the GPU's own signatures."""
+    from abi import assert_candidates_match, assert_index_matches
+
+    for s in range(first_seed, first_seed + 12):
+        rng = np.random.default_rng(s)
+        fam = ["rplsh", "pslsh", "minhash"][s % 3]
+        n = int(rng.choice([1, 2, 63, 64, 65, 127, 128, 129, 1000, 4095, 4096, 4097, 8191, 8192, 8193, 12345, 20000]))
+        nq = int(rng.choice([1, 3, 64, 100, 257]))
+        T = int(rng.choice([1, 2, 3, 7, 16, 33, 70]))
+        H = int(rng.choice([1, 2, 3, 4, 5, 8, 12, 16, 17, 32, 33, 40]))
+        d = int(rng.choice([1, 3, 4, 15, 16, 17, 64, 100, 128, 130]))
+        dtype = np.float32 if rng.random() < 0.7 else np.float64
+        bs = int(rng.choice([-1, 1, 10, 64]))
+        _announce("random_shapes", s, fam, n, nq, T, H, d, dtype.__name__, bs)
+        if fam == "minhash":
+            dcols = int(rng.choice([5, 50, 400, 70000]))
+            nnz = int(rng.choice([1, 4, 30]))
+            indices, indptr = make_csr(rng, n, dcols, nnz, empty_rows=(0,) if n > 3 and rng.random() < 0.5 else ())
+            qindices, qindptr = make_csr(rng, nq, dcols, nnz)
+            A, B = o.generate_hash_integers(s, T * H)
+            sig = o.minhash_hash(indices, indptr, A, B, T, H)
+            qsig = o.minhash_hash(qindices, qindptr, A, B, T, H)
+            ih = ctx.minhash_fit(indices, indptr, dcols, T, H, A=A, B=B)
+            got_q = ctx.minhash_query(qindices, qindptr, ih)
+            got_fq = ctx.minhash_fit_query(indices, indptr, dcols, T, H, A=A, B=B)
+        else:
+            X = rng.standard_normal((n, d)).astype(dtype)
+            Q = np.concatenate([X[:min(n, nq // 2 + 1)], rng.standard_normal((nq, d)).astype(dtype)])[:nq]
+            if fam == "rplsh":
+                P = rng.standard_normal((T * H, d)).astype(dtype)
+                sig, qsig = ctx.rplsh_hash(X, P, T, H), ctx.rplsh_hash(Q, P, T, H)
+                ih = ctx.rplsh_fit(X, T, H, P=P)
+                got_q = ctx.rplsh_query(Q, ih, batch_size=bs)
+                got_fq = ctx.rplsh_fit_query(X, T, H, P=P)
+            else:
+                w = int(rng.choice([1, 2, 4, 50]))
+                P, b = o.generate_random_projections_biases(s, T * H, d, w, dtype)
+                sig, qsig = ctx.pslsh_hash(X, P, b, T, H), ctx.pslsh_hash(Q, P, b, T, H)
+                ih = ctx.pslsh_fit(X, T, H, w, P=P, b=b)
+                got_q = ctx.pslsh_query(Q, ih, batch_size=bs)
+                got_fq = ctx.pslsh_fit_query(X, T, H, w, P=P, b=b)
+        exp_ix = o.fit_index(sig, H)
+        assert_index_matches(ctx.index_arrays(ih), exp_ix)
+        assert_candidates_match(got_q, o.query_index(qsig, exp_ix))
+        assert_candidates_match(got_fq, o.fit_query(sig, H))
+        ctx.free_index(ih)
+
+
 def test_minhash_rank_keys_edge_cases(ctx):
     """MinHash keys are stored as column ranks when every fitted column id is below n_features.
     Checked against the oracle: query rows whose minimum comes from a column >= n_features (they
