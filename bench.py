@@ -166,8 +166,8 @@ def main() -> int:
                     "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s",
                     "frac": round(achieved / PEAK_FP32_MFMA_TFLOPS, 4),
                     # HBM bytes of the fit launch at the default size: rocprofv3 FETCH_SIZE x 2.0
-                    # (494.7 MiB) + WRITE_SIZE x 1.0 (122.1 MiB), scale factors from a 1 GiB copy
-                    "traffic": 646_800_000 if (n, nq) == (1_000_000, 10_000) else None,
+                    # (490.4 MiB) + WRITE_SIZE x 1.0 (122.1 MiB), scale factors from a 1 GiB copy
+                    "traffic": 642_300_000 if (n, nq) == (1_000_000, 10_000) else None,
                     "work": "2*(n+q)*d*T*H flop per step over the fit and query launches",
                     "dominant_kernel_by_time": dominant}
 
