@@ -115,6 +115,28 @@ def test_rplsh_fit_query_equals_fit_then_query(dtype):
     np.testing.assert_array_equal(a.get_indices(), c.get_indices())
 
 
+def test_estimator_fitted_again_matches_fresh_estimators():
+    """An estimator keeps its core (stream, scratch, seeded parameters) between fits: fitting it on
+    other data, another shape and another dtype gives what a fresh estimator gives, and models
+    fitted earlier keep answering from their own index."""
+    from culsh_amd import RPLSH, PStableLSH
+
+    lsh = RPLSH(n_hash_tables=8, n_hashes=8, seed=7)
+    inputs = [dense(500, 32, np.float32, seed=1), dense(700, 48, np.float32, seed=2), dense(300, 32, np.float64, seed=3)]
+    models = [lsh.fit(X) for X in inputs]
+    for X, model in zip(inputs, models):
+        fresh = RPLSH(n_hash_tables=8, n_hashes=8, seed=7).fit(X)
+        a, b = model.query(X[:50]), fresh.query(X[:50])
+        np.testing.assert_array_equal(a.get_indices(), b.get_indices())
+        np.testing.assert_array_equal(a.get_offsets(), b.get_offsets())
+        np.testing.assert_array_equal(model.index.get_projection_matrix(), fresh.index.get_projection_matrix())
+    ps = PStableLSH(n_hash_tables=4, n_hashes=4, window_size="auto", seed=3)   # the window, hence the core, follows the data
+    for X in (inputs[0], 10.0 * inputs[0]):
+        a = ps.fit(X).query(X[:20])
+        b = PStableLSH(n_hash_tables=4, n_hashes=4, window_size="auto", seed=3).fit(X).query(X[:20])
+        np.testing.assert_array_equal(a.get_indices(), b.get_indices())
+
+
 @pytest.mark.parametrize("batch_size", [10, 50, 100])
 def test_rplsh_batched_query(batch_size):
     """python/tests/test_rplsh.py:177-209"""
