@@ -309,11 +309,12 @@ def test_core_query_after_look_back_gives_up(ctx, monkeypatch):
     ctx.free_index(ih)
 
 
-def test_core_query_more_than_64_tables(ctx):
-    """More tables than a wavefront has lanes (the spans of the next query are then not prefetched)."""
-    _announce("many_tables")
+@pytest.mark.parametrize("T,n,nq,H", [(90, 3000, 400, 3), (1024, 300, 40, 2)])
+def test_core_query_more_than_64_tables(ctx, T, n, nq, H):
+    """More tables than a wavefront has lanes (the spans of the next query are then not prefetched),
+    up to the most a query supports (one thread per table); one more is an error, not a wrong answer."""
+    _announce("many_tables", T)
     rng = np.random.default_rng(6)
-    T, n, nq, H = 90, 3000, 400, 3
     sig = random_sigs(rng, T, n, H, "rplsh")
     qsig = random_sigs(rng, T, nq, H, "rplsh")
     ih, _ = ctx.core_fit_index(sig, H)
@@ -321,6 +322,12 @@ def test_core_query_more_than_64_tables(ctx):
 
     assert_candidates_match(ctx.core_query_index(qsig, ih), o.query_index(qsig, o.fit_index(sig, H)))
     ctx.free_index(ih)
+    if T == 1024:
+        too_many = rng.integers(0, 2, size=(T + 1, 20, 1), dtype=np.uint8)
+        ih2, _ = ctx.core_fit_index(too_many, 1)
+        with pytest.raises(RuntimeError, match="n_hash_tables > 1024"):
+            ctx.core_query_index(too_many[:, :5], ih2)
+        ctx.free_index(ih2)
 
 
 def test_core_query_tables_that_overlap_completely(ctx, c_oracle):
