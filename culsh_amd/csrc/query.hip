@@ -239,20 +239,21 @@ __device__ __forceinline__ unsigned long long look_back(unsigned long long* stat
     return excl;
 }
 
-// The `ew` (8, 4 or 1) consecutive bitmap words a lane owns in one read-out step.
+// The `ew` (8, 4 or 1) consecutive bitmap words a lane owns in one read-out step.  The words are
+// merged from the three cases as two vector values and only then spread into the array: filling
+// the array inside the branches makes the compiler keep it in scratch memory.
 __device__ __forceinline__ void load_step_words(const uint32_t* p, int ew, uint32_t (&words)[8]) {
+    uint4 v0 = make_uint4(0u, 0u, 0u, 0u), v1 = make_uint4(0u, 0u, 0u, 0u);
     if (ew == 8) {
-        const uint4 v0 = *reinterpret_cast<const uint4*>(p), v1 = *reinterpret_cast<const uint4*>(p + 4);
-        words[0] = v0.x; words[1] = v0.y; words[2] = v0.z; words[3] = v0.w;
-        words[4] = v1.x; words[5] = v1.y; words[6] = v1.z; words[7] = v1.w;
+        v0 = *reinterpret_cast<const uint4*>(p);
+        v1 = *reinterpret_cast<const uint4*>(p + 4);
     } else if (ew == 4) {
-        const uint4 v0 = *reinterpret_cast<const uint4*>(p);
-        words[0] = v0.x; words[1] = v0.y; words[2] = v0.z; words[3] = v0.w;
-        words[4] = words[5] = words[6] = words[7] = 0u;
+        v0 = *reinterpret_cast<const uint4*>(p);
     } else {
-        words[0] = p[0];
-        words[1] = words[2] = words[3] = words[4] = words[5] = words[6] = words[7] = 0u;
+        v0.x = p[0];
     }
+    words[0] = v0.x; words[1] = v0.y; words[2] = v0.z; words[3] = v0.w;
+    words[4] = v1.x; words[5] = v1.y; words[6] = v1.z; words[7] = v1.w;
 }
 
 // One workgroup per query.  COUNT marks the rows of the query's spans in the LDS bitmap and
