@@ -153,15 +153,16 @@ __device__ __forceinline__ void walk_candidates(const int32_t* __restrict__ cand
         __syncthreads();
         const uint32_t here = min(static_cast<uint32_t>(DD_THREADS), n_pieces - r0);
         for (uint32_t p0 = wave; p0 < here; p0 += NWAVES * WALK_U) {
+            // table entries of all pieces first (one LDS round trip instead of one per piece), then the loads
             int rows[WALK_U];
+            int2 ent[WALK_U];
+#pragma unroll
+            for (int u = 0; u < WALK_U; ++u) ent[u] = tab[min(p0 + u * NWAVES, here - 1u)];
 #pragma unroll
             for (int u = 0; u < WALK_U; ++u) {
                 const uint32_t pi = p0 + u * NWAVES;
                 rows[u] = -1;
-                if (pi < here) {  // uniform across the wavefront
-                    const int2 e = tab[pi];
-                    if (lane < (e.y & 255)) rows[u] = cand[e.x + lane];
-                }
+                if (pi < here && lane < (ent[u].y & 255)) rows[u] = cand[ent[u].x + lane];
             }
 #pragma unroll
             for (int u = 0; u < WALK_U; ++u) {
