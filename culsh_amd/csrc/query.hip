@@ -171,7 +171,7 @@ __device__ __forceinline__ void walk_candidates(const int32_t* __restrict__ cand
                     const uint32_t pi = p0 + u * NWAVES;
                     if (pi < here) {
                         const unsigned long long below = __ballot(static_cast<uint32_t>(rows[u]) < row_end);  // -1 is not
-                        if (lane == 0 && below) atomicAdd(&s_cnt[tab[pi].y >> 8], __popcll(below));
+                        if (lane == 0 && below) atomicAdd(&s_cnt[ent[u].y >> 8], __popcll(below));
                     }
                 }
             }
