@@ -790,6 +790,31 @@ def test_random_shapes_all_families(ctx, first_seed):
         ctx.free_index(ih)
 
 
+def test_objects_cross_contexts(ctx):
+    """An index built through one context answers queries issued through another (objects belong to
+    the device, not to the context that made them), also after the first context is gone, and two
+    contexts used in turns do not disturb each other's scratch memory."""
+    _announce("cross_contexts")
+    from abi import Ctx, assert_candidates_match
+
+    rng = np.random.default_rng(11)
+    T, n, nq, H = 5, 6000, 120, 3
+    sig = random_sigs(rng, T, n, H, "rplsh")
+    qsig = random_sigs(rng, T, nq, H, "rplsh")
+    exp = o.query_index(qsig, o.fit_index(sig, H))
+    other = Ctx(0)
+    ih, _ = other.core_fit_index(sig, H)
+    assert_candidates_match(ctx.core_query_index(qsig, ih), exp)        # built there, queried here
+    ih2, _ = ctx.core_fit_index(sig, H)
+    for _ in range(3):                                                    # in turns
+        assert_candidates_match(other.core_query_index(qsig, ih2), exp)
+        assert_candidates_match(ctx.core_query_index(qsig, ih), exp)
+    other.close()
+    assert_candidates_match(ctx.core_query_index(qsig, ih), exp)        # its maker is gone
+    ctx.free_index(ih)
+    ctx.free_index(ih2)
+
+
 def test_minhash_rank_keys_edge_cases(ctx):
     """MinHash keys are stored as column ranks when every fitted column id is below n_features.
     Checked against the oracle: query rows whose minimum comes from a column >= n_features (they
