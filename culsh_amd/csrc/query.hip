@@ -14,9 +14,9 @@
 // workgroup publishes its count and obtains the sum of its predecessors' counts by
 // looking back over their published values (a chained scan), then stores its list.  The
 // output is allocated for the number of raw candidates, an upper bound of the result.
-// Larger row ranges take several passes per query, in the same launch: a query's spans
-// shrink from pass to pass (rows ascend inside a bucket), its list is written where its raw
-// candidates would start (no workgroup waits for another), and a copy closes the gaps
+// Larger row ranges take several passes per query, in the same launch: rows ascend inside a
+// bucket, so a search cuts every span at the passes' row bounds and a pass reads only its own
+// part; the query's list is written where its raw candidates would start (no workgroup waits for another), and a copy closes the gaps
 // between the lists afterwards.  A path of two launches (count, scan, emit) with no
 // cooperation between workgroups stands behind both.
 #include <algorithm>
@@ -130,13 +130,10 @@ constexpr int WALK_U = 16;  // pieces in flight per wavefront
 // starts is looked up once per piece (one binary search per thread over the spans'
 // piece counts, all pieces of a round in parallel) and kept in `tab`, so the per-lane
 // work is an add, a compare and the load.  Contains barriers: all threads must call it.
-// TALLY: also counts, per span, the visited rows below `row_end` into s_cnt (zero on entry); the
-// rows of a span ascend, so that count is how far the span's next pass may skip.
-template <bool TALLY, typename F>
+template <typename F>
 __device__ __forceinline__ void walk_candidates(const int32_t* __restrict__ cand, const int* s_start,
                                                 const int* s_len, const uint32_t* s_ppref, int T,
-                                                uint32_t n_pieces, int2* tab, uint32_t row_end, int* s_cnt,
-                                                F&& f) {
+                                                uint32_t n_pieces, int2* tab, F&& f) {
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     for (uint32_t r0 = 0; r0 < n_pieces; r0 += DD_THREADS) {
         const uint32_t pc = r0 + static_cast<uint32_t>(tid);
@@ -147,8 +144,7 @@ __device__ __forceinline__ void walk_candidates(const int32_t* __restrict__ cand
                 if (s_ppref[mid] <= pc) tl = mid; else th = mid;
             }
             const int first = static_cast<int>(pc - s_ppref[tl]) * 64;
-            // (length, span) share a word: lengths are at most 64
-            tab[tid] = make_int2(s_start[tl] + first, min(64, s_len[tl] - first) | (tl << 8));
+            tab[tid] = make_int2(s_start[tl] + first, min(64, s_len[tl] - first));
         }
         __syncthreads();
         const uint32_t here = min(static_cast<uint32_t>(DD_THREADS), n_pieces - r0);
@@ -162,21 +158,40 @@ __device__ __forceinline__ void walk_candidates(const int32_t* __restrict__ cand
             for (int u = 0; u < WALK_U; ++u) {
                 const uint32_t pi = p0 + u * NWAVES;
                 rows[u] = -1;
-                if (pi < here && lane < (ent[u].y & 255)) rows[u] = cand[ent[u].x + lane];
+                if (pi < here && lane < ent[u].y) rows[u] = cand[ent[u].x + lane];
             }
 #pragma unroll
-            for (int u = 0; u < WALK_U; ++u) {
+            for (int u = 0; u < WALK_U; ++u)
                 if (rows[u] >= 0) f(rows[u]);
-                if (TALLY) {
-                    const uint32_t pi = p0 + u * NWAVES;
-                    if (pi < here) {
-                        const unsigned long long below = __ballot(static_cast<uint32_t>(rows[u]) < row_end);  // -1 is not
-                        if (lane == 0 && below) atomicAdd(&s_cnt[ent[u].y >> 8], __popcll(below));
-                    }
-                }
-            }
         }
         __syncthreads();  // tab is rewritten by the next round
+    }
+}
+
+constexpr int SPLIT_BATCH = 3;  // row bounds located per search round of split_spans
+
+// The rows of a span ascend.  For every span t < T and each of the K row bounds bound0 + k * chunk_rows
+// this counts the span's rows below the bound, into s_split[k * T + t].  Four neighbouring lanes share
+// one search and cut its range into five parts per round: a span of 500 rows takes four dependent
+// loads, and 256 searches run side by side.  All threads must call it; the caller places the barriers.
+__device__ __forceinline__ void split_spans(const int32_t* __restrict__ cand, const int* s_org_start,
+                                            const int* s_org_len, int T, int K, uint32_t bound0,
+                                            uint32_t chunk_rows, int* s_split) {
+    const int sub = threadIdx.x & 3, group_shift = threadIdx.x & 60;
+    for (int task = threadIdx.x >> 2; task < T * K; task += DD_THREADS / 4) {
+        const int k = task / T, t = task - k * T;
+        const uint32_t bound = bound0 + static_cast<uint32_t>(k) * chunk_rows;
+        const int32_t* rows = cand + s_org_start[t];
+        int first = 0, len = s_org_len[t];  // rows before `first` are below the bound, rows from first + len on are not
+        while (len > 0) {
+            const int step = (len + 4) / 5, end = first + len;
+            const int pos = first + (sub + 1) * step - 1;  // last row of part `sub`
+            const bool below = pos < end && static_cast<uint32_t>(rows[pos]) < bound;
+            const int nb = __popc(static_cast<uint32_t>(__ballot(below) >> group_shift) & 15u);  // parts wholly below
+            first += nb * step;
+            len = nb == 4 ? end - first : min(step - 1, end - first);  // what is left of part `nb`, minus its probed last row
+        }
+        if (sub == 0) s_split[task] = first;
     }
 }
 
@@ -276,7 +291,10 @@ __global__ __launch_bounds__(DD_THREADS) void dedup_kernel(DedupArgs a) {
     uint32_t* s_ppref = reinterpret_cast<uint32_t*>(s_len + T);  // [T+1]
     uint32_t* scratch = s_ppref + T + 1;                         // [17]
     uint32_t* wtot = scratch + 17;                               // [NWAVES + 1]
-    int* s_cnt = reinterpret_cast<int*>(wtot + NWAVES + 1);      // [T] FUSED with several passes: rows of the pass, per span
+    // FUSED with several passes: the query's spans as given, and where the next row bounds cut them
+    int* s_org_start = reinterpret_cast<int*>(wtot + NWAVES + 1);  // [T]
+    int* s_org_len = s_org_start + T;                              // [T]
+    int* s_split = s_org_len + T;                                  // [SPLIT_BATCH][T]
 
 #define DD_TICK(k)                                                                      \
     if (a.ticks && tid == 0) {                                                          \
@@ -306,8 +324,18 @@ __global__ __launch_bounds__(DD_THREADS) void dedup_kernel(DedupArgs a) {
   for (;;) {  // the queries of this workgroup (a single one unless FUSED)
     int q_next = a.n_queries;
     int2 sp_next = make_int2(0, 0);
-    uint32_t n_pieces;
-    {
+    // FUSED with several passes: a query's list starts where its raw candidates would (no dependence
+    // on other queries, the host closes the gaps afterwards), and every pass walks the part of each
+    // span whose rows fall into its range; split_spans finds those parts, a few passes ahead.
+    constexpr bool several = MODE == DD_FUSED_PASSES;
+    uint32_t n_pieces = 0;
+    int covered = 0;  // several passes: rows of span `tid` that earlier passes walked
+    if (several) {
+        if (tid < T) {
+            s_org_start[tid] = sp.x;
+            s_org_len[tid] = sp.y;
+        }
+    } else {
         if (tid < T) {
             s_start[tid] = sp.x;
             s_len[tid] = sp.y;
@@ -320,10 +348,6 @@ __global__ __launch_bounds__(DD_THREADS) void dedup_kernel(DedupArgs a) {
     const uint64_t out_base = MODE == DD_EMIT ? a.offsets[q] : 0;
     const uint32_t chunk_rows = static_cast<uint32_t>(chunk_words) * 32u;
 
-    // FUSED with several passes: a query's list starts where its raw candidates would (no dependence
-    // on other queries, the host closes the gaps afterwards), and the spans shrink from pass to pass
-    // by the rows already written.
-    constexpr bool several = MODE == DD_FUSED_PASSES;
     const unsigned long long raw_base = several ? a.raw_offsets[q] : 0ull;
     for (int chunk = 0; chunk < a.n_chunks; ++chunk) {
         const uint32_t lo = static_cast<uint32_t>(chunk) * chunk_rows;
@@ -332,8 +356,27 @@ __global__ __launch_bounds__(DD_THREADS) void dedup_kernel(DedupArgs a) {
             uint4* bm4 = reinterpret_cast<uint4*>(bm);
             for (int i = tid; i < chunk_words / 4; i += DD_THREADS) bm4[i] = make_uint4(0u, 0u, 0u, 0u);
         }
+        if (several) {
+            const int ahead = chunk % SPLIT_BATCH;
+            if (ahead == 0 && !last) {
+                __syncthreads();  // the spans are in place, the previous bounds are used up
+                split_spans(a.cand, s_org_start, s_org_len, T, min(SPLIT_BATCH, a.n_chunks - 1 - chunk),
+                            lo + chunk_rows, chunk_rows, s_split);
+                __syncthreads();
+            }
+            uint32_t pieces = 0;
+            if (tid < T) {
+                const int end = last ? sp.y : s_split[ahead * T + tid];
+                s_start[tid] = sp.x + covered;
+                s_len[tid] = end - covered;
+                pieces = (static_cast<uint32_t>(end - covered) + 63u) >> 6;
+                covered = end;
+            }
+            const uint32_t ex = block_exclusive_sum(pieces, scratch, &n_pieces);
+            if (tid < T) s_ppref[tid] = ex;
+            if (tid == 0) s_ppref[T] = n_pieces;
+        }
         if (tid <= NWAVES) wtot[tid] = 0;
-        if (several && tid < T) s_cnt[tid] = 0;
         __syncthreads();
         DD_TICK(0)  // setup + clear
         // Mark the rows of this pass (collect_candidates_kernel, core/query.cuh:199-237, but into
@@ -350,22 +393,7 @@ __global__ __launch_bounds__(DD_THREADS) void dedup_kernel(DedupArgs a) {
                 }
             }
         };
-        if (several && !last) {
-            walk_candidates<true>(a.cand, s_start, s_len, s_ppref, T, n_pieces, tab, lo + chunk_rows, s_cnt, mark);
-            // the next pass starts behind the rows of this one (the walk ended with a barrier, or saw nothing)
-            uint32_t pieces = 0;
-            if (tid < T) {
-                const int c = s_cnt[tid];
-                s_start[tid] += c;
-                s_len[tid] -= c;
-                pieces = (static_cast<uint32_t>(s_len[tid]) + 63u) >> 6;
-            }
-            const uint32_t ex = block_exclusive_sum(pieces, scratch, &n_pieces);
-            if (tid < T) s_ppref[tid] = ex;
-            if (tid == 0) s_ppref[T] = n_pieces;
-        } else {
-            walk_candidates<false>(a.cand, s_start, s_len, s_ppref, T, n_pieces, tab, 0u, nullptr, mark);
-        }
+        walk_candidates(a.cand, s_start, s_len, s_ppref, T, n_pieces, tab, mark);
         DD_TICK(1)  // gather
         if (MODE == DD_COUNT) {
             // a row is counted by whichever lane set its bit first
@@ -564,17 +592,22 @@ struct DedupGeometry {
 culsh_status dedup_geometry(const culsh_ctx* ctx, const culsh_index* index, DedupGeometry* g) {
     const int T = index->n_hash_tables;
     const int n = index->n_total_candidates / T;  // candidates are row ids < n
-    const size_t fixed = (4 + static_cast<size_t>(4 * T) + 1 + 2 * DD_THREADS + 17 + (NWAVES + 1) + 8) * sizeof(uint32_t);
-    auto lds_need = [&](int w) { return static_cast<size_t>(DD_THREADS) * w * 4 + fixed; };
-    int wpt_max = 1;
     const int wpt_limit = std::max(1, std::min(32, env_int("CULSH_DEDUP_WPT", 32)));
-    while (wpt_max * 2 <= wpt_limit && lds_need(wpt_max * 2) <= static_cast<size_t>(ctx->lds_max)) wpt_max *= 2;
-    int wpt = 1;
-    while (wpt < wpt_max && static_cast<long long>(DD_THREADS) * wpt * 32 < n) wpt *= 2;
-    const long long chunk_rows = static_cast<long long>(DD_THREADS) * wpt * 32;
-    g->wpt = wpt;
-    g->n_chunks = static_cast<int>((n + chunk_rows - 1) / chunk_rows);
-    g->lds_bytes = lds_need(wpt);
+    // beside the bitmap: 3T + 1 words of spans for one pass, 2T + SPLIT_BATCH * T more when a query takes several
+    for (int several = 0; several < 2; ++several) {
+        const size_t per_table = several ? 5 + SPLIT_BATCH : 3;
+        const size_t fixed = (4 + per_table * T + 1 + 2 * DD_THREADS + 17 + (NWAVES + 1) + 8) * sizeof(uint32_t);
+        auto lds_need = [&](int w) { return static_cast<size_t>(DD_THREADS) * w * 4 + fixed; };
+        int wpt_max = 1;
+        while (wpt_max * 2 <= wpt_limit && lds_need(wpt_max * 2) <= static_cast<size_t>(ctx->lds_max)) wpt_max *= 2;
+        int wpt = 1;
+        while (wpt < wpt_max && static_cast<long long>(DD_THREADS) * wpt * 32 < n) wpt *= 2;
+        const long long chunk_rows = static_cast<long long>(DD_THREADS) * wpt * 32;
+        g->wpt = wpt;
+        g->n_chunks = static_cast<int>((n + chunk_rows - 1) / chunk_rows);
+        g->lds_bytes = lds_need(wpt);
+        if (g->n_chunks == 1) break;
+    }
     CULSH_REQUIRE(g->lds_bytes <= static_cast<size_t>(ctx->lds_max), CULSH_ERR_INTERNAL, "LDS budget exceeded");
     return CULSH_OK;
 }
