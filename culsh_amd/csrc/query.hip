@@ -411,8 +411,11 @@ __global__ __launch_bounds__(DD_THREADS) void dedup_kernel(DedupArgs a) {
         const int ew = wpw >= 512 ? 8 : (wpw >= 256 ? 4 : 1);   // words per lane and step
         const int steps = wpw / (64 * ew);
         uint32_t* wbm = bm + wave * wpw;
+        // How many rows each wavefront holds.  One pass per query: counted first, so that the query's
+        // count is published before the line-up.  Several passes: nobody waits for the count, and the
+        // line-up's own totals serve.
         uint32_t wave_total = 0;
-        for (int j = 0; j < steps; ++j) {
+        for (int j = 0; !several && j < steps; ++j) {
             const uint32_t* p = wbm + (j * 64 + lane) * ew;
             if (ew == 8) {
                 const uint4 v0 = *reinterpret_cast<const uint4*>(p), v1 = *reinterpret_cast<const uint4*>(p + 4);
@@ -425,15 +428,17 @@ __global__ __launch_bounds__(DD_THREADS) void dedup_kernel(DedupArgs a) {
                 wave_total += __popc(p[0]);
             }
         }
-        wave_total = wave_sum(wave_total);
-        if (lane == 0) wtot[wave] = wave_total;
-        __syncthreads();
         uint32_t wave_base = 0, chunk_total = 0;
+        if (!several) {
+            wave_total = wave_sum(wave_total);
+            if (lane == 0) wtot[wave] = wave_total;
+            __syncthreads();
 #pragma unroll
-        for (int w = 0; w < NWAVES; ++w) {
-            const uint32_t v = wtot[w];
-            wave_base += (w < wave) ? v : 0u;
-            chunk_total += v;
+            for (int w = 0; w < NWAVES; ++w) {
+                const uint32_t v = wtot[w];
+                wave_base += (w < wave) ? v : 0u;
+                chunk_total += v;
+            }
         }
         // FUSED: the first wavefront publishes the count before anything else, so that later
         // queries can go on, and looks back only after lining up its own rows.
@@ -479,26 +484,45 @@ __global__ __launch_bounds__(DD_THREADS) void dedup_kernel(DedupArgs a) {
         DD_TICK(5)
         uint64_t base = out_base + running;
         bool store = true;
-        if (FUSED) {
+        if (several) {
+            if (lane == 0) wtot[wave] = st_total[0] + st_total[1] + st_total[2] + st_total[3];
+            if (last && wave == 0) {
+                const int qn = min(static_cast<int>(__shfl(ticket_next, 0, 64)), a.n_queries);
+                if (T <= 64 && qn < a.n_queries && lane < T) sp_next = a.spans[static_cast<size_t>(qn) * T + lane];
+                if (lane == 0) *sh_q = qn;
+            }
+            DD_TICK(6)
+            __syncthreads();
+#pragma unroll
+            for (int w = 0; w < NWAVES; ++w) {
+                const uint32_t v = wtot[w];
+                wave_base += (w < wave) ? v : 0u;
+                chunk_total += v;
+            }
+            base = raw_base + running;
+            store = base + chunk_total <= a.capacity;  // cannot fail with capacity = raw candidates
+            if (tid == 0) {
+                if (!store) atomicOr(a.err, 2u);
+                if (last) a.counts[q] = running + chunk_total;
+            }
+            if (last) q_next = *sh_q;
+        } else if (FUSED) {
             if (wave == 0) {
                 const int qn = min(static_cast<int>(__shfl(ticket_next, 0, 64)), a.n_queries);
                 // spans of the next query (they all sit in this wavefront when T <= 64)
-                if (last && T <= 64 && qn < a.n_queries && lane < T) sp_next = a.spans[static_cast<size_t>(qn) * T + lane];
-                const unsigned long long excl =
-                    several ? raw_base + running : look_back(a.state, q, chunk_total, a.spin_limit, a.err);
+                if (T <= 64 && qn < a.n_queries && lane < T) sp_next = a.spans[static_cast<size_t>(qn) * T + lane];
+                const unsigned long long excl = look_back(a.state, q, chunk_total, a.spin_limit, a.err);
                 if (lane == 0) {
-                    if (last) *sh_q = qn;
+                    *sh_q = qn;
                     unsigned long long b = excl;
                     if (excl + chunk_total > a.capacity) {  // cannot happen with capacity = raw candidates
                         atomicOr(a.err, 2u);
                         b = ~0ull;
                     }
                     *sh_base = b;
-                    if (last) a.counts[q] = running + chunk_total;
-                    if (!several) {
-                        a.offsets[q] = excl;
-                        if (q == a.n_queries - 1) a.offsets[a.n_queries] = excl + chunk_total;
-                    }
+                    a.counts[q] = running + chunk_total;
+                    a.offsets[q] = excl;
+                    if (q == a.n_queries - 1) a.offsets[a.n_queries] = excl + chunk_total;
                 }
             }
             DD_TICK(6)
