@@ -257,9 +257,9 @@ def test_core_query_wide_row_range(ctx, c_oracle, n):
 @pytest.mark.parametrize("two_pass", [False, True])
 def test_core_query_many_bitmap_passes(ctx, monkeypatch, two_pass):
     """A small bitmap (32768 rows per pass) makes a 150k-row index take five passes per query: in the
-    single launch every (query, pass) is a unit of the chained scan and spans shrink from pass to
-    pass; passes without any row and queries without candidates are among them.  Also through the
-    count / scan / emit launches."""
+    single launch every span is cut at the passes' row bounds and the lists are written at raw-count
+    spacing, then moved together; passes without any row and queries without candidates are among
+    them.  Also through the count / scan / emit launches."""
     _announce("many_bitmap_passes", two_pass)
     monkeypatch.setenv("CULSH_DEDUP_WPT", "1")
     if two_pass:
@@ -275,6 +275,29 @@ def test_core_query_many_bitmap_passes(ctx, monkeypatch, two_pass):
     from abi import assert_candidates_match
 
     assert_candidates_match(ctx.core_query_index(qsig, ih), o.query_index(qsig, o.fit_index(sig, H)))
+    ctx.free_index(ih)
+
+
+def test_core_query_bitmap_passes_long_spans_many_tables(ctx, c_oracle, monkeypatch):
+    """Several passes per query with 100 tables (more span cuts than one search round holds, spans
+    reloaded per query) and buckets of ~30k rows (every span crosses every row bound, the search
+    takes seven rounds), next to buckets of one row and buckets that end exactly at a bound."""
+    _announce("bitmap_passes_long_spans_many_tables")
+    monkeypatch.setenv("CULSH_DEDUP_WPT", "1")
+    rng = np.random.default_rng(78)
+    T, n, nq, H = 100, 120_000, 24, 1
+    sig = rng.integers(0, 4, size=(T, n, H)).astype(np.uint8)
+    sig[:50, :32768, 0] = 9                     # a bucket that is exactly the first pass
+    sig[50:, 32768:65536 + 1, 0] = 9            # one that overshoots the second pass by a row
+    sig[:, 100_000, 0] = 77                     # single-row buckets in the last pass
+    qsig = rng.integers(0, 4, size=(T, nq, H)).astype(np.uint8)
+    qsig[:, 3::4, 0] = 9
+    qsig[:, 5, 0] = 77
+    qsig[:, 6, 0] = 200                         # no candidates
+    ih, _ = ctx.core_fit_index(sig, H)
+    from abi import assert_candidates_match
+
+    assert_candidates_match(ctx.core_query_index(qsig, ih), c_oracle.query_index_c(qsig, c_oracle.fit_index_c(sig, H)))
     ctx.free_index(ih)
 
 
