@@ -375,6 +375,7 @@ __global__ __launch_bounds__(DD_THREADS) void dedup_kernel(DedupArgs a) {
             const uint32_t ex = block_exclusive_sum(pieces, scratch, &n_pieces);
             if (tid < T) s_ppref[tid] = ex;
             if (tid == 0) s_ppref[T] = n_pieces;
+            if (n_pieces == 0 && !last) continue;  // no row in this range; the bitmap is clean
         }
         if (tid <= NWAVES) wtot[tid] = 0;
         __syncthreads();
