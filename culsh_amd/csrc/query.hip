@@ -291,7 +291,7 @@ __global__ __launch_bounds__(DD_THREADS) void dedup_kernel(DedupArgs a) {
     uint32_t* s_ppref = reinterpret_cast<uint32_t*>(s_len + T);  // [T+1]
     uint32_t* scratch = s_ppref + T + 1;                         // [17]
     uint32_t* wtot = scratch + 17;                               // [NWAVES + 1]
-    // FUSED with several passes: the query's spans as given, and where the next row bounds cut them
+    // several passes per query: the query's spans as given, and where the next row bounds cut them
     int* s_org_start = reinterpret_cast<int*>(wtot + NWAVES + 1);  // [T]
     int* s_org_len = s_org_start + T;                              // [T]
     int* s_split = s_org_len + T;                                  // [SPLIT_BATCH][T]
@@ -328,9 +328,10 @@ __global__ __launch_bounds__(DD_THREADS) void dedup_kernel(DedupArgs a) {
     // on other queries, the host closes the gaps afterwards), and every pass walks the part of each
     // span whose rows fall into its range; split_spans finds those parts, a few passes ahead.
     constexpr bool several = MODE == DD_FUSED_PASSES;
+    const bool cut = MODE != DD_FUSED && a.n_chunks > 1;  // several passes, in one launch or two
     uint32_t n_pieces = 0;
     int covered = 0;  // several passes: rows of span `tid` that earlier passes walked
-    if (several) {
+    if (cut) {
         if (tid < T) {
             s_org_start[tid] = sp.x;
             s_org_len[tid] = sp.y;
@@ -356,7 +357,7 @@ __global__ __launch_bounds__(DD_THREADS) void dedup_kernel(DedupArgs a) {
             uint4* bm4 = reinterpret_cast<uint4*>(bm);
             for (int i = tid; i < chunk_words / 4; i += DD_THREADS) bm4[i] = make_uint4(0u, 0u, 0u, 0u);
         }
-        if (several) {
+        if (cut) {
             const int ahead = chunk % SPLIT_BATCH;
             if (ahead == 0 && !last) {
                 __syncthreads();  // the spans are in place, the previous bounds are used up
@@ -375,7 +376,7 @@ __global__ __launch_bounds__(DD_THREADS) void dedup_kernel(DedupArgs a) {
             const uint32_t ex = block_exclusive_sum(pieces, scratch, &n_pieces);
             if (tid < T) s_ppref[tid] = ex;
             if (tid == 0) s_ppref[T] = n_pieces;
-            if (n_pieces == 0 && !last) continue;  // no row in this range; the bitmap is clean
+            if (several && n_pieces == 0 && !last) continue;  // no row in this range; the bitmap is clean
         }
         if (tid <= NWAVES) wtot[tid] = 0;
         __syncthreads();
