@@ -134,7 +134,7 @@ template <typename F>
 __device__ __forceinline__ void walk_candidates(const int32_t* __restrict__ cand, const int* s_start,
                                                 const int* s_len, const uint32_t* s_ppref, int T,
                                                 uint32_t n_pieces, int2* tab, F&& f) {
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // the same in every lane: kept in a scalar register
     for (uint32_t r0 = 0; r0 < n_pieces; r0 += DD_THREADS) {
         const uint32_t pc = r0 + static_cast<uint32_t>(tid);
         if (pc < n_pieces) {
@@ -280,7 +280,7 @@ template <int MODE>
 __global__ __launch_bounds__(DD_THREADS) void dedup_kernel(DedupArgs a) {
     constexpr bool FUSED = MODE == DD_FUSED || MODE == DD_FUSED_PASSES;
     extern __shared__ uint32_t lds[];
-    const int T = a.T, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int T = a.T, tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int chunk_words = DD_THREADS * a.wpt;                  // multiple of 1024
     uint32_t* bm = lds;                                          // [chunk_words]
     unsigned long long* sh_base = reinterpret_cast<unsigned long long*>(bm + chunk_words);  // [1]
@@ -441,6 +441,9 @@ __global__ __launch_bounds__(DD_THREADS) void dedup_kernel(DedupArgs a) {
                 wave_base += (w < wave) ? v : 0u;
                 chunk_total += v;
             }
+            // the same in every lane: summed here and kept in scalar registers, not as 16 values until their use
+            wave_base = __builtin_amdgcn_readfirstlane(wave_base);
+            chunk_total = __builtin_amdgcn_readfirstlane(chunk_total);
         }
         // FUSED: the first wavefront publishes the count before anything else, so that later
         // queries can go on, and looks back only after lining up its own rows.
@@ -501,6 +504,9 @@ __global__ __launch_bounds__(DD_THREADS) void dedup_kernel(DedupArgs a) {
                 wave_base += (w < wave) ? v : 0u;
                 chunk_total += v;
             }
+            // the same in every lane: summed here and kept in scalar registers, not as 16 values until their use
+            wave_base = __builtin_amdgcn_readfirstlane(wave_base);
+            chunk_total = __builtin_amdgcn_readfirstlane(chunk_total);
             base = raw_base + running;
             store = base + chunk_total <= a.capacity;  // cannot fail with capacity = raw candidates
             if (tid == 0) {
