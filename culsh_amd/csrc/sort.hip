@@ -238,7 +238,7 @@ __global__ __launch_bounds__(THREADS) void radix_scatter_kernel(
     int32_t* st_row = reinterpret_cast<int32_t*>(st_key + TILE * (TWO_WORDS ? 2 : 1));  // [TILE] when staged
     const int tile = CHAINED ? static_cast<int>(blockIdx.x / T) : static_cast<int>(blockIdx.x);
     const int t = CHAINED ? static_cast<int>(blockIdx.x - static_cast<unsigned>(tile) * T) : static_cast<int>(blockIdx.y);
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // the same in every lane: scalar
     for (int i = tid; i < NW * 256; i += THREADS) (&whist[0][0])[i] = 0;
     __syncthreads();
 
