@@ -473,14 +473,14 @@ __global__ __launch_bounds__(DD_THREADS) void dedup_kernel(DedupArgs a) {
             const uint32_t incl = wave_inclusive_sum_dpp(c);
             st_total[j] = __shfl(incl, 63, 64);
             if (st_total[j] <= region) {
-                uint32_t pos = incl - c;
+                uint32_t* slot = sreg + (incl - c);  // runs on from word to word
                 const uint32_t row_base = lo + (static_cast<uint32_t>(wave * wpw + w0) << 5);
 #pragma unroll
                 for (int k = 0; k < 8; ++k) {
                     uint32_t bits = words[k];
                     const uint32_t r0 = row_base + (k << 5);
                     while (bits) {
-                        sreg[pos++] = r0 + (__ffs(static_cast<int>(bits)) - 1);
+                        *slot++ = r0 + (__ffs(static_cast<int>(bits)) - 1);
                         bits &= bits - 1u;
                     }
                 }
