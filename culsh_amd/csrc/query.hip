@@ -255,18 +255,26 @@ __device__ __forceinline__ unsigned long long look_back(unsigned long long* stat
     return excl;
 }
 
-// The `ew` (8, 4 or 1) consecutive bitmap words a lane owns in one read-out step.  The words are
-// merged from the three cases as two vector values and only then spread into the array: filling
-// the array inside the branches makes the compiler keep it in scratch memory.
-__device__ __forceinline__ void load_step_words(const uint32_t* p, int ew, uint32_t (&words)[8]) {
+// Where bitmap word `w` sits in LDS.  With eight words per lane and step, a lane's words 0-3 and 4-7
+// are stored 256 words apart, so that each of the two 16-byte reads of a step is contiguous over the
+// lanes (a lane stride of 32 bytes makes every such read hit each bank twice).  Inside a step region
+// of 512 words the index bits (lane:6, half:1, word:2) become (half:1, lane:6, word:2).
+__device__ __forceinline__ uint32_t bitmap_slot(uint32_t w, bool eight) {
+    return eight ? ((w & ~0x1FFu) | ((w & 4u) << 6) | ((w & 0x1F8u) >> 1) | (w & 3u)) : w;
+}
+
+// The `ew` (8, 4 or 1) consecutive bitmap words a lane owns in one read-out step, whose region starts
+// at `region`.  The words are merged from the three cases as two vector values and only then spread
+// into the array: filling the array inside the branches makes the compiler keep it in scratch memory.
+__device__ __forceinline__ void load_step_words(const uint32_t* region, int lane, int ew, uint32_t (&words)[8]) {
     uint4 v0 = make_uint4(0u, 0u, 0u, 0u), v1 = make_uint4(0u, 0u, 0u, 0u);
     if (ew == 8) {
-        v0 = *reinterpret_cast<const uint4*>(p);
-        v1 = *reinterpret_cast<const uint4*>(p + 4);
+        v0 = *reinterpret_cast<const uint4*>(region + lane * 4);
+        v1 = *reinterpret_cast<const uint4*>(region + 256 + lane * 4);
     } else if (ew == 4) {
-        v0 = *reinterpret_cast<const uint4*>(p);
+        v0 = *reinterpret_cast<const uint4*>(region + lane * 4);
     } else {
-        v0.x = p[0];
+        v0.x = region[lane];
     }
     words[0] = v0.x; words[1] = v0.y; words[2] = v0.z; words[3] = v0.w;
     words[4] = v1.x; words[5] = v1.y; words[6] = v1.z; words[7] = v1.w;
@@ -348,6 +356,9 @@ __global__ __launch_bounds__(DD_THREADS) void dedup_kernel(DedupArgs a) {
     uint64_t running = 0;  // unique candidates found in earlier passes
     const uint64_t out_base = MODE == DD_EMIT ? a.offsets[q] : 0;
     const uint32_t chunk_rows = static_cast<uint32_t>(chunk_words) * 32u;
+    const int wpw = chunk_words / NWAVES;                  // bitmap words per wavefront in the read-out, >= 64
+    const int ew = wpw >= 512 ? 8 : (wpw >= 256 ? 4 : 1);  // words per lane and read-out step
+    const bool eight = ew == 8;
 
     const unsigned long long raw_base = several ? a.raw_offsets[q] : 0ull;
     for (int chunk = 0; chunk < a.n_chunks; ++chunk) {
@@ -387,11 +398,11 @@ __global__ __launch_bounds__(DD_THREADS) void dedup_kernel(DedupArgs a) {
         auto mark = [&](int row) {
             const uint32_t bit = static_cast<uint32_t>(row) - lo;
             if (bit < chunk_rows) {
-                const uint32_t m = 1u << (bit & 31u);
+                const uint32_t m = 1u << (bit & 31u), slot = bitmap_slot(bit >> 5, eight);
                 if (MODE == DD_COUNT) {
-                    fresh += (atomicOr(&bm[bit >> 5], m) & m) == 0u;
+                    fresh += (atomicOr(&bm[slot], m) & m) == 0u;
                 } else {
-                    atomicOr(&bm[bit >> 5], m);
+                    atomicOr(&bm[slot], m);
                 }
             }
         };
@@ -409,26 +420,15 @@ __global__ __launch_bounds__(DD_THREADS) void dedup_kernel(DedupArgs a) {
         }
         // Ordered read-out.  Wavefront w owns the consecutive words [w*wpw, (w+1)*wpw); in a step
         // every lane takes EW consecutive words, so row order = (wave, step, lane, word, bit).
-        const int wpw = chunk_words / NWAVES;                 // words per wavefront, >= 64
-        const int ew = wpw >= 512 ? 8 : (wpw >= 256 ? 4 : 1);   // words per lane and step
         const int steps = wpw / (64 * ew);
         uint32_t* wbm = bm + wave * wpw;
         // How many rows each wavefront holds.  One pass per query: counted first, so that the query's
         // count is published before the line-up.  Several passes: nobody waits for the count, and the
         // line-up's own totals serve.
         uint32_t wave_total = 0;
-        for (int j = 0; !several && j < steps; ++j) {
-            const uint32_t* p = wbm + (j * 64 + lane) * ew;
-            if (ew == 8) {
-                const uint4 v0 = *reinterpret_cast<const uint4*>(p), v1 = *reinterpret_cast<const uint4*>(p + 4);
-                wave_total += __popc(v0.x) + __popc(v0.y) + __popc(v0.z) + __popc(v0.w) + __popc(v1.x) +
-                              __popc(v1.y) + __popc(v1.z) + __popc(v1.w);
-            } else if (ew == 4) {
-                const uint4 v0 = *reinterpret_cast<const uint4*>(p);
-                wave_total += __popc(v0.x) + __popc(v0.y) + __popc(v0.z) + __popc(v0.w);
-            } else {
-                wave_total += __popc(p[0]);
-            }
+        for (int i = lane; !several && i < wpw / 4; i += 64) {  // in any order: contiguous reads
+            const uint4 v = reinterpret_cast<const uint4*>(wbm)[i];
+            wave_total += __popc(v.x) + __popc(v.y) + __popc(v.z) + __popc(v.w);
         }
         uint32_t wave_base = 0, chunk_total = 0;
         if (!several) {
@@ -466,7 +466,7 @@ __global__ __launch_bounds__(DD_THREADS) void dedup_kernel(DedupArgs a) {
             const int w0 = (j * 64 + lane) * ew;
             uint32_t* sreg = wbm + j * region;
             uint32_t words[8];
-            load_step_words(wbm + w0, ew, words);
+            load_step_words(sreg, lane, ew, words);
             uint32_t c = 0;
 #pragma unroll
             for (int k = 0; k < 8; ++k) c += __popc(words[k]);
@@ -552,7 +552,7 @@ __global__ __launch_bounds__(DD_THREADS) void dedup_kernel(DedupArgs a) {
                 } else {  // dense step: every lane stores the rows of its own words
                     const int w0 = (j * 64 + lane) * ew;
                     uint32_t words[8];
-                    load_step_words(wbm + w0, ew, words);
+                    load_step_words(sreg, lane, ew, words);
                     uint32_t c = 0;
 #pragma unroll
                     for (int k = 0; k < 8; ++k) c += __popc(words[k]);
