@@ -255,12 +255,12 @@ __device__ __forceinline__ unsigned long long look_back(unsigned long long* stat
     return excl;
 }
 
-// Where bitmap word `w` sits in LDS.  With eight words per lane and step, a lane's words 0-3 and 4-7
-// are stored 256 words apart, so that each of the two 16-byte reads of a step is contiguous over the
-// lanes (a lane stride of 32 bytes makes every such read hit each bank twice).  Inside a step region
-// of 512 words the index bits (lane:6, half:1, word:2) become (half:1, lane:6, word:2).
-__device__ __forceinline__ uint32_t bitmap_slot(uint32_t w, bool eight) {
-    return eight ? ((w & ~0x1FFu) | ((w & 4u) << 6) | ((w & 0x1F8u) >> 1) | (w & 3u)) : w;
+// Where bitmap word `w` sits in LDS.  With eight words per lane and step a lane reads two 16-byte
+// halves at a lane stride of 32 bytes, and sixteen neighbouring lanes would hit every bank twice per
+// read.  Lanes 8-15 of every sixteen keep their two halves in swapped places (index bit 2 = the half,
+// bit 6 = lane bit 3), so that the sixteen reads cover sixteen different 16-byte columns.
+__device__ __forceinline__ uint32_t bitmap_slot(uint32_t w, uint32_t swap_mask) {  // swap_mask: 4 for eight words per lane, else 0
+    return w ^ ((w >> 4) & swap_mask);
 }
 
 // The `ew` (8, 4 or 1) consecutive bitmap words a lane owns in one read-out step, whose region starts
@@ -269,8 +269,9 @@ __device__ __forceinline__ uint32_t bitmap_slot(uint32_t w, bool eight) {
 __device__ __forceinline__ void load_step_words(const uint32_t* region, int lane, int ew, uint32_t (&words)[8]) {
     uint4 v0 = make_uint4(0u, 0u, 0u, 0u), v1 = make_uint4(0u, 0u, 0u, 0u);
     if (ew == 8) {
-        v0 = *reinterpret_cast<const uint4*>(region + lane * 4);
-        v1 = *reinterpret_cast<const uint4*>(region + 256 + lane * 4);
+        const int swap = (lane >> 1) & 4;  // bitmap_slot of this lane's words
+        v0 = *reinterpret_cast<const uint4*>(region + ((lane * 8) ^ swap));
+        v1 = *reinterpret_cast<const uint4*>(region + ((lane * 8 + 4) ^ swap));
     } else if (ew == 4) {
         v0 = *reinterpret_cast<const uint4*>(region + lane * 4);
     } else {
@@ -358,7 +359,7 @@ __global__ __launch_bounds__(DD_THREADS) void dedup_kernel(DedupArgs a) {
     const uint32_t chunk_rows = static_cast<uint32_t>(chunk_words) * 32u;
     const int wpw = chunk_words / NWAVES;                  // bitmap words per wavefront in the read-out, >= 64
     const int ew = wpw >= 512 ? 8 : (wpw >= 256 ? 4 : 1);  // words per lane and read-out step
-    const bool eight = ew == 8;
+    const uint32_t swap_mask = ew == 8 ? 4u : 0u;
 
     const unsigned long long raw_base = several ? a.raw_offsets[q] : 0ull;
     for (int chunk = 0; chunk < a.n_chunks; ++chunk) {
@@ -398,7 +399,7 @@ __global__ __launch_bounds__(DD_THREADS) void dedup_kernel(DedupArgs a) {
         auto mark = [&](int row) {
             const uint32_t bit = static_cast<uint32_t>(row) - lo;
             if (bit < chunk_rows) {
-                const uint32_t m = 1u << (bit & 31u), slot = bitmap_slot(bit >> 5, eight);
+                const uint32_t m = 1u << (bit & 31u), slot = bitmap_slot(bit >> 5, swap_mask);
                 if (MODE == DD_COUNT) {
                     fresh += (atomicOr(&bm[slot], m) & m) == 0u;
                 } else {
