@@ -129,7 +129,8 @@ constexpr int WALK_U = 16;  // pieces in flight per wavefront
 // the wavefronts, and a wavefront reads a piece with one load per lane.  Where piece p
 // starts is looked up once per piece (one binary search per thread over the spans'
 // piece counts, all pieces of a round in parallel) and kept in `tab`, so the per-lane
-// work is an add, a compare and the load.  Contains barriers: all threads must call it.
+// work is an add, a compare and the load.  `f` is also called with -1, for the lanes beyond a
+// piece's end, and must ignore it.  Contains barriers: all threads must call it.
 template <typename F>
 __device__ __forceinline__ void walk_candidates(const int32_t* __restrict__ cand, const int* s_start,
                                                 const int* s_len, const uint32_t* s_ppref, int T,
@@ -161,8 +162,7 @@ __device__ __forceinline__ void walk_candidates(const int32_t* __restrict__ cand
                 if (pi < here && lane < ent[u].y) rows[u] = cand[ent[u].x + lane];
             }
 #pragma unroll
-            for (int u = 0; u < WALK_U; ++u)
-                if (rows[u] >= 0) f(rows[u]);
+            for (int u = 0; u < WALK_U; ++u) f(rows[u]);  // -1 where the lane has no row: f tells by its range check
         }
         __syncthreads();  // tab is rewritten by the next round
     }
@@ -398,7 +398,7 @@ __global__ __launch_bounds__(DD_THREADS) void dedup_kernel(DedupArgs a) {
         uint32_t fresh = 0;  // COUNT: bits this thread set first
         auto mark = [&](int row) {
             const uint32_t bit = static_cast<uint32_t>(row) - lo;
-            if (bit < chunk_rows) {
+            if (bit < chunk_rows) {  // also false for -1 (no row): lo + chunk_rows stays below 2^32
                 const uint32_t m = 1u << (bit & 31u), slot = bitmap_slot(bit >> 5, swap_mask);
                 if (MODE == DD_COUNT) {
                     fresh += (atomicOr(&bm[slot], m) & m) == 0u;
