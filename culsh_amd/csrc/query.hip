@@ -159,12 +159,32 @@ __device__ __forceinline__ void walk_candidates(const int32_t* __restrict__ cand
             for (int u = 0; u < WALK_U; ++u) {
                 const uint32_t pi = p0 + u * NWAVES;
                 rows[u] = -1;
-                if (pi < here && lane < ent[u].y) rows[u] = cand[ent[u].x + lane];
+                if (pi < here && lane < ent[u].y) rows[u] = cand[static_cast<uint32_t>(ent[u].x + lane)];  // unsigned: no sign extension per load
             }
 #pragma unroll
             for (int u = 0; u < WALK_U; ++u) f(rows[u]);  // -1 where the lane has no row: f tells by its range check
         }
         __syncthreads();  // tab is rewritten by the next round
+    }
+}
+
+// Piece numbering of the spans handed to walk_candidates: s_ppref[t] = pieces of the spans before t,
+// s_ppref[T] = all pieces.  `pieces` is the piece count of span threadIdx.x (0 beyond the T-th thread).
+// Up to 64 spans sit in the first wavefront, which then does it alone, without a barrier; all threads
+// must call it, and a barrier has to follow before s_ppref is read.
+__device__ __forceinline__ void number_pieces(uint32_t pieces, int T, uint32_t* s_ppref, uint32_t* scratch) {
+    const int tid = threadIdx.x;
+    if (T <= 64) {
+        if (tid < 64) {
+            const uint32_t incl = wave_inclusive_sum_dpp(pieces);
+            if (tid < T) s_ppref[tid] = incl - pieces;
+            if (tid == 63) s_ppref[T] = incl;
+        }
+    } else {
+        uint32_t total;
+        const uint32_t ex = block_exclusive_sum(pieces, scratch, &total);
+        if (tid < T) s_ppref[tid] = ex;
+        if (tid == 0) s_ppref[T] = total;
     }
 }
 
@@ -338,7 +358,7 @@ __global__ __launch_bounds__(DD_THREADS) void dedup_kernel(DedupArgs a) {
     // span whose rows fall into its range; split_spans finds those parts, a few passes ahead.
     constexpr bool several = MODE == DD_FUSED_PASSES;
     const bool cut = MODE != DD_FUSED && a.n_chunks > 1;  // several passes, in one launch or two
-    uint32_t n_pieces = 0;
+    uint32_t n_pieces;
     int covered = 0;  // several passes: rows of span `tid` that earlier passes walked
     if (cut) {
         if (tid < T) {
@@ -350,9 +370,7 @@ __global__ __launch_bounds__(DD_THREADS) void dedup_kernel(DedupArgs a) {
             s_start[tid] = sp.x;
             s_len[tid] = sp.y;
         }
-        const uint32_t ex = block_exclusive_sum((static_cast<uint32_t>(sp.y) + 63u) >> 6, scratch, &n_pieces);
-        if (tid < T) s_ppref[tid] = ex;
-        if (tid == 0) s_ppref[T] = n_pieces;
+        number_pieces((static_cast<uint32_t>(sp.y) + 63u) >> 6, T, s_ppref, scratch);
     }
     uint64_t running = 0;  // unique candidates found in earlier passes
     const uint64_t out_base = MODE == DD_EMIT ? a.offsets[q] : 0;
@@ -385,13 +403,15 @@ __global__ __launch_bounds__(DD_THREADS) void dedup_kernel(DedupArgs a) {
                 pieces = (static_cast<uint32_t>(end - covered) + 63u) >> 6;
                 covered = end;
             }
-            const uint32_t ex = block_exclusive_sum(pieces, scratch, &n_pieces);
-            if (tid < T) s_ppref[tid] = ex;
-            if (tid == 0) s_ppref[T] = n_pieces;
-            if (several && n_pieces == 0 && !last) continue;  // no row in this range; the bitmap is clean
+            number_pieces(pieces, T, s_ppref, scratch);
         }
         if (tid <= NWAVES) wtot[tid] = 0;
         __syncthreads();
+        n_pieces = s_ppref[T];
+        if (several && n_pieces == 0 && !last) {  // no row in this range; the bitmap is clean
+            __syncthreads();                      // s_ppref is rewritten by the next pass
+            continue;
+        }
         DD_TICK(0)  // setup + clear
         // Mark the rows of this pass (collect_candidates_kernel, core/query.cuh:199-237, but into
         // the bitmap instead of memory).  Rows outside [lo, lo + chunk_rows) belong to another pass.
