@@ -1137,6 +1137,22 @@ culsh_status culsh_index_load(culsh_ctx* ctx, culsh_kind kind, int is_double, co
     } else if (kind != CULSH_KIND_CORE) {
         CULSH_REQUIRE(S == 4 * H, CULSH_ERR_INVALID, "sig_nbytes must be 4 * n_hashes for this family");
     }
+    // The kernels trust these arrays (a span outside all_candidate_indices or a row id outside the
+    // bitmap's range would be a stray access on the device), so a file that does not add up is refused here.
+    CULSH_REQUIRE(n_total_candidates % T == 0, CULSH_ERR_INVALID, "n_total_candidates is not a multiple of n_hash_tables");
+    CULSH_REQUIRE(tbo[0] == 0 && tbo[T] == n_total_buckets, CULSH_ERR_INVALID, "table_bucket_offsets do not span the buckets");
+    for (int t = 0; t < T; ++t)
+        CULSH_REQUIRE(tbo[t] <= tbo[t + 1], CULSH_ERR_INVALID, "table_bucket_offsets must not decrease");
+    CULSH_REQUIRE(bco[0] == 0 && bco[n_total_buckets] == n_total_candidates, CULSH_ERR_INVALID,
+                  "bucket_candidate_offsets do not span the candidates");
+    for (int i = 0; i < n_total_buckets; ++i)
+        CULSH_REQUIRE(bco[i] <= bco[i + 1], CULSH_ERR_INVALID, "bucket_candidate_offsets must not decrease");
+    {
+        const uint32_t n_rows = static_cast<uint32_t>(n_total_candidates / T);
+        uint32_t beyond = 0;
+        for (int i = 0; i < n_total_candidates; ++i) beyond |= static_cast<uint32_t>(static_cast<uint32_t>(cand[i]) >= n_rows);
+        CULSH_REQUIRE(beyond == 0, CULSH_ERR_INVALID, "candidate index outside [0, n_total_candidates / n_hash_tables)");
+    }
     ArenaScope scope(ctx);
     CULSH_TRY(scope.begin_status);
     IndexPtr ix(new (std::nothrow) culsh_index());

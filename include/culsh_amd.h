@@ -187,7 +187,9 @@ culsh_status culsh_index_array_info(const culsh_index*, culsh_array which, uint6
 culsh_status culsh_index_copy_array(culsh_ctx*, const culsh_index*, culsh_array which, void* dst, uint64_t dst_bytes, int dst_is_device);
 /* Rebuilds an index from host arrays: load_rplsh_index / load_pslsh_index / load_minhash_index
  * (bindings.cu:407-476).  `param0_host`: projection (RPLSH, p-stable) or hash_a (MinHash);
- * `param1_host`: bias (p-stable) or hash_b (MinHash), NULL for RPLSH. */
+ * `param1_host`: bias (p-stable) or hash_b (MinHash), NULL for RPLSH.  Unlike the reference, arrays that
+ * do not add up (offsets that decrease or do not span the arrays, candidate indices outside
+ * [0, n_total_candidates / n_hash_tables)) are refused with CULSH_ERR_INVALID: the query kernels trust them. */
 culsh_status culsh_index_load(culsh_ctx*, culsh_kind kind, int is_double,
                               const int32_t* candidate_indices_host, const uint8_t* bucket_signatures_host,
                               const int32_t* bucket_candidate_offsets_host, const int32_t* table_bucket_offsets_host,

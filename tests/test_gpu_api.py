@@ -100,6 +100,40 @@ def test_rplsh_save_load(tmp_path, dtype, as_torch):
         "projection"])
 
 
+def test_load_refuses_arrays_that_do_not_add_up():
+    """Offsets that decrease or do not span their arrays, and candidate indices beyond the row count,
+    would send the query kernels outside the arrays; loading such an index is an error (the
+    reference loads it unchecked)."""
+    from culsh_amd import RPLSH
+    from culsh_amd._culsh_core import RPLSHIndex
+
+    X = dense(500, 32, np.float32)
+    ix = RPLSH(n_hash_tables=4, n_hashes=6, seed=3).fit(X).index
+    good = dict(candidate_indices=ix.get_candidate_indices(), bucket_signatures=ix.get_bucket_signatures(),
+                bucket_candidate_offsets=ix.get_bucket_candidate_offsets(),
+                table_bucket_offsets=ix.get_table_bucket_offsets(), projection=ix.get_projection_matrix(),
+                n_total_candidates=ix.n_total_candidates, n_total_buckets=ix.n_total_buckets,
+                n_hash_tables=ix.n_hash_tables, n_hashes=ix.n_hashes, sig_nbytes=ix.sig_nbytes,
+                n_features=ix.n_features, seed=ix.seed)
+    again = RPLSHIndex.load_float(**good)
+    np.testing.assert_array_equal(again.get_candidate_indices(), good["candidate_indices"])
+
+    def broken(name, change):
+        bad = dict(good)
+        arr = good[name].copy()
+        change(arr)
+        bad[name] = arr
+        with pytest.raises(RuntimeError):
+            RPLSHIndex.load_float(**bad)
+
+    broken("candidate_indices", lambda a: a.__setitem__(7, 500))          # one past the last row
+    broken("candidate_indices", lambda a: a.__setitem__(0, -1))
+    broken("bucket_candidate_offsets", lambda a: a.__setitem__(3, a[4] + 1))   # decreases afterwards
+    broken("bucket_candidate_offsets", lambda a: a.__setitem__(-1, a[-1] + 5))  # beyond the candidates
+    broken("table_bucket_offsets", lambda a: a.__setitem__(2, a[1] - 1))
+    broken("table_bucket_offsets", lambda a: a.__setitem__(0, 1))
+
+
 @pytest.mark.parametrize("dtype", [np.float32, np.float64])
 def test_rplsh_fit_query_equals_fit_then_query(dtype):
     """python/tests/test_rplsh.py:145-174"""
