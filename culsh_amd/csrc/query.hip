@@ -76,7 +76,7 @@ __global__ __launch_bounds__(256) void lookup_kernel(const uint32_t* __restrict_
 // Span of every matched bucket (count_candidates_kernel, core/query.cuh:114-132).
 __global__ __launch_bounds__(256) void span_kernel(const int32_t* __restrict__ matched,
                                                   const int32_t* __restrict__ bucket_candidate_offsets,
-                                                  size_t pairs, int2* __restrict__ spans,
+                                                  size_t pairs, int n_buckets, int2* __restrict__ spans,
                                                   unsigned long long* __restrict__ raw_total) {
     __shared__ unsigned long long block_raw;
     if (threadIdx.x == 0) block_raw = 0ull;
@@ -85,7 +85,7 @@ __global__ __launch_bounds__(256) void span_kernel(const int32_t* __restrict__ m
     int2 sp = make_int2(0, 0);
     if (idx < pairs) {
         const int b = matched[idx];
-        if (b >= 0) {
+        if (b >= 0 && b < n_buckets) {  // -1 = no bucket; an id beyond the buckets is taken the same way
             sp.x = bucket_candidate_offsets[b];
             sp.y = bucket_candidate_offsets[b + 1] - sp.x;
         }
@@ -859,7 +859,7 @@ culsh_status query_from_matched(culsh_ctx* ctx, const int32_t* matched, int n_qu
     CULSH_TRY(dedup_geometry(ctx, index, &g));
     CULSH_TRY(alloc_query_words(ctx, n_queries, g, &raw_total));
     CULSH_LAUNCH(ctx, span_kernel, dim3(div_up(pairs, 256)), dim3(256), 0, ctx->stream, matched,
-                 index->bucket_candidate_offsets, pairs, spans, raw_total);
+                 index->bucket_candidate_offsets, pairs, index->n_total_buckets, spans, raw_total);
     CULSH_LAUNCH_CHECK();
     return query_from_spans(ctx, spans, raw_total, n_queries, index, g, out);
 }

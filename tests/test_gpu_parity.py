@@ -234,6 +234,11 @@ def test_core_query_from_matched_with_misses(ctx):
 
     assert_candidates_match(ctx.core_query_from_matched(matched, nq, ih),
                             o.query_from_matched_buckets(matched, nq, exp_ix))
+    # ids beyond the buckets are not followed: same result as with -1 in their place
+    beyond = matched.copy()
+    beyond[matched < 0] = exp_ix.n_total_buckets + np.arange(int((matched < 0).sum()), dtype=np.int32) * 1000
+    assert_candidates_match(ctx.core_query_from_matched(beyond, nq, ih),
+                            o.query_from_matched_buckets(matched, nq, exp_ix))
     ctx.free_index(ih)
 
 
