@@ -233,6 +233,7 @@ void free_index_arrays(culsh_index* ix) {
     dev_free(ix->bucket_candidate_offsets);
     dev_free(ix->table_bucket_offsets);
     dev_free(ix->bucket_keys);
+    dev_free(ix->key_dir);
     dev_free(ix->P);
     dev_free(ix->b);
     dev_free(ix->A);
@@ -244,6 +245,7 @@ void free_index_arrays(culsh_index* ix) {
     ix->bucket_candidate_offsets = nullptr;
     ix->table_bucket_offsets = nullptr;
     ix->bucket_keys = nullptr;
+    ix->key_dir = nullptr;
     ix->P = ix->b = nullptr;
     ix->A = ix->B = nullptr;
 }
@@ -1204,6 +1206,7 @@ culsh_status culsh_index_load(culsh_ctx* ctx, culsh_kind kind, int is_double, co
     }
     CULSH_HIP(dev_malloc(&ix->bucket_keys, std::max<size_t>(1, static_cast<size_t>(n_total_buckets) * ix->key_w) * 4));
     CULSH_TRY(launch_sig_to_keys(ctx, ix->all_bucket_signatures, n_total_buckets, S, enc, ix->key_w, ix->bucket_keys));
+    CULSH_TRY(build_key_directory(ctx, ix.get()));
     CULSH_TRY(arena_end(ctx));
     *out = ix.release();
     return CULSH_OK;

@@ -135,6 +135,7 @@ struct culsh_index {
     uint64_t seed = 0;
     // sort-order form of the bucket signatures: uint32 [n_total_buckets][key_w]
     uint32_t* bucket_keys = nullptr;
+    uint32_t* key_dir = nullptr;  // directory over the keys' leading bits (build_key_directory), or null
     culsh_amd::KeyEnc enc = culsh_amd::ENC_BE;
     int key_w = 0;
     culsh_amd::PsCodec psc;  // enc == ENC_PSC only
@@ -304,6 +305,13 @@ culsh_status fit_index_from_keys(culsh_ctx* ctx, uint32_t* keys, int n, int T, i
 // `matched` ([n_queries][T] bucket ids, -1 = none) and `spans` ([n_queries][T] int2 (start,
 // length) into all_candidate_indices) are both optional outputs; with `spans` the sum of
 // the span lengths is added to *raw_total (device).
+// Directory in front of the bucket lookup's binary search: for every table and every value of the
+// KEY_DIR_BITS leading bits of a key's first word (counted from the highest bit any bucket key has
+// set), where the buckets with that value start.  Layout: [0] = largest first word of any bucket key,
+// then per table KEY_DIR_SIZE + 1 bucket numbers.  Not built for more than KEY_DIR_MAX_TABLES tables.
+constexpr int KEY_DIR_BITS = 12, KEY_DIR_SIZE = 1 << KEY_DIR_BITS, KEY_DIR_MAX_TABLES = 1024;
+culsh_status build_key_directory(culsh_ctx* ctx, culsh_index* index);
+
 culsh_status launch_find_matching_buckets(culsh_ctx* ctx, const uint32_t* q_keys, int n_queries,
                                           const culsh_index* index, int32_t* matched, void* spans = nullptr,
                                           unsigned long long* raw_total = nullptr);

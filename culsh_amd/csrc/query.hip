@@ -31,10 +31,50 @@ namespace {
 
 constexpr int DD_THREADS = 1024;
 
-// Binary search of every (query, table) key among the table's sorted bucket keys; writes
+// Bits to drop from a key's first word to get its directory entry: the entry is made of the
+// KEY_DIR_BITS bits from the highest bit that the largest first word has set.
+__device__ __forceinline__ int key_dir_shift(uint32_t largest_word) {
+    return max(0, 32 - __clz(static_cast<int>(largest_word)) - KEY_DIR_BITS);
+}
+
+// Largest first key word over the tables' last buckets (keys ascend inside a table), into dir[0].
+__global__ __launch_bounds__(256) void key_dir_max_kernel(const uint32_t* __restrict__ bucket_keys,
+                                                         const int32_t* __restrict__ table_bucket_offsets, int T,
+                                                         int W, uint32_t* __restrict__ dir) {
+    const int t = blockIdx.x * 256 + threadIdx.x;
+    if (t < T && table_bucket_offsets[t + 1] > table_bucket_offsets[t])
+        atomicMax(&dir[0], bucket_keys[static_cast<size_t>(table_bucket_offsets[t + 1] - 1) * W]);
+}
+
+// entry[x] of table blockIdx.y = first bucket whose leading bits are >= x; entry[KEY_DIR_SIZE] = the
+// table's end.  A bucket fills the entries between its predecessor's leading bits and its own.
+__global__ __launch_bounds__(256) void key_dir_fill_kernel(const uint32_t* __restrict__ bucket_keys,
+                                                          const int32_t* __restrict__ table_bucket_offsets, int W,
+                                                          uint32_t* __restrict__ dir) {
+    const int t = blockIdx.y;
+    const int shift = key_dir_shift(dir[0]);
+    const int begin = table_bucket_offsets[t], end = table_bucket_offsets[t + 1];
+    uint32_t* entry = dir + 1 + static_cast<size_t>(t) * (KEY_DIR_SIZE + 1);
+    const int first = blockIdx.x * 256 + threadIdx.x, stride = gridDim.x * 256;
+    if (begin == end) {  // no bucket: every entry is the empty range
+        for (int x = first; x <= KEY_DIR_SIZE; x += stride) entry[x] = static_cast<uint32_t>(begin);
+        return;
+    }
+    for (int i = begin + first; i < end; i += stride) {
+        const int lead = static_cast<int>(bucket_keys[static_cast<size_t>(i) * W] >> shift);  // < KEY_DIR_SIZE
+        const int before = i == begin ? -1 : static_cast<int>(bucket_keys[static_cast<size_t>(i - 1) * W] >> shift);
+        for (int x = before + 1; x <= lead; ++x) entry[x] = static_cast<uint32_t>(i);
+        if (i == end - 1)
+            for (int x = lead + 1; x <= KEY_DIR_SIZE; ++x) entry[x] = static_cast<uint32_t>(end);
+    }
+}
+
+// Binary search of every (query, table) key among the table's sorted bucket keys, inside the range
+// the directory gives for the key's leading bits (the whole table without a directory); writes
 // the matched bucket id (-1 = none) and / or its span (start, length) of candidate rows.
 __global__ __launch_bounds__(256) void lookup_kernel(const uint32_t* __restrict__ q_keys,
                                                     const uint32_t* __restrict__ bucket_keys,
+                                                    const uint32_t* __restrict__ dir,
                                                     const int32_t* __restrict__ table_bucket_offsets,
                                                     const int32_t* __restrict__ bucket_candidate_offsets,
                                                     int n_queries, int T, int W, int32_t* __restrict__ matched,
@@ -48,6 +88,16 @@ __global__ __launch_bounds__(256) void lookup_kernel(const uint32_t* __restrict_
     const int q = live ? static_cast<int>(idx / T) : 0, t = live ? static_cast<int>(idx - static_cast<size_t>(q) * T) : 0;
     const uint32_t* key = q_keys + (static_cast<size_t>(t) * n_queries + q) * W;
     int lo = live ? table_bucket_offsets[t] : 0, hi = live ? table_bucket_offsets[t + 1] - 1 : -1;
+    if (live && dir) {
+        const uint32_t lead = key[0] >> key_dir_shift(dir[0]);
+        if (lead >= static_cast<uint32_t>(KEY_DIR_SIZE)) {
+            hi = lo - 1;  // beyond every bucket key
+        } else {
+            const uint32_t* entry = dir + 1 + static_cast<size_t>(t) * (KEY_DIR_SIZE + 1) + lead;
+            lo = static_cast<int>(entry[0]);
+            hi = static_cast<int>(entry[1]) - 1;
+        }
+    }
     int found = -1;
     while (lo <= hi) {
         const int mid = lo + ((hi - lo) >> 1);
@@ -615,6 +665,26 @@ __global__ __launch_bounds__(DD_THREADS) void dedup_kernel(DedupArgs a) {
 
 }  // namespace
 
+culsh_status build_key_directory(culsh_ctx* ctx, culsh_index* index) {
+    const int T = index->n_hash_tables;
+    dev_free(index->key_dir);
+    index->key_dir = nullptr;
+    if (T > KEY_DIR_MAX_TABLES || index->key_w < 1) return CULSH_OK;
+    const size_t words = 1 + static_cast<size_t>(T) * (KEY_DIR_SIZE + 1);
+    CULSH_HIP(dev_malloc(&index->key_dir, words * sizeof(uint32_t)));
+    CULSH_HIP(hipMemsetAsync(index->key_dir, 0, sizeof(uint32_t), ctx->stream));
+    CULSH_LAUNCH(ctx, key_dir_max_kernel, dim3(div_up(static_cast<size_t>(T), 256)), dim3(256), 0, ctx->stream,
+                 index->bucket_keys, index->table_bucket_offsets, T, index->key_w, index->key_dir);
+    CULSH_LAUNCH_CHECK();
+    // a table holds at most one bucket per row
+    const size_t rows = static_cast<size_t>(index->n_total_candidates / T);
+    const unsigned per_table = static_cast<unsigned>(std::max<size_t>(1, std::min<size_t>(64, div_up(rows, 1024))));
+    CULSH_LAUNCH(ctx, key_dir_fill_kernel, dim3(per_table, static_cast<unsigned>(T)), dim3(256), 0, ctx->stream,
+                 index->bucket_keys, index->table_bucket_offsets, index->key_w, index->key_dir);
+    CULSH_LAUNCH_CHECK();
+    return CULSH_OK;
+}
+
 culsh_status launch_find_matching_buckets(culsh_ctx* ctx, const uint32_t* q_keys, int n_queries,
                                           const culsh_index* index, int32_t* matched, void* spans,
                                           unsigned long long* raw_total) {
@@ -622,7 +692,7 @@ culsh_status launch_find_matching_buckets(culsh_ctx* ctx, const uint32_t* q_keys
     CULSH_REQUIRE(pairs / 256 < (1ull << 31), CULSH_ERR_LIMIT, "too many (query, table) pairs");
     CULSH_REQUIRE(!spans || raw_total, CULSH_ERR_INTERNAL, "spans need a raw candidate counter");
     CULSH_LAUNCH(ctx, lookup_kernel, dim3(div_up(pairs, 256)), dim3(256), 0, ctx->stream, q_keys,
-                 index->bucket_keys, index->table_bucket_offsets, index->bucket_candidate_offsets, n_queries,
+                 index->bucket_keys, index->key_dir, index->table_bucket_offsets, index->bucket_candidate_offsets, n_queries,
                  index->n_hash_tables, index->key_w, matched, static_cast<int2*>(spans), raw_total);
     CULSH_LAUNCH_CHECK();
     return CULSH_OK;

@@ -259,6 +259,36 @@ def test_core_query_wide_row_range(ctx, c_oracle, n):
     ctx.free_index(ih)
 
 
+@pytest.mark.parametrize("top", [0xFFFFFFFF, 0x000FFFFF, 0x00000FFF, 5, 0])
+def test_core_lookup_directory_edges(ctx, top):
+    """The lookup narrows its binary search through a directory over the leading bits of the keys'
+    first words, counted from the highest bit any bucket key has set.  Keys at both ends of the range
+    up to `top`, directory cells that are empty, full or shared by many buckets, and query keys below,
+    between and beyond the bucket keys (also beyond `top`) must all be found or missed as by the oracle."""
+    _announce("lookup_directory_edges", top)
+    rng = np.random.default_rng(top % 1000 + 3)
+    T, n, nq = 3, 3000, 600
+
+    def as_sig(words):  # opaque 4-byte signatures whose byte order is the key order
+        return np.ascontiguousarray(words.astype(">u4")).view(np.uint8).reshape(words.shape + (4,))
+
+    special = np.array([0, 1, top // 2, max(top, 1) - 1, top], dtype=np.uint64)
+    words = rng.integers(0, int(top) + 1, size=(T, n), dtype=np.uint64)
+    words[:, :400] = words[:, :1] // 2                      # one crowded bucket per table
+    words[:, 400:400 + special.size] = special
+    words[2, :] = top                                       # a table with a single bucket, at the top
+    q = rng.integers(0, min(int(top) * 2 + 2, 1 << 32), size=(T, nq), dtype=np.uint64)
+    q[:, :200] = words[:, rng.integers(0, n, 200)]          # exact hits
+    q[:, 200:210] = np.array([0, 1, top, min(top + 1, 0xFFFFFFFF), 0xFFFFFFFF, top // 2, 2, 3, 4, 5], dtype=np.uint64)
+    q[:, 210:300] = np.minimum(words[:, 1000:1090] + 1, 0xFFFFFFFF)   # just beside a bucket key
+    sig, qsig = as_sig(words.astype(np.uint32)), as_sig(q.astype(np.uint32))
+    ih, _ = ctx.core_fit_index(sig, 1)
+    from abi import assert_candidates_match
+
+    assert_candidates_match(ctx.core_query_index(qsig, ih), o.query_index(qsig, o.fit_index(sig, 1)))
+    ctx.free_index(ih)
+
+
 @pytest.mark.parametrize("two_pass", [False, True])
 def test_core_query_many_bitmap_passes(ctx, monkeypatch, two_pass):
     """A small bitmap (32768 rows per pass) makes a 150k-row index take five passes per query: in the
