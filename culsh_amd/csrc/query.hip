@@ -85,7 +85,10 @@ __global__ __launch_bounds__(256) void lookup_kernel(const uint32_t* __restrict_
     __syncthreads();
     const size_t idx = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
     const bool live = idx < static_cast<size_t>(n_queries) * T;
-    const int q = live ? static_cast<int>(idx / T) : 0, t = live ? static_cast<int>(idx - static_cast<size_t>(q) * T) : 0;
+    // neighbouring threads: neighbouring queries of one table (their keys are neighbours in memory and
+    // they walk the same table's directory and buckets); results are stored per query
+    const int t = live ? static_cast<int>(idx / n_queries) : 0, q = live ? static_cast<int>(idx - static_cast<size_t>(t) * n_queries) : 0;
+    const size_t slot = static_cast<size_t>(q) * T + t;
     const uint32_t* key = q_keys + (static_cast<size_t>(t) * n_queries + q) * W;
     int lo = live ? table_bucket_offsets[t] : 0, hi = live ? table_bucket_offsets[t + 1] - 1 : -1;
     if (live && dir) {
@@ -107,14 +110,14 @@ __global__ __launch_bounds__(256) void lookup_kernel(const uint32_t* __restrict_
         if (cmp == 0) { found = mid; break; }
         if (cmp < 0) hi = mid - 1; else lo = mid + 1;
     }
-    if (live && matched) matched[idx] = found;
+    if (live && matched) matched[slot] = found;
     if (spans) {
         int2 sp = make_int2(0, 0);
         if (found >= 0) {
             sp.x = bucket_candidate_offsets[found];
             sp.y = bucket_candidate_offsets[found + 1] - sp.x;
         }
-        if (live) spans[idx] = sp;
+        if (live) spans[slot] = sp;
         // number of raw candidates: one atomic per wavefront in LDS, one per workgroup in memory
         const unsigned long long wsum = wave_sum(static_cast<unsigned long long>(sp.y));
         if ((threadIdx.x & 63) == 0 && wsum) atomicAdd(&block_raw, wsum);
