@@ -2,7 +2,7 @@
 """
 Benchmark of the RPLSH fit/query hot path on one MI355X.
 
-Workload (BASELINE.json configs[1], the one the metric is quoted on): X = 1,000,000 x 128
+Workload (the second of the reference's benchmark configurations, the one its headline figures are quoted on): X = 1,000,000 x 128
 fp32 with integer entries in [0,255] from a clipped Gamma(0.5, 30); Q = 10,000 rows
 sampled from X plus N(0, 3^2) noise, clipped to [0,255]; 32 tables x 16 hashes; P ~ N(0,1)
 from seed 42.  One step = fit(X) followed by query(Q) with X and Q already resident in

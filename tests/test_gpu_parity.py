@@ -644,7 +644,7 @@ def test_object_memory_is_reused_and_trimmed(ctx):
 
 
 def test_full_size_invariants(ctx):
-    """BASELINE config 2 at its real size (1M x 128, 32 tables x 16 hashes, 10k queries): properties
+    """Benchmark configuration 2 of the reference at its real size (1M x 128, 32 tables x 16 hashes, 10k queries): properties
     that hold for any correct index / candidate set, checked on everything, plus a brute-force
     comparison for a sample of queries."""
     _announce("full_size")
@@ -707,7 +707,7 @@ def test_full_size_invariants(ctx):
 
 
 def test_config5_full_size_invariants(ctx):
-    """BASELINE config 5 at its real shape (4M x 768 rows of a 1000-component Gaussian mixture on the
+    """Benchmark configuration 5 of the reference at its real shape (4M x 768 rows of a 1000-component Gaussian mixture on the
     unit sphere, 64 tables x 16 hashes), 20k queries in batches of 10k: the index takes 2^28 items, a
     query four bitmap passes over the row range, and the batches are merged.  Data are made and the
     properties checked on the device; a sample of buckets and of queries is compared with brute force."""
