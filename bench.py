@@ -8,7 +8,7 @@ sampled from X plus N(0, 3^2) noise, clipped to [0,255]; 32 tables x 16 hashes; 
 from seed 42.  One step = fit(X) followed by query(Q) with X and Q already resident in
 HBM.  `value` is the fit throughput in Mvec/s; the query throughput is reported beside it.
 
-Prints ONE JSON line (see the driver contract): metric/value/unit, per-step time,
+Prints ONE JSON line: metric/value/unit, per-step time,
 `roofline` for the dominant kernel (algorithmic work / HIP-event time measured inside this
 run) and `cpu_baseline` (the C restatement in oracle/ timed on this host's cores on the
 same workload; it is also the parity check of this run).
