@@ -112,6 +112,10 @@ struct culsh_ctx {
     // switch to the unchained passes after a give-up
     uint32_t* sort_err_dev = nullptr;
     bool sort_unchained = false;
+    // raw candidates per query of the last query call and the shape of the index it went to (rows,
+    // buckets, tables, hashes): sizes the next call's output without a host round trip (query.hip)
+    uint64_t raw_guess_key = 0;
+    double raw_guess_per_query = 0.0;
     int lds_max = 0;                     // max LDS bytes per workgroup
     int n_cus = 0;
     // per-kernel timing with HIP events on `stream` (off unless enabled)

@@ -789,10 +789,33 @@ culsh_status query_from_spans(culsh_ctx* ctx, const int2* spans, const unsigned 
     bool fused = env_int("CULSH_DEDUP_TWO_PASS", 0) == 0;
     const bool several = n_chunks > 1;
     uint64_t U = 0;
-    if (fused) {
+    // The output is sized by the number of raw candidates R.  One pass per query: when the previous call
+    // went to an index of the same shape (the same index, or one fitted again), its raw candidates per query (plus a quarter) size this call's output and
+    // R is read back together with the result, one host round trip instead of two; the kernel does not
+    // write beyond the capacity, and a call that would have is redone with R known.
+    // CULSH_QUERY_RAW_GUESS (tests): raw candidates per query to assume, 0 = never guess.
+    const int forced_guess = env_int("CULSH_QUERY_RAW_GUESS", -1);
+    const uint64_t shape = (static_cast<uint64_t>(index->n_total_candidates) << 32 ^ static_cast<uint64_t>(index->n_total_buckets)) *
+                               0x9E3779B97F4A7C15ull +
+                           (static_cast<uint64_t>(T) << 20 ^ static_cast<uint64_t>(index->n_hashes));
+    double guess = forced_guess >= 0 ? static_cast<double>(forced_guess)
+                                     : (ctx->raw_guess_key == shape ? ctx->raw_guess_per_query : 0.0);
+    for (int attempt = 0; fused && attempt < 2; ++attempt) {
+        const uint64_t bound = static_cast<uint64_t>(n_queries) * static_cast<uint64_t>(n);
+        const bool guessed = attempt == 0 && !several && guess > 0.0;
+        unsigned long long* words = const_cast<unsigned long long*>(raw_total);
         uint64_t R = 0;
-        CULSH_TRY(read_back_u64(ctx, reinterpret_cast<const uint64_t*>(raw_total), 1, &R));  // host sync 1 of 2
-        if (R == 0) {  // no query matched any bucket (query.cuh:358-365: counts/offsets stay, indices stay null)
+        if (attempt == 1) {  // the guess was too small: R is known by now, the kernel's words start from zero again
+            R = ctx->pinned[2];
+            CULSH_HIP(hipMemsetAsync(words + 1, 0, (1 + static_cast<size_t>(n_queries)) * sizeof(unsigned long long), ctx->stream));
+        } else if (!guessed) {
+            CULSH_TRY(read_back_u64(ctx, reinterpret_cast<const uint64_t*>(raw_total), 1, &R));  // host sync 1 of 2
+        }
+        if (!guessed) {
+            ctx->raw_guess_key = shape;
+            ctx->raw_guess_per_query = static_cast<double>(R) / n_queries;
+        }
+        if (!guessed && R == 0) {  // no query matched any bucket (query.cuh:358-365: counts/offsets stay, indices stay null)
             CULSH_HIP(hipMemsetAsync(out->query_candidate_counts, 0, static_cast<size_t>(n_queries) * sizeof(uint64_t), ctx->stream));
             CULSH_HIP(hipMemsetAsync(out->query_candidate_offsets, 0, (static_cast<size_t>(n_queries) + 1) * sizeof(uint64_t), ctx->stream));
             out->n_total_candidates = 0;
@@ -802,8 +825,9 @@ culsh_status query_from_spans(culsh_ctx* ctx, const int2* spans, const unsigned 
         // One pass: lists are packed by a chained scan over the queries; a query holds at most n
         // distinct rows, which bounds the output when buckets overlap heavily.  Several passes: list q
         // starts at the sum of the raw counts of the queries before it, and the gaps are closed below.
-        const uint64_t cap = several ? R : std::min<uint64_t>(R, static_cast<uint64_t>(n_queries) * static_cast<uint64_t>(n));
-        unsigned long long* words = const_cast<unsigned long long*>(raw_total);
+        const uint64_t cap = several ? R
+                             : guessed ? std::min<uint64_t>(bound, static_cast<uint64_t>(guess * n_queries * 1.25) + 1024)
+                                       : std::min<uint64_t>(R, bound);
         unsigned int* err = reinterpret_cast<unsigned int*>(words + 1);  // [0] error flags, [1] ticket counter
         a.state = words + 2;
         a.ticket = err + 1;
@@ -842,9 +866,21 @@ culsh_status query_from_spans(culsh_ctx* ctx, const int2* spans, const unsigned 
         CULSH_HIP(hipMemcpyAsync(&ctx->pinned[0], out->query_candidate_offsets + n_queries, sizeof(uint64_t),
                                  hipMemcpyDeviceToHost, ctx->stream));
         CULSH_HIP(hipMemcpyAsync(&ctx->pinned[1], err, sizeof(unsigned int), hipMemcpyDeviceToHost, ctx->stream));
-        CULSH_HIP(hipStreamSynchronize(ctx->stream));  // host sync 2 of 2
+        if (guessed)
+            CULSH_HIP(hipMemcpyAsync(&ctx->pinned[2], raw_total, sizeof(uint64_t), hipMemcpyDeviceToHost, ctx->stream));
+        CULSH_HIP(hipStreamSynchronize(ctx->stream));  // host sync 2 of 2 (the only one after a guess)
         U = ctx->pinned[0];
         const unsigned int e = static_cast<unsigned int>(ctx->pinned[1] & 0xffffffffu);
+        if (guessed) {
+            ctx->raw_guess_key = shape;
+            ctx->raw_guess_per_query = static_cast<double>(ctx->pinned[2]) / n_queries;
+        }
+        if (guessed && e == 2u) {  // the guess was too small and nothing else went wrong: once more with R
+            dev_free(lists);
+            out->query_candidate_indices = nullptr;
+            guess = 0.0;
+            continue;
+        }
         if (e != 0) {  // never seen; the two-launch path below needs no cooperation between workgroups
             dev_free(lists);
             out->query_candidate_indices = nullptr;
@@ -876,6 +912,7 @@ culsh_status query_from_spans(culsh_ctx* ctx, const int2* spans, const unsigned 
             dev_free(lists);
             CULSH_HIP(err_copy);
         }
+        break;
     }
     if (!fused) {
         CULSH_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(dedup_kernel<DD_COUNT>),

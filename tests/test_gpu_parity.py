@@ -259,6 +259,33 @@ def test_core_query_wide_row_range(ctx, c_oracle, n):
     ctx.free_index(ih)
 
 
+def test_core_query_output_sized_from_previous_call(ctx, monkeypatch):
+    """A second query call on an index sizes its output from the first call's raw candidates per query
+    and reads the true number back afterwards.  Calls whose queries bring fewer, as many, and far more
+    candidates than the call before (the last overflows the guessed size and is redone), then forced
+    guesses of one candidate per query and of more than the index holds, and a call without any match."""
+    _announce("output_sized_from_previous_call")
+    from abi import assert_candidates_match
+
+    rng = np.random.default_rng(61)
+    T, n, H = 6, 20000, 2
+    sig = rng.integers(0, 30, size=(T, n, H)).astype(np.uint8)
+    sig[:, :5000, :] = 7                                   # one bucket of 5000 rows per table
+    ih, _ = ctx.core_fit_index(sig, H)
+    exp_ix = o.fit_index(sig, H)
+    few = rng.integers(8, 30, size=(T, 300, H)).astype(np.uint8)
+    many = few.copy()
+    many[:, ::2, :] = 7                                    # every other query hits the large bucket in every table
+    none = np.full((T, 50, H), 200, np.uint8)
+    for qsig in (few, few, many, few, none, few, many[:, :10], many):
+        assert_candidates_match(ctx.core_query_index(qsig, ih), o.query_index(qsig, exp_ix))
+    for forced in ("1", "100000000", "0"):
+        monkeypatch.setenv("CULSH_QUERY_RAW_GUESS", forced)
+        for qsig in (many, none, few):
+            assert_candidates_match(ctx.core_query_index(qsig, ih), o.query_index(qsig, exp_ix))
+    ctx.free_index(ih)
+
+
 @pytest.mark.parametrize("top", [0xFFFFFFFF, 0x000FFFFF, 0x00000FFF, 5, 0])
 def test_core_lookup_directory_edges(ctx, top):
     """The lookup narrows its binary search through a directory over the leading bits of the keys'
