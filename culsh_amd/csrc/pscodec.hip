@@ -194,7 +194,7 @@ __global__ __launch_bounds__(256) void ps_keys_to_sig_kernel(const uint32_t* __r
     const int t_first = static_cast<int>(tb[0]);
     const bool staged = use_lds && static_cast<int>(tb[nb - 1]) - t_first <= 1;  // uniform over the workgroup
     if (staged) {
-        const int words = min(2, T - t_first) * H * rmax;
+        const int words = (static_cast<int>(tb[nb - 1]) - t_first + 1) * H * rmax;  // one table's values, or two
         const int32_t* src = inv + static_cast<size_t>(t_first) * H * rmax;
         for (int i = threadIdx.x; i < words; i += 256) lut[i] = src[i];
         __syncthreads();
