@@ -192,6 +192,32 @@ __global__ __launch_bounds__(256) void keys_to_sig_kernel(const uint32_t* __rest
     }
 }
 
+// Sign-bit keys, signature width a multiple of four bytes: a thread expands VEC (1 or 4) groups of four
+// key bits into four 0/1 bytes each and stores them at once.  The four bits, highest first, go to
+// bytes 0..3 of a word: ((nibble * 0x08040201) >> 3) & 0x01010101.
+template <int VEC>
+__global__ __launch_bounds__(256) void bit_keys_to_sig_kernel(const uint32_t* __restrict__ keys, size_t count,
+                                                             const uint64_t* __restrict__ count_dev, int S, int W,
+                                                             uint32_t* __restrict__ sig) {
+    if (count_dev) count = min(count, static_cast<size_t>(*count_dev));  // exact count known on the device only
+    const uint32_t per_item = static_cast<uint32_t>(S) / (4u * VEC);     // stores per bucket
+    const size_t g = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (g >= count * per_item) return;
+    const size_t item = g / per_item;
+    const uint32_t first = static_cast<uint32_t>(g - item * per_item) * VEC;  // first group of four bits
+    const uint32_t word = keys[item * W + (first >> 3)];
+    uint32_t out[VEC];
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) {
+        const uint32_t nibble = (word >> (28u - 4u * ((first + v) & 7u))) & 15u;
+        out[v] = ((nibble * 0x08040201u) >> 3) & 0x01010101u;
+    }
+    if (VEC == 4)
+        reinterpret_cast<uint4*>(sig)[g] = make_uint4(out[0], out[VEC > 1 ? 1 : 0], out[VEC > 2 ? 2 : 0], out[VEC > 3 ? 3 : 0]);
+    else
+        sig[g] = out[0];
+}
+
 }  // namespace
 
 culsh_status launch_sig_to_keys(culsh_ctx* ctx, const uint8_t* sig, size_t n_items, int S, KeyEnc enc, int W,
@@ -211,8 +237,16 @@ culsh_status launch_keys_to_sig(culsh_ctx* ctx, const uint32_t* keys, size_t cou
     const size_t total = count * S;
     CULSH_REQUIRE(total / 1024 < (1ull << 31), CULSH_ERR_LIMIT, "too many buckets");
     CULSH_REQUIRE(reinterpret_cast<uintptr_t>(sig) % 4 == 0, CULSH_ERR_INTERNAL, "signature array is not 4-byte aligned");
-    CULSH_LAUNCH(ctx, keys_to_sig_kernel, dim3(div_up(div_up(total, 4), 256)), dim3(256), 0, ctx->stream, keys, count,
-                 count_dev, S, static_cast<int>(enc), W, sig);
+    if (enc == ENC_BITS && S % 16 == 0 && reinterpret_cast<uintptr_t>(sig) % 16 == 0) {
+        CULSH_LAUNCH(ctx, bit_keys_to_sig_kernel<4>, dim3(div_up(total / 16, 256)), dim3(256), 0, ctx->stream, keys, count,
+                     count_dev, S, W, reinterpret_cast<uint32_t*>(sig));
+    } else if (enc == ENC_BITS && S % 4 == 0) {
+        CULSH_LAUNCH(ctx, bit_keys_to_sig_kernel<1>, dim3(div_up(total / 4, 256)), dim3(256), 0, ctx->stream, keys, count,
+                     count_dev, S, W, reinterpret_cast<uint32_t*>(sig));
+    } else {
+        CULSH_LAUNCH(ctx, keys_to_sig_kernel, dim3(div_up(div_up(total, 4), 256)), dim3(256), 0, ctx->stream, keys, count,
+                     count_dev, S, static_cast<int>(enc), W, sig);
+    }
     CULSH_LAUNCH_CHECK();
     return CULSH_OK;
 }
