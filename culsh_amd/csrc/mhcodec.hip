@@ -263,13 +263,25 @@ __global__ __launch_bounds__(256) void mh_keys_to_sig_kernel(const uint32_t* __r
     for (int i = threadIdx.x; i < nb * W; i += 256) kw[i] = keys[b0 * W + i];
     __syncthreads();
     const uint32_t mask = (1u << bits) - 1u;
-    for (int i = threadIdx.x; i < nb * H; i += 256) {
-        const int bl = i / H, h = i - bl * H;
+    auto value = [&](int bl, int h) -> uint32_t {
         const uint32_t* k = kw + bl * W;
         const int o = h * bits, w0 = o >> 5, sh = o & 31;
         const unsigned long long two = (static_cast<unsigned long long>(k[w0]) << 32) | (w0 + 1 < W ? k[w0 + 1] : 0u);
         const uint32_t code = static_cast<uint32_t>(two >> (64 - sh - bits)) & mask;
-        sig[b0 * H + i] = code < static_cast<uint32_t>(d) ? inv[static_cast<size_t>(tb[bl] * H + h) * d + code] : 0xFFFFFFFFu;
+        return code < static_cast<uint32_t>(d) ? inv[static_cast<size_t>(tb[bl] * H + h) * d + code] : 0xFFFFFFFFu;
+    };
+    uint32_t* out = sig + b0 * H;
+    if (H % 4 == 0 && reinterpret_cast<uintptr_t>(sig) % 16 == 0) {  // four hashes of a bucket per thread and store
+        const int qpb = H >> 2;
+        for (int q = threadIdx.x; q < nb * qpb; q += 256) {
+            const int bl = q / qpb, h = (q - bl * qpb) << 2;
+            *reinterpret_cast<uint4*>(out + 4 * q) = make_uint4(value(bl, h), value(bl, h + 1), value(bl, h + 2), value(bl, h + 3));
+        }
+    } else {
+        for (int i = threadIdx.x; i < nb * H; i += 256) {
+            const int bl = i / H;
+            out[i] = value(bl, i - bl * H);
+        }
     }
 }
 
