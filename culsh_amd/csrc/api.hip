@@ -1206,7 +1206,7 @@ culsh_status culsh_index_load(culsh_ctx* ctx, culsh_kind kind, int is_double, co
     }
     CULSH_HIP(dev_malloc(&ix->bucket_keys, std::max<size_t>(1, static_cast<size_t>(n_total_buckets) * ix->key_w) * 4));
     CULSH_TRY(launch_sig_to_keys(ctx, ix->all_bucket_signatures, n_total_buckets, S, enc, ix->key_w, ix->bucket_keys));
-    CULSH_TRY(build_key_directory(ctx, ix.get()));
+    CULSH_TRY(build_key_directory(ctx, ix.get(), static_cast<size_t>(n_total_buckets)));
     CULSH_TRY(arena_end(ctx));
     *out = ix.release();
     return CULSH_OK;

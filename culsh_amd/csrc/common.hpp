@@ -314,7 +314,8 @@ culsh_status fit_index_from_keys(culsh_ctx* ctx, uint32_t* keys, int n, int T, i
 // set), where the buckets with that value start.  Layout: [0] = largest first word of any bucket key,
 // then per table KEY_DIR_SIZE + 1 bucket numbers.  Not built for more than KEY_DIR_MAX_TABLES tables.
 constexpr int KEY_DIR_BITS = 12, KEY_DIR_SIZE = 1 << KEY_DIR_BITS, KEY_DIR_MAX_TABLES = 1024;
-culsh_status build_key_directory(culsh_ctx* ctx, culsh_index* index);
+// `bucket_bound`: the number of buckets or an upper bound of it (sizes the launch only).
+culsh_status build_key_directory(culsh_ctx* ctx, culsh_index* index, size_t bucket_bound);
 
 culsh_status launch_find_matching_buckets(culsh_ctx* ctx, const uint32_t* q_keys, int n_queries,
                                           const culsh_index* index, int32_t* matched, void* spans = nullptr,

@@ -292,7 +292,7 @@ culsh_status build_index_from_sorted(culsh_ctx* ctx, const uint32_t* sorted_keys
                        sorted_keys, rows_sorted_owned, N, n, T, W, tile_base, total_dev, index->bucket_candidate_offsets,
                        index->bucket_keys, index->table_bucket_offsets, item_to_bucket_opt);
     CULSH_LAUNCH_CHECK();
-    CULSH_TRY(build_key_directory(ctx, index));
+    CULSH_TRY(build_key_directory(ctx, index, B_bound));
     if (enc == ENC_PSC)
         CULSH_TRY(launch_ps_keys_to_sig(ctx, index, B_bound, total_dev, index->all_bucket_signatures));
     else if (enc == ENC_MHR)

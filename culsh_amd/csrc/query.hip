@@ -46,27 +46,54 @@ __global__ __launch_bounds__(256) void key_dir_max_kernel(const uint32_t* __rest
         atomicMax(&dir[0], bucket_keys[static_cast<size_t>(table_bucket_offsets[t + 1] - 1) * W]);
 }
 
-// entry[x] of table blockIdx.y = first bucket whose leading bits are >= x; entry[KEY_DIR_SIZE] = the
-// table's end.  A bucket fills the entries between its predecessor's leading bits and its own.
-__global__ __launch_bounds__(256) void key_dir_fill_kernel(const uint32_t* __restrict__ bucket_keys,
+// entry[x] of table t = first bucket whose leading bits are >= x; entry[KEY_DIR_SIZE] = the table's
+// end.  Two steps.  Mark (table blockIdx.y): the first bucket with leading bits x writes entry[x]; all
+// other entries hold ~0 from a fill before.  Close (one workgroup per table): every entry takes the
+// smallest value at or behind it, the last one being the table's end.
+__global__ __launch_bounds__(256) void key_dir_mark_kernel(const uint32_t* __restrict__ bucket_keys,
                                                           const int32_t* __restrict__ table_bucket_offsets, int W,
                                                           uint32_t* __restrict__ dir) {
     const int t = blockIdx.y;
     const int shift = key_dir_shift(dir[0]);
     const int begin = table_bucket_offsets[t], end = table_bucket_offsets[t + 1];
     uint32_t* entry = dir + 1 + static_cast<size_t>(t) * (KEY_DIR_SIZE + 1);
-    const int first = blockIdx.x * 256 + threadIdx.x, stride = gridDim.x * 256;
-    if (begin == end) {  // no bucket: every entry is the empty range
-        for (int x = first; x <= KEY_DIR_SIZE; x += stride) entry[x] = static_cast<uint32_t>(begin);
-        return;
+    for (int i = begin + blockIdx.x * 256 + threadIdx.x; i < end; i += gridDim.x * 256) {
+        const uint32_t lead = bucket_keys[static_cast<size_t>(i) * W] >> shift;  // < KEY_DIR_SIZE
+        if (i == begin || (bucket_keys[static_cast<size_t>(i - 1) * W] >> shift) != lead) entry[lead] = static_cast<uint32_t>(i);
     }
-    for (int i = begin + first; i < end; i += stride) {
-        const int lead = static_cast<int>(bucket_keys[static_cast<size_t>(i) * W] >> shift);  // < KEY_DIR_SIZE
-        const int before = i == begin ? -1 : static_cast<int>(bucket_keys[static_cast<size_t>(i - 1) * W] >> shift);
-        for (int x = before + 1; x <= lead; ++x) entry[x] = static_cast<uint32_t>(i);
-        if (i == end - 1)
-            for (int x = lead + 1; x <= KEY_DIR_SIZE; ++x) entry[x] = static_cast<uint32_t>(end);
+}
+
+__global__ __launch_bounds__(256) void key_dir_close_kernel(const int32_t* __restrict__ table_bucket_offsets,
+                                                           uint32_t* __restrict__ dir) {
+    constexpr int PER = KEY_DIR_SIZE / 256;  // entries per thread
+    __shared__ uint32_t tail[256];
+    const int t = blockIdx.x, tid = threadIdx.x;
+    uint32_t* entry = dir + 1 + static_cast<size_t>(t) * (KEY_DIR_SIZE + 1);
+    const uint32_t end = static_cast<uint32_t>(table_bucket_offsets[t + 1]);
+    uint32_t v[PER];
+    uint32_t low = end;  // smallest value at or behind this thread's entries, inside its own part
+#pragma unroll
+    for (int k = PER - 1; k >= 0; --k) {
+        low = min(low, entry[tid * PER + k]);
+        v[k] = low;
     }
+    // smallest value of the threads behind this one: inside the wavefront by shuffles, then over the
+    // wavefronts behind
+    const int lane = tid & 63, wave = tid >> 6;
+    uint32_t incl = low;  // minimum over lanes >= this one
+#pragma unroll
+    for (int step = 1; step < 64; step <<= 1) {
+        const uint32_t other = __shfl_down(incl, step, 64);
+        if (lane + step < 64) incl = min(incl, other);
+    }
+    uint32_t behind = __shfl_down(incl, 1, 64);
+    if (lane == 63) behind = end;
+    if (lane == 0) tail[wave] = incl;
+    __syncthreads();
+    for (int w = wave + 1; w < 4; ++w) behind = min(behind, tail[w]);
+#pragma unroll
+    for (int k = 0; k < PER; ++k) entry[tid * PER + k] = min(v[k], behind);
+    if (tid == 0) entry[KEY_DIR_SIZE] = end;
 }
 
 // Binary search of every (query, table) key among the table's sorted bucket keys, inside the range
@@ -668,22 +695,25 @@ __global__ __launch_bounds__(DD_THREADS) void dedup_kernel(DedupArgs a) {
 
 }  // namespace
 
-culsh_status build_key_directory(culsh_ctx* ctx, culsh_index* index) {
+culsh_status build_key_directory(culsh_ctx* ctx, culsh_index* index, size_t bucket_bound) {
     const int T = index->n_hash_tables;
     dev_free(index->key_dir);
     index->key_dir = nullptr;
     if (T > KEY_DIR_MAX_TABLES || index->key_w < 1) return CULSH_OK;
     const size_t words = 1 + static_cast<size_t>(T) * (KEY_DIR_SIZE + 1);
     CULSH_HIP(dev_malloc(&index->key_dir, words * sizeof(uint32_t)));
+    CULSH_HIP(hipMemsetAsync(index->key_dir, 0xFF, words * sizeof(uint32_t), ctx->stream));
     CULSH_HIP(hipMemsetAsync(index->key_dir, 0, sizeof(uint32_t), ctx->stream));
     CULSH_LAUNCH(ctx, key_dir_max_kernel, dim3(div_up(static_cast<size_t>(T), 256)), dim3(256), 0, ctx->stream,
                  index->bucket_keys, index->table_bucket_offsets, T, index->key_w, index->key_dir);
     CULSH_LAUNCH_CHECK();
-    // a table holds at most one bucket per row
-    const size_t rows = static_cast<size_t>(index->n_total_candidates / T);
-    const unsigned per_table = static_cast<unsigned>(std::max<size_t>(1, std::min<size_t>(64, div_up(rows, 1024))));
-    CULSH_LAUNCH(ctx, key_dir_fill_kernel, dim3(per_table, static_cast<unsigned>(T)), dim3(256), 0, ctx->stream,
+    // about two buckets per thread for tables of even size; larger tables take more rounds
+    const unsigned per_table = static_cast<unsigned>(std::max<size_t>(1, std::min<size_t>(4096, div_up(bucket_bound / T + 1, 512))));
+    CULSH_LAUNCH(ctx, key_dir_mark_kernel, dim3(per_table, static_cast<unsigned>(T)), dim3(256), 0, ctx->stream,
                  index->bucket_keys, index->table_bucket_offsets, index->key_w, index->key_dir);
+    CULSH_LAUNCH_CHECK();
+    CULSH_LAUNCH(ctx, key_dir_close_kernel, dim3(static_cast<unsigned>(T)), dim3(256), 0, ctx->stream,
+                 index->table_bucket_offsets, index->key_dir);
     CULSH_LAUNCH_CHECK();
     return CULSH_OK;
 }
