@@ -37,13 +37,25 @@ __device__ __forceinline__ int key_dir_shift(uint32_t largest_word) {
     return max(0, 32 - __clz(static_cast<int>(largest_word)) - KEY_DIR_BITS);
 }
 
-// Largest first key word over the tables' last buckets (keys ascend inside a table), into dir[0].
-__global__ __launch_bounds__(256) void key_dir_max_kernel(const uint32_t* __restrict__ bucket_keys,
-                                                         const int32_t* __restrict__ table_bucket_offsets, int T,
-                                                         int W, uint32_t* __restrict__ dir) {
-    const int t = blockIdx.x * 256 + threadIdx.x;
-    if (t < T && table_bucket_offsets[t + 1] > table_bucket_offsets[t])
-        atomicMax(&dir[0], bucket_keys[static_cast<size_t>(table_bucket_offsets[t + 1] - 1) * W]);
+// Workgroup t sets the entries of table t to ~0 ("no bucket starts here"); workgroup 0 also finds the
+// largest first key word over the tables' last buckets (keys ascend inside a table), into dir[0].
+__global__ __launch_bounds__(256) void key_dir_init_kernel(const uint32_t* __restrict__ bucket_keys,
+                                                          const int32_t* __restrict__ table_bucket_offsets, int T,
+                                                          int W, uint32_t* __restrict__ dir) {
+    __shared__ uint32_t largest[4];
+    const int tid = threadIdx.x;
+    uint32_t* entry = dir + 1 + static_cast<size_t>(blockIdx.x) * (KEY_DIR_SIZE + 1);
+    for (int x = tid; x <= KEY_DIR_SIZE; x += 256) entry[x] = 0xFFFFFFFFu;
+    if (blockIdx.x != 0) return;
+    uint32_t m = 0;
+    for (int t = tid; t < T; t += 256)
+        if (table_bucket_offsets[t + 1] > table_bucket_offsets[t])
+            m = max(m, bucket_keys[static_cast<size_t>(table_bucket_offsets[t + 1] - 1) * W]);
+#pragma unroll
+    for (int step = 32; step > 0; step >>= 1) m = max(m, static_cast<uint32_t>(__shfl_xor(m, step, 64)));
+    if ((tid & 63) == 0) largest[tid >> 6] = m;
+    __syncthreads();
+    if (tid == 0) dir[0] = max(max(largest[0], largest[1]), max(largest[2], largest[3]));
 }
 
 // entry[x] of table t = first bucket whose leading bits are >= x; entry[KEY_DIR_SIZE] = the table's
@@ -702,9 +714,7 @@ culsh_status build_key_directory(culsh_ctx* ctx, culsh_index* index, size_t buck
     if (T > KEY_DIR_MAX_TABLES || index->key_w < 1) return CULSH_OK;
     const size_t words = 1 + static_cast<size_t>(T) * (KEY_DIR_SIZE + 1);
     CULSH_HIP(dev_malloc(&index->key_dir, words * sizeof(uint32_t)));
-    CULSH_HIP(hipMemsetAsync(index->key_dir, 0xFF, words * sizeof(uint32_t), ctx->stream));
-    CULSH_HIP(hipMemsetAsync(index->key_dir, 0, sizeof(uint32_t), ctx->stream));
-    CULSH_LAUNCH(ctx, key_dir_max_kernel, dim3(div_up(static_cast<size_t>(T), 256)), dim3(256), 0, ctx->stream,
+    CULSH_LAUNCH(ctx, key_dir_init_kernel, dim3(static_cast<unsigned>(T)), dim3(256), 0, ctx->stream,
                  index->bucket_keys, index->table_bucket_offsets, T, index->key_w, index->key_dir);
     CULSH_LAUNCH_CHECK();
     // about two buckets per thread for tables of even size; larger tables take more rounds
