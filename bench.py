@@ -27,7 +27,6 @@ import numpy as np
 
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
-sys.path.insert(0, os.path.join(ROOT, "tests"))
 
 # MI355X published peaks used for the roofline fractions
 PEAK_FP32_MFMA_TFLOPS = 157.3
@@ -73,7 +72,7 @@ def main() -> int:
         return 2
 
     import torch
-    from abi import Ctx, dev, hp, ptr
+    from culsh_amd.abi import Ctx, dev, hp, ptr
     from culsh_amd import _lib as L
 
     n, d, nq, T, H = args.n, 128, args.queries, 32, 16

@@ -32,26 +32,31 @@ static constexpr size_t ARENA_ALIGN = 256;
 culsh_status arena_begin(culsh_ctx* ctx) {
     CULSH_HIP(hipSetDevice(ctx->device));
     ctx->arena_off = 0;
+    ctx->arena_live = 0;
+    ctx->sort_err_dev = nullptr;  // pointed into the arena of an earlier call
     if (ctx->arena_want > ctx->arena_cap) {  // stream is idle here: every call ends with a sync
-        if (ctx->arena) CULSH_HIP(hipFree(ctx->arena));
-        ctx->arena = nullptr;
-        ctx->arena_cap = 0;
+        // the new block first: a grow that fails keeps the arena there is
         const size_t want = align_up(ctx->arena_want + ctx->arena_want / 8, 1 << 20);
         void* p = nullptr;
         if (hipMalloc(&p, want) == hipSuccess) {
+            if (ctx->arena) (void)hipFree(ctx->arena);
             ctx->arena = static_cast<char*>(p);
             ctx->arena_cap = want;
         } else {
-            (void)hipGetLastError();  // fall back to per-allocation blocks
+            (void)hipGetLastError();  // what does not fit falls back to per-allocation blocks
         }
     }
     ctx->arena_want = 0;
     return CULSH_OK;
 }
 
+// `arena_want` is the high-water mark of the bytes live at once (arena + overflow blocks), which is
+// what the next call's arena is sized by; a caller that rewinds with arena_rewind (batched queries)
+// therefore asks for one batch's scratch, not the sum over the batches.
 culsh_status arena_alloc(culsh_ctx* ctx, size_t bytes, void** out) {
     bytes = align_up(std::max<size_t>(bytes, 1), ARENA_ALIGN);
-    ctx->arena_want += bytes;
+    ctx->arena_live += bytes;
+    ctx->arena_want = std::max(ctx->arena_want, ctx->arena_live);
     if (ctx->arena && ctx->arena_off + bytes <= ctx->arena_cap) {
         *out = ctx->arena + ctx->arena_off;
         ctx->arena_off += bytes;
@@ -62,6 +67,15 @@ culsh_status arena_alloc(culsh_ctx* ctx, size_t bytes, void** out) {
     ctx->overflow.push_back(p);
     *out = p;
     return CULSH_OK;
+}
+
+ArenaMark arena_mark(const culsh_ctx* ctx) { return ArenaMark{ctx->arena_off, ctx->arena_live}; }
+
+// Gives back what was allocated since `mark`.  The stream must be idle (the memory may be handed out
+// again at once); overflow blocks stay until the end of the call.
+void arena_rewind(culsh_ctx* ctx, const ArenaMark& mark) {
+    ctx->arena_off = mark.off;
+    ctx->arena_live = mark.live;
 }
 
 StageTimer::StageTimer(culsh_ctx* c, const char* name) : ctx(c) {
@@ -311,11 +325,15 @@ static culsh_status upload_params(culsh_ctx* ctx, const T* host, size_t count, T
     return CULSH_OK;
 }
 
-static culsh_status check_fit_args(culsh_ctx* ctx, const void* X, int n, int d, int T, int H, void* out) {
+// `with_query`: the fit is followed by a query of the fitted rows (fit_query), which has the query path's
+// limit on the number of tables; refused here, before any device work.
+static culsh_status check_fit_args(culsh_ctx* ctx, const void* X, int n, int d, int T, int H, void* out,
+                                   bool with_query = false) {
     CULSH_REQUIRE(ctx && X && out, CULSH_ERR_INVALID, "null argument");
     CULSH_REQUIRE(n > 0 && d > 0, CULSH_ERR_INVALID, "n_samples and n_features must be positive");
     CULSH_REQUIRE(T > 0 && H > 0, CULSH_ERR_INVALID, "n_hash_tables and n_hashes must be positive");
     CULSH_REQUIRE(T <= 65535, CULSH_ERR_LIMIT, "n_hash_tables > 65535 is not supported");
+    CULSH_REQUIRE(!with_query || T <= 1024, CULSH_ERR_LIMIT, "fit_query: n_hash_tables > 1024 is not supported");
     CULSH_REQUIRE(static_cast<long long>(n) * T < (1ll << 31), CULSH_ERR_LIMIT,
                   "n_samples * n_hash_tables must be below 2^31 (int32 candidate positions)");
     return CULSH_OK;
@@ -444,7 +462,7 @@ static culsh_status dense_query(culsh_ctx* ctx, Family fam, const T* Q, int nq, 
     std::vector<CandPtr> parts;
     for (int start = 0; start < nq; start += batch_size) {
         const int bn = std::min(batch_size, nq - start);
-        const size_t mark = ctx->arena_off;
+        const ArenaMark mark = arena_mark(ctx);
         uint32_t* keys = nullptr;
         int W = 0;
         CULSH_TRY(hash_dense_to_keys<T>(ctx, fam, Q + static_cast<size_t>(start) * d, bn, d, nT, H, ix->P, ix->b,
@@ -454,7 +472,7 @@ static culsh_status dense_query(culsh_ctx* ctx, Family fam, const T* Q, int nq, 
         part->device = ctx->device;
         CULSH_TRY(query_keys(ctx, keys, bn, ix, part.get()));
         parts.push_back(std::move(part));
-        ctx->arena_off = mark;  // later kernels run after these on the same stream
+        arena_rewind(ctx, mark);  // the batch's query has ended with the stream idle
     }
     if (parts.size() == 1) {
         CULSH_TRY(arena_end(ctx));
@@ -487,7 +505,8 @@ template <typename T>
 static culsh_status dense_fit_once(culsh_ctx* ctx, Family fam, const T* X, int n, int d, int nT, int H, int window,
                               uint64_t seed, const T* P_host, const T* b_host, culsh_index** index_out,
                               culsh_candidates** cands_out) {
-    CULSH_TRY(check_fit_args(ctx, X, n, d, nT, H, index_out ? static_cast<void*>(index_out) : static_cast<void*>(cands_out)));
+    CULSH_TRY(check_fit_args(ctx, X, n, d, nT, H, index_out ? static_cast<void*>(index_out) : static_cast<void*>(cands_out),
+                             cands_out != nullptr));
     if (fam == FAM_PSLSH) {
         CULSH_REQUIRE(window > 0, CULSH_ERR_INVALID, "window_size must be positive");
         CULSH_REQUIRE((P_host == nullptr) == (b_host == nullptr), CULSH_ERR_INVALID,
@@ -559,7 +578,8 @@ static culsh_status dense_fit_once(culsh_ctx* ctx, Family fam, const T* X, int n
 static culsh_status minhash_fit_once(culsh_ctx* ctx, const int32_t* indices, const int32_t* indptr, int n, int d,
                                      int nT, int H, uint64_t seed, const uint32_t* A_host, const uint32_t* B_host,
                                      culsh_index** index_out, culsh_candidates** cands_out) {
-    CULSH_TRY(check_fit_args(ctx, indptr, n, d, nT, H, index_out ? static_cast<void*>(index_out) : static_cast<void*>(cands_out)));
+    CULSH_TRY(check_fit_args(ctx, indptr, n, d, nT, H, index_out ? static_cast<void*>(index_out) : static_cast<void*>(cands_out),
+                             cands_out != nullptr));
     CULSH_REQUIRE((A_host == nullptr) == (B_host == nullptr), CULSH_ERR_INVALID, "hash_a and hash_b must be given together");
     ArenaScope scope(ctx);
     CULSH_TRY(scope.begin_status);
@@ -976,23 +996,32 @@ culsh_status culsh_core_fit_index(culsh_ctx* ctx, const void* X_sig, int n, int 
     return with_sort_retry(ctx, [&] { return core_fit_index_once(ctx, X_sig, n, T, H, S, item_to_bucket, out); });
 }
 
-static culsh_status sig_query_keys(culsh_ctx* ctx, const void* Q_sig, int nq, int S, const culsh_index* ix,
-                                   uint32_t** keys) {
+// Query signatures in the reference layout -> key words of the index's encoding, into `keys`
+// ([T][nq][key_w] words that the caller provides).
+static culsh_status sig_query_keys_into(culsh_ctx* ctx, const void* Q_sig, int nq, int S, const culsh_index* ix,
+                                        uint32_t* keys) {
     CULSH_REQUIRE(ctx && Q_sig && ix, CULSH_ERR_INVALID, "null argument");
     CULSH_REQUIRE(nq > 0, CULSH_ERR_INVALID, "n_queries must be positive");
     CULSH_REQUIRE(S == ix->sig_nbytes, CULSH_ERR_INVALID, "sig_nbytes (%d) != index sig_nbytes (%d)", S,
                   ix->sig_nbytes);  // core/query.cuh:494
-    CULSH_TRY(arena_alloc_t(ctx, static_cast<size_t>(nq) * ix->n_hash_tables * ix->key_w, keys));
     if (ix->enc == ENC_PSC) {
         CULSH_REQUIRE(reinterpret_cast<uintptr_t>(Q_sig) % 4 == 0, CULSH_ERR_INVALID, "signatures must be 4-byte aligned");
-        return launch_ps_compress(ctx, static_cast<const int32_t*>(Q_sig), nq, ix->n_hash_tables, ix->n_hashes, ix, *keys);
+        return launch_ps_compress(ctx, static_cast<const int32_t*>(Q_sig), nq, ix->n_hash_tables, ix->n_hashes, ix, keys);
     }
     if (ix->enc == ENC_MHR) {
         CULSH_REQUIRE(reinterpret_cast<uintptr_t>(Q_sig) % 4 == 0, CULSH_ERR_INVALID, "signatures must be 4-byte aligned");
-        return launch_mh_sig_to_keys(ctx, static_cast<const uint32_t*>(Q_sig), nq, ix, *keys);
+        return launch_mh_sig_to_keys(ctx, static_cast<const uint32_t*>(Q_sig), nq, ix, keys);
     }
     return launch_sig_to_keys(ctx, static_cast<const uint8_t*>(Q_sig), static_cast<size_t>(nq) * ix->n_hash_tables,
-                              S, ix->enc, ix->key_w, *keys);
+                              S, ix->enc, ix->key_w, keys);
+}
+
+static culsh_status sig_query_keys(culsh_ctx* ctx, const void* Q_sig, int nq, int S, const culsh_index* ix,
+                                   uint32_t** keys) {
+    CULSH_REQUIRE(ctx && Q_sig && ix, CULSH_ERR_INVALID, "null argument");
+    CULSH_REQUIRE(nq > 0, CULSH_ERR_INVALID, "n_queries must be positive");
+    CULSH_TRY(arena_alloc_t(ctx, static_cast<size_t>(nq) * ix->n_hash_tables * ix->key_w, keys));
+    return sig_query_keys_into(ctx, Q_sig, nq, S, ix, *keys);
 }
 
 culsh_status culsh_core_find_matching_buckets(culsh_ctx* ctx, const void* Q_sig, int nq, int S,
@@ -1038,7 +1067,7 @@ culsh_status culsh_core_query_from_matched_buckets(culsh_ctx* ctx, const int32_t
 
 static culsh_status core_fit_query_once(culsh_ctx* ctx, const void* X_sig, int n, int T, int H, int S,
                                   culsh_candidates** out) {
-    CULSH_TRY(check_fit_args(ctx, X_sig, n, 1, T, H, out));
+    CULSH_TRY(check_fit_args(ctx, X_sig, n, 1, T, H, out, true));
     CULSH_REQUIRE(S > 0 && S <= 256, CULSH_ERR_INVALID, "sig_nbytes must be in [1, 256]");
     ArenaScope scope(ctx);
     CULSH_TRY(scope.begin_status);

@@ -93,7 +93,8 @@ struct culsh_ctx {
     char* arena = nullptr;
     size_t arena_cap = 0;
     size_t arena_off = 0;
-    size_t arena_want = 0;               // high-water mark incl. overflow blocks
+    size_t arena_live = 0;               // bytes handed out and not rewound in this call (arena + overflow)
+    size_t arena_want = 0;               // high-water mark of arena_live
     std::vector<void*> overflow;         // freed at the end of the call
     uint64_t* pinned = nullptr;          // 64 x u64 pinned host words for D2H scalars
     // pinned staging for hash parameters on their way to the device (grown on demand); calls end
@@ -184,6 +185,9 @@ void dev_trim();
 culsh_status arena_begin(culsh_ctx* ctx);                 // start of an API call
 culsh_status arena_alloc(culsh_ctx* ctx, size_t bytes, void** out);
 culsh_status arena_end(culsh_ctx* ctx);                   // syncs the stream, frees overflow
+struct ArenaMark { size_t off, live; };
+ArenaMark arena_mark(const culsh_ctx* ctx);
+void arena_rewind(culsh_ctx* ctx, const ArenaMark& mark);  // stream idle; frees what came after the mark
 template <typename T>
 inline culsh_status arena_alloc_t(culsh_ctx* ctx, size_t count, T** out) {
     void* p = nullptr;

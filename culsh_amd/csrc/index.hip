@@ -95,9 +95,13 @@ __global__ __launch_bounds__(IB_THREADS) void build_index_kernel(
     const uint64_t* __restrict__ tile_base, const uint64_t* __restrict__ n_buckets_dev,
     int32_t* __restrict__ bucket_candidate_offsets,
     uint32_t* __restrict__ bucket_keys, int32_t* __restrict__ table_bucket_offsets,
-    int32_t* __restrict__ item_to_bucket) {
+    int32_t* __restrict__ item_to_bucket, const uint32_t* __restrict__ sort_gave_up) {
     __shared__ uint64_t scratch[17];
     __shared__ uint16_t head_slot[IB_TILE];  // tile-local item numbers of the heads, ascending
+    // A sort that gave up leaves slots of keys and rows unwritten: the bucket count may then exceed
+    // the arrays sized for it and the rows are no valid addresses.  The flag is final by now (same
+    // stream); the host repeats the fit.
+    if (sort_gave_up && *sort_gave_up) return;
     const size_t tile_start = static_cast<size_t>(blockIdx.x) * IB_TILE;
     const size_t base = tile_start + threadIdx.x * IB_ITEMS;
     uint32_t flag[IB_ITEMS];
@@ -119,7 +123,8 @@ __global__ __launch_bounds__(IB_THREADS) void build_index_kernel(
         }
         if (item_to_bucket) {
             const size_t t = pos / n;
-            item_to_bucket[static_cast<size_t>(rows[pos]) * T + t] = bucket;  // fit.cuh:180-185
+            const uint32_t row = static_cast<uint32_t>(rows[pos]);
+            if (row < static_cast<uint32_t>(n)) item_to_bucket[static_cast<size_t>(row) * T + t] = bucket;  // fit.cuh:180-185
         }
     }
     __syncthreads();
@@ -273,8 +278,15 @@ culsh_status build_index_from_sorted(culsh_ctx* ctx, const uint32_t* sorted_keys
     if (enc == ENC_BITS && S < 31) B_bound = std::min<size_t>(N, static_cast<size_t>(T) << S);
     const bool deferred = B_bound * (8 + static_cast<size_t>(4) * W + S) <= (static_cast<size_t>(256) << 20);
     uint64_t n_buckets64 = 0;
+    uint32_t sort_gave_up = 0;
     if (!deferred) {
-        CULSH_TRY(read_back_u64(ctx, total_dev, 1, &n_buckets64));  // host sync (fit.cuh:332-337)
+        // host sync (fit.cuh:332-337); the sort's give-up flag comes along, before anything is sized
+        // by a count taken from keys that a failed sort left incomplete
+        CULSH_TRY(read_back_pair(ctx, total_dev, ctx->sort_err_dev, &n_buckets64, &sort_gave_up));
+        if (sort_gave_up) {
+            ctx->sort_err_dev = nullptr;
+            return CULSH_RETRY_UNCHAINED;
+        }
         B_bound = static_cast<size_t>(n_buckets64);
     }
     index->all_candidate_indices = rows_sorted_owned;
@@ -290,7 +302,8 @@ culsh_status build_index_from_sorted(culsh_ctx* ctx, const uint32_t* sorted_keys
     CULSH_HIP(dev_malloc(&index->all_bucket_signatures, std::max<size_t>(1, B_bound * S)));
     CULSH_LAUNCH(ctx, build_index_kernel, dim3(static_cast<unsigned>(tiles)), dim3(IB_THREADS), 0, ctx->stream,
                        sorted_keys, rows_sorted_owned, N, n, T, W, tile_base, total_dev, index->bucket_candidate_offsets,
-                       index->bucket_keys, index->table_bucket_offsets, item_to_bucket_opt);
+                       index->bucket_keys, index->table_bucket_offsets, item_to_bucket_opt,
+                       static_cast<const uint32_t*>(ctx->sort_err_dev));
     CULSH_LAUNCH_CHECK();
     CULSH_TRY(build_key_directory(ctx, index, B_bound));
     if (enc == ENC_PSC)
@@ -299,13 +312,9 @@ culsh_status build_index_from_sorted(culsh_ctx* ctx, const uint32_t* sorted_keys
         CULSH_TRY(launch_mh_keys_to_sig(ctx, index, B_bound, total_dev, index->all_bucket_signatures));
     else
         CULSH_TRY(launch_keys_to_sig(ctx, index->bucket_keys, B_bound, total_dev, S, enc, W, index->all_bucket_signatures));
-    // end-of-build read-back: the bucket count (unless fetched above) and the sort's give-up flag
-    uint32_t sort_gave_up = 0;
-    if (deferred) {
-        CULSH_TRY(read_back_pair(ctx, total_dev, ctx->sort_err_dev, &n_buckets64, &sort_gave_up));
-    } else if (ctx->sort_err_dev) {
-        CULSH_TRY(read_back_u32(ctx, ctx->sort_err_dev, 1, &sort_gave_up));
-    }
+    // end-of-build read-back: the bucket count and the sort's give-up flag (unless fetched above); the
+    // kernels launched since then have skipped their work if the flag was set
+    if (deferred) CULSH_TRY(read_back_pair(ctx, total_dev, ctx->sort_err_dev, &n_buckets64, &sort_gave_up));
     ctx->sort_err_dev = nullptr;
     if (sort_gave_up) return CULSH_RETRY_UNCHAINED;
     index->n_total_buckets = static_cast<int>(n_buckets64);

@@ -88,14 +88,19 @@ __global__ __launch_bounds__(256) void mh_hash_columns_kernel(const uint32_t* __
 // sorted_cols[c][r] = column of rank r; sorted_keys[c][r] = its byte-swapped hash
 __global__ __launch_bounds__(256) void mh_invert_kernel(const int32_t* __restrict__ sorted_cols,
                                                        const uint32_t* __restrict__ sorted_keys, size_t total, int d,
-                                                       uint32_t* __restrict__ rank, uint32_t* __restrict__ inv) {
+                                                       uint32_t* __restrict__ rank, uint32_t* __restrict__ inv,
+                                                       const uint32_t* __restrict__ sort_gave_up) {
     const size_t i = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
     if (i >= total) return;
+    // a column sort that gave up leaves slots unwritten: their columns are no valid addresses (the
+    // host reads the flag next and repeats the fit)
+    if (sort_gave_up && *sort_gave_up) return;
     const size_t c = i / d;
     const uint32_t r = static_cast<uint32_t>(i - c * d);
     // A multiplier that is 0 mod p gives every column the same value, hence the same rank (0); any
     // other multiplier gives d different values.
-    rank[c * d + static_cast<uint32_t>(sorted_cols[i])] = sorted_keys[i] == sorted_keys[c * d] ? 0u : r;
+    const uint32_t col = static_cast<uint32_t>(sorted_cols[i]);
+    if (col < static_cast<uint32_t>(d)) rank[c * d + col] = sorted_keys[i] == sorted_keys[c * d] ? 0u : r;
     inv[i] = __builtin_bswap32(sorted_keys[i]);
 }
 
@@ -332,7 +337,7 @@ culsh_status mh_build_codec(culsh_ctx* ctx, const int32_t* indices, size_t nnz, 
     CULSH_HIP(dev_malloc(&mc.inv, total * sizeof(uint32_t)));
     CULSH_HIP(dev_malloc(&mc.ainv, TH * sizeof(uint32_t)));
     CULSH_LAUNCH(ctx, mh_invert_kernel, dim3(div_up(total, 256)), dim3(256), 0, ctx->stream, cols, sorted, total, d,
-                 mc.rank, mc.inv);
+                 mc.rank, mc.inv, static_cast<const uint32_t*>(ctx->sort_err_dev));
     CULSH_LAUNCH_CHECK();
     CULSH_LAUNCH(ctx, mh_inverse_kernel, dim3(div_up(TH, 256)), dim3(256), 0, ctx->stream, ix->A, static_cast<int>(TH),
                  mc.ainv);

@@ -171,8 +171,10 @@ __global__ __launch_bounds__(256) void ps_keys_to_sig_kernel(const uint32_t* __r
                                                             const int32_t* __restrict__ table_bucket_offsets, int T,
                                                             int H, int bits, int rmax, int W, int use_lds,
                                                             const int32_t* __restrict__ inv,
-                                                            int32_t* __restrict__ sig) {
+                                                            int32_t* __restrict__ sig,
+                                                            const uint32_t* __restrict__ sort_gave_up) {
     extern __shared__ uint32_t ps_lds[];  // [PS_BPB] table ids, [PS_BPB][W] key words, then the value tables
+    if (sort_gave_up && *sort_gave_up) return;  // bucket keys of a failed sort may hold ranks beyond the tables
     uint32_t* tb = ps_lds;
     uint32_t* kw = ps_lds + PS_BPB;
     int32_t* lut = reinterpret_cast<int32_t*>(kw + PS_BPB * W);
@@ -333,7 +335,7 @@ culsh_status launch_ps_keys_to_sig(culsh_ctx* ctx, const culsh_index* ix, size_t
     CULSH_REQUIRE(lds <= 64 * 1024, CULSH_ERR_LIMIT, "key width too large for the signature restore kernel");
     CULSH_LAUNCH(ctx, ps_keys_to_sig_kernel, dim3(div_up(count, PS_BPB)), dim3(256), lds, ctx->stream, ix->bucket_keys,
                  count, count_dev, ix->table_bucket_offsets, ix->n_hash_tables, ix->n_hashes, pc.bits, pc.rmax,
-                 ix->key_w, use_lds, pc.inv, reinterpret_cast<int32_t*>(sig));
+                 ix->key_w, use_lds, pc.inv, reinterpret_cast<int32_t*>(sig), static_cast<const uint32_t*>(ctx->sort_err_dev));
     CULSH_LAUNCH_CHECK();
     return CULSH_OK;
 }

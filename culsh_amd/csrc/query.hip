@@ -41,8 +41,10 @@ __device__ __forceinline__ int key_dir_shift(uint32_t largest_word) {
 // largest first key word over the tables' last buckets (keys ascend inside a table), into dir[0].
 __global__ __launch_bounds__(256) void key_dir_init_kernel(const uint32_t* __restrict__ bucket_keys,
                                                           const int32_t* __restrict__ table_bucket_offsets, int T,
-                                                          int W, uint32_t* __restrict__ dir) {
+                                                          int W, uint32_t* __restrict__ dir,
+                                                          const uint32_t* __restrict__ sort_gave_up) {
     __shared__ uint32_t largest[4];
+    if (sort_gave_up && *sort_gave_up) return;  // keys and offsets of a failed sort are not to be trusted; the fit is repeated
     const int tid = threadIdx.x;
     uint32_t* entry = dir + 1 + static_cast<size_t>(blockIdx.x) * (KEY_DIR_SIZE + 1);
     for (int x = tid; x <= KEY_DIR_SIZE; x += 256) entry[x] = 0xFFFFFFFFu;
@@ -64,7 +66,9 @@ __global__ __launch_bounds__(256) void key_dir_init_kernel(const uint32_t* __res
 // smallest value at or behind it, the last one being the table's end.
 __global__ __launch_bounds__(256) void key_dir_mark_kernel(const uint32_t* __restrict__ bucket_keys,
                                                           const int32_t* __restrict__ table_bucket_offsets, int W,
-                                                          uint32_t* __restrict__ dir) {
+                                                          uint32_t* __restrict__ dir,
+                                                          const uint32_t* __restrict__ sort_gave_up) {
+    if (sort_gave_up && *sort_gave_up) return;
     const int t = blockIdx.y;
     const int shift = key_dir_shift(dir[0]);
     const int begin = table_bucket_offsets[t], end = table_bucket_offsets[t + 1];
@@ -76,9 +80,11 @@ __global__ __launch_bounds__(256) void key_dir_mark_kernel(const uint32_t* __res
 }
 
 __global__ __launch_bounds__(256) void key_dir_close_kernel(const int32_t* __restrict__ table_bucket_offsets,
-                                                           uint32_t* __restrict__ dir) {
+                                                           uint32_t* __restrict__ dir,
+                                                           const uint32_t* __restrict__ sort_gave_up) {
     constexpr int PER = KEY_DIR_SIZE / 256;  // entries per thread
     __shared__ uint32_t tail[256];
+    if (sort_gave_up && *sort_gave_up) return;
     const int t = blockIdx.x, tid = threadIdx.x;
     uint32_t* entry = dir + 1 + static_cast<size_t>(t) * (KEY_DIR_SIZE + 1);
     const uint32_t end = static_cast<uint32_t>(table_bucket_offsets[t + 1]);
@@ -714,16 +720,17 @@ culsh_status build_key_directory(culsh_ctx* ctx, culsh_index* index, size_t buck
     if (T > KEY_DIR_MAX_TABLES || index->key_w < 1) return CULSH_OK;
     const size_t words = 1 + static_cast<size_t>(T) * (KEY_DIR_SIZE + 1);
     CULSH_HIP(dev_malloc(&index->key_dir, words * sizeof(uint32_t)));
+    const uint32_t* gave_up = ctx->sort_err_dev;  // null outside a fit (loaded indices)
     CULSH_LAUNCH(ctx, key_dir_init_kernel, dim3(static_cast<unsigned>(T)), dim3(256), 0, ctx->stream,
-                 index->bucket_keys, index->table_bucket_offsets, T, index->key_w, index->key_dir);
+                 index->bucket_keys, index->table_bucket_offsets, T, index->key_w, index->key_dir, gave_up);
     CULSH_LAUNCH_CHECK();
     // about two buckets per thread for tables of even size; larger tables take more rounds
     const unsigned per_table = static_cast<unsigned>(std::max<size_t>(1, std::min<size_t>(4096, div_up(bucket_bound / T + 1, 512))));
     CULSH_LAUNCH(ctx, key_dir_mark_kernel, dim3(per_table, static_cast<unsigned>(T)), dim3(256), 0, ctx->stream,
-                 index->bucket_keys, index->table_bucket_offsets, index->key_w, index->key_dir);
+                 index->bucket_keys, index->table_bucket_offsets, index->key_w, index->key_dir, gave_up);
     CULSH_LAUNCH_CHECK();
     CULSH_LAUNCH(ctx, key_dir_close_kernel, dim3(static_cast<unsigned>(T)), dim3(256), 0, ctx->stream,
-                 index->table_bucket_offsets, index->key_dir);
+                 index->table_bucket_offsets, index->key_dir, gave_up);
     CULSH_LAUNCH_CHECK();
     return CULSH_OK;
 }

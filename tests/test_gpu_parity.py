@@ -162,6 +162,51 @@ def test_core_fit_index_sort_fallbacks(ctx, c_oracle, monkeypatch, knob):
         own.close()
 
 
+def test_fit_after_sort_gives_up_touches_nothing_it_should_not(c_oracle, monkeypatch):
+    """A give-up of the chained scan leaves sorted keys and rows incomplete.  The kernels queued behind
+    the sort must skip their work on seeing the flag (they would otherwise use stale rows as addresses
+    and write more buckets than the arrays sized for sign-bit keys hold), and the repeated fit must
+    give the oracle's result: RPLSH fit_query (row -> bucket map, bucket arrays sized by 2^H per table)
+    and a MinHash fit whose column sort and item sort both span several tiles."""
+    _announce("sort_give_up_fit_query_and_minhash")
+    monkeypatch.setenv("CULSH_SORT_SPIN_LIMIT", "0")
+    from abi import Ctx, assert_candidates_match, assert_index_matches
+
+    rng = np.random.default_rng(31)
+    n, d, T, H = 20000, 32, 4, 8                    # 3 tiles of 8192 one-word keys per table
+    X = rng.standard_normal((n, d)).astype(np.float32)
+    P = rng.standard_normal((T * H, d)).astype(np.float32)
+    own = Ctx(0)                                    # a give-up switches its context to unchained passes for good
+    try:
+        sig = own.rplsh_hash(X, P, T, H)
+        got = own.rplsh_fit_query(X, T, H, seed=1, P=P)
+        assert_candidates_match(got, c_oracle.fit_query(sig, H))
+    finally:
+        own.close()
+
+    n, dcols, T, H = 30000, 20000, 2, 2             # 15-bit rank codes: one key word, 4 tiles; 3 tiles of columns
+    indices, indptr = make_csr(rng, n, dcols, 6)
+    A, B = o.generate_hash_integers(5, T * H)
+    own = Ctx(0)
+    try:
+        ih = own.minhash_fit(indices, indptr, dcols, T, H, seed=5, A=A, B=B)
+        sig = c_oracle.minhash_hash(indices, indptr, A, B, T, H)
+        assert_index_matches(own.index_arrays(ih), c_oracle.fit_index_c(sig, H).to_numpy(n))
+        own.free_index(ih)
+    finally:
+        own.close()
+
+
+def test_fit_query_refuses_more_than_1024_tables_up_front(ctx):
+    """The query path handles up to 1024 tables; fit_query says so before it hashes or sorts anything."""
+    sig = np.zeros((1025, 4, 1), dtype=np.uint8)
+    with pytest.raises(RuntimeError, match="1024"):
+        ctx.core_fit_query(sig, 1)
+    X = np.zeros((4, 8), dtype=np.float32)
+    with pytest.raises(RuntimeError, match="1024"):
+        ctx.rplsh_fit_query(X, 1025, 1)
+
+
 def test_core_fit_index_single_bucket_per_table(ctx):
     """All signatures equal: no radix pass runs and rows stay in identity order."""
     sig = np.full((3, 1000, 4), 1, dtype=np.uint8)
@@ -447,6 +492,77 @@ def test_core_fit_query(ctx, kind):
     again = ctx.core_query_index(sig, ih)
     for k in ("indices", "offsets", "counts"):
         np.testing.assert_array_equal(got[k], again[k])
+    ctx.free_index(ih)
+
+
+def test_candidates_merge_and_handles(ctx):
+    """Candidates::merge (core/candidates.cuh:139-197) at the C ABI: parts of one query set, merged one
+    after the other, equal the unbatched result; an empty accumulator takes the other object as it is
+    (:144-148), an empty other changes nothing (:140-142), a part without any candidate still adds its
+    queries.  Also the device-pointer, stream and synchronize exports."""
+    from abi import assert_candidates_match
+    from culsh_amd import _lib as L
+
+    rng = np.random.default_rng(41)
+    T, n, H, nq = 4, 3000, 3, 90
+    sig = random_sigs(rng, T, n, H, "rplsh")
+    qsig = random_sigs(rng, T, nq, H, "rplsh")
+    ih, _ = ctx.core_fit_index(sig, H)
+    exp_ix = o.fit_index(sig, H)
+    whole = o.query_index(qsig, exp_ix)
+
+    # three parts, chained: NULL accumulator first, then two appends
+    cuts = [0, 25, 60, nq]
+    acc = None
+    for a, b in zip(cuts[:-1], cuts[1:]):
+        part = ctx.core_query_index(np.ascontiguousarray(qsig[:, a:b]), ih, as_handle=True)
+        acc = ctx.candidates_merge(acc, part)
+    meta = ctx.candidates_meta(acc)
+    assert meta["n_queries"] == nq and meta["n_total_candidates"] == whole.n_total_candidates
+    # device pointers of the merged object hold the same arrays the copy calls return
+    import torch
+
+    def view(address, count, typestr):
+        class Raw:
+            __cuda_array_interface__ = {"shape": (count,), "typestr": typestr, "data": (address, False), "version": 2}
+        return torch.as_tensor(Raw(), device="cuda").cpu().numpy()
+
+    pi = ctx.candidates_device_ptr(acc, L.ARR_QUERY_INDICES)
+    pc = ctx.candidates_device_ptr(acc, L.ARR_QUERY_COUNTS)
+    po = ctx.candidates_device_ptr(acc, L.ARR_QUERY_OFFSETS)
+    assert pi != 0 and pc != 0 and po != 0
+    assert ctx.stream() != 0
+    ctx.synchronize()
+    np.testing.assert_array_equal(view(pi, whole.n_total_candidates, "<i4"), whole.query_candidate_indices)
+    np.testing.assert_array_equal(view(pc, nq, "<i8").view(np.uint64), whole.query_candidate_counts)
+    np.testing.assert_array_equal(view(po, nq + 1, "<i8").view(np.uint64), whole.query_candidate_offsets)
+    assert_candidates_match(ctx.candidates_arrays(acc), whole)
+
+    # empty accumulator object (no arrays) takes `other`; empty other leaves the accumulator as it is
+    queries_without_bucket = np.full((T, 5, H), 7, dtype=np.uint8)   # byte 7 never occurs in 0/1 signatures
+    none = ctx.core_query_index(queries_without_bucket, ih, as_handle=True)
+    m = ctx.candidates_meta(none)
+    assert m["n_queries"] == 5 and m["n_total_candidates"] == 0 and not m["is_empty"]
+    assert ctx.candidates_device_ptr(none, L.ARR_QUERY_INDICES) == 0
+    part = ctx.core_query_index(np.ascontiguousarray(qsig[:, :25]), ih, as_handle=True)
+    acc = ctx.candidates_merge(none, part)       # a part with no candidate in front: offsets start with zeros
+    got = ctx.candidates_arrays(acc)
+    first = o.query_index(np.ascontiguousarray(qsig[:, :25]), exp_ix)
+    assert got["n_queries"] == 30 and got["n_total_candidates"] == first.n_total_candidates
+    np.testing.assert_array_equal(got["counts"], np.concatenate([np.zeros(5, np.uint64), first.query_candidate_counts]))
+    np.testing.assert_array_equal(got["offsets"], np.concatenate([np.zeros(5, np.uint64), first.query_candidate_offsets]))
+    np.testing.assert_array_equal(got["indices"], first.query_candidate_indices)
+    # ... and behind: the oracle's merge says what comes out
+    a = ctx.core_query_index(np.ascontiguousarray(qsig[:, :25]), ih, as_handle=True)
+    b = ctx.core_query_index(queries_without_bucket, ih, as_handle=True)
+    acc = ctx.candidates_merge(a, b)
+    exp = o.merge(first, o.query_index(queries_without_bucket, exp_ix))
+    assert_candidates_match(ctx.candidates_arrays(acc), exp)
+    # NULL other: nothing happens, the accumulator handle stays valid
+    a = ctx.core_query_index(np.ascontiguousarray(qsig[:, :25]), ih, as_handle=True)
+    same = ctx.candidates_merge(a, None)
+    assert same.value == a.value
+    assert_candidates_match(ctx.candidates_arrays(same), first)
     ctx.free_index(ih)
 
 
