@@ -91,6 +91,7 @@ PROTOTYPES = {
     "culsh_core_fit_index": [_P, _P, _I, _I, _I, _I, _P, _PP],
     "culsh_core_query_index": [_P, _P, _I, _I, _P, _PP],
     "culsh_core_find_matching_buckets": [_P, _P, _I, _I, _P, _P],
+    "culsh_core_find_matching_buckets_static": [_P, _P, _I, _I, _P, _P],
     "culsh_core_query_from_matched_buckets": [_P, _P, _I, _P, _PP],
     "culsh_core_fit_query": [_P, _P, _I, _I, _I, _I, _PP],
     "culsh_index_get_meta": [_P, C.POINTER(IndexMeta)],

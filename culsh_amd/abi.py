@@ -164,12 +164,17 @@ class Ctx:
         L.check(self.lib.culsh_core_query_index(self.h, ptr(dsig), nq, S, ih, C.byref(ch)))
         return ch if as_handle else self.candidates_arrays(ch)
 
-    def core_find_matching_buckets(self, qsig: np.ndarray, ih) -> np.ndarray:
+    def core_find_matching_buckets(self, qsig: np.ndarray, ih, static: bool = False) -> np.ndarray:
+        """`static`: through the entry point that allocates nothing (asynchronous: synchronised here)."""
         b, T, nq, S = self._sig_bytes(qsig)
         t = torch()
         dsig = dev(b.reshape(-1))
         m = t.empty(nq * T, dtype=t.int32, device="cuda")
-        L.check(self.lib.culsh_core_find_matching_buckets(self.h, ptr(dsig), nq, S, ih, ptr(m)))
+        if static:
+            L.check(self.lib.culsh_core_find_matching_buckets_static(self.h, ptr(dsig), nq, S, ih, ptr(m)))
+            self.synchronize()
+        else:
+            L.check(self.lib.culsh_core_find_matching_buckets(self.h, ptr(dsig), nq, S, ih, ptr(m)))
         return m.cpu().numpy()
 
     def core_query_from_matched(self, matched: np.ndarray, nq: int, ih):

@@ -6,6 +6,7 @@
 #include <cmath>
 #include <cstring>
 #include <memory>
+#include <mutex>
 #include <new>
 #include <thread>
 #include <vector>
@@ -719,6 +720,26 @@ extern "C" {
 const char* culsh_last_error(void) { return g_last_error.c_str(); }
 const char* culsh_version(void) { return "culsh_amd 0.1.0 (gfx950)"; }
 
+// ---- the entry point that allocates nothing
+// Key words of the queries on their way to the lookup kernel live in this array instead of the
+// context's arena.  Every device the library runs on holds its own copy at its own address; the
+// array's name is only a host-side handle of the symbol, so the address is asked for once per device
+// (culsh_ctx_create, with that device current) and kept.
+static __device__ __align__(256) uint32_t g_static_scratch[CULSH_STATIC_SCRATCH_WORDS];
+static std::mutex g_static_scratch_mutex;
+static uint32_t* g_static_scratch_ptr[64] = {};
+
+static culsh_status static_scratch_init(int device) {  // `device` is current
+    if (device < 0 || device >= 64) return CULSH_OK;   // such a device has no static entry point
+    std::lock_guard<std::mutex> lock(g_static_scratch_mutex);
+    if (g_static_scratch_ptr[device]) return CULSH_OK;
+    void* p = nullptr;
+    CULSH_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(g_static_scratch)));
+    CULSH_REQUIRE(p != nullptr, CULSH_ERR_HIP, "hipGetSymbolAddress returned a null address");
+    g_static_scratch_ptr[device] = static_cast<uint32_t*>(p);
+    return CULSH_OK;
+}
+
 culsh_status culsh_ctx_create(int device, culsh_ctx** out) {
     CULSH_REQUIRE(out, CULSH_ERR_INVALID, "null argument");
     *out = nullptr;
@@ -749,6 +770,12 @@ culsh_status culsh_ctx_create(int device, culsh_ctx** out) {
         return CULSH_ERR_NOMEM;
     }
     ctx->pinned = static_cast<uint64_t*>(pinned);
+    const culsh_status scratch_status = static_scratch_init(device);
+    if (scratch_status != CULSH_OK) {
+        (void)hipHostFree(pinned);
+        (void)hipStreamDestroy(ctx->stream);
+        return scratch_status;
+    }
     *out = ctx.release();
     return CULSH_OK;
 }
@@ -1033,6 +1060,29 @@ culsh_status culsh_core_find_matching_buckets(culsh_ctx* ctx, const void* Q_sig,
     CULSH_TRY(sig_query_keys(ctx, Q_sig, nq, S, ix, &keys));
     CULSH_TRY(launch_find_matching_buckets(ctx, keys, nq, ix, matched));
     return arena_end(ctx);
+}
+
+// ---- the entry point that allocates nothing (workspace: g_static_scratch, set up in culsh_ctx_create)
+culsh_status culsh_core_find_matching_buckets_static(culsh_ctx* ctx, const void* Q_sig, int nq, int S,
+                                                     const culsh_index* ix, int32_t* matched) {
+    CULSH_REQUIRE(ctx && Q_sig && ix && matched, CULSH_ERR_INVALID, "null argument");
+    CULSH_REQUIRE(nq > 0, CULSH_ERR_INVALID, "n_queries must be positive");
+    CULSH_REQUIRE(ix->device == ctx->device, CULSH_ERR_INVALID, "index and context are on different devices");
+    const size_t words = static_cast<size_t>(nq) * ix->n_hash_tables * ix->key_w;
+    CULSH_REQUIRE(words <= CULSH_STATIC_SCRATCH_WORDS, CULSH_ERR_LIMIT,
+                  "find_matching_buckets_static: n_queries * n_hash_tables * key words = %zu exceeds the static "
+                  "workspace of %zu words; use culsh_core_find_matching_buckets",
+                  words, static_cast<size_t>(CULSH_STATIC_SCRATCH_WORDS));
+    uint32_t* keys = (ctx->device >= 0 && ctx->device < 64) ? g_static_scratch_ptr[ctx->device] : nullptr;
+    CULSH_REQUIRE(keys != nullptr, CULSH_ERR_INTERNAL, "static workspace of device %d was not set up", ctx->device);
+    CULSH_HIP(hipSetDevice(ctx->device));
+    // no event objects either: launches of this call are not timed
+    const bool profiling = ctx->profiling;
+    ctx->profiling = false;
+    culsh_status st = sig_query_keys_into(ctx, Q_sig, nq, S, ix, keys);
+    if (st == CULSH_OK) st = launch_find_matching_buckets(ctx, keys, nq, ix, matched);
+    ctx->profiling = profiling;
+    return st;
 }
 
 culsh_status culsh_core_query_index(culsh_ctx* ctx, const void* Q_sig, int nq, int S, const culsh_index* ix,

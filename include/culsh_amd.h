@@ -174,6 +174,20 @@ culsh_status culsh_core_fit_index(culsh_ctx*, const void* X_sig_dev, int n_sampl
 culsh_status culsh_core_query_index(culsh_ctx*, const void* Q_sig_dev, int n_queries, int sig_nbytes, const culsh_index*, culsh_candidates** out);
 /* find_matching_buckets_kernel, core/query.cuh:72-101: int32 matched_dev[n_queries * T]. */
 culsh_status culsh_core_find_matching_buckets(culsh_ctx*, const void* Q_sig_dev, int n_queries, int sig_nbytes, const culsh_index*, int32_t* matched_dev);
+/* The same lookup for callers that cannot allocate (code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc).  No counterpart in the reference.  The key words of the queries,
+ * which culsh_core_find_matching_buckets keeps in the context's scratch arena, live in a workspace that
+ * is part of the library's device image (CULSH_STATIC_SCRATCH_WORDS 32-bit words per GPU, held until the
+ * process ends); the call makes no hipMalloc / hipFree, creates no events and does not wait for the
+ * stream: it enqueues its kernels on the context's stream and returns, and `matched_dev` is complete
+ * after culsh_ctx_synchronize (or any other call on the context, all of which end with the stream
+ * idle).  n_queries * n_hash_tables * key words per signature beyond the workspace is refused with
+ * CULSH_ERR_LIMIT (key words: ceil(n_hashes / 32) for RPLSH indices, at most ceil(sig_nbytes / 4)
+ * otherwise).  All calls on one GPU share that GPU's workspace, which keeps the last call's contents
+ * (every call overwrites the part it reads): calls on one context follow each other on its stream, but
+ * calls of two contexts that overlap in time on one GPU race. */
+#define CULSH_STATIC_SCRATCH_WORDS (1u << 20) /* 4 MiB */
+culsh_status culsh_core_find_matching_buckets_static(culsh_ctx*, const void* Q_sig_dev, int n_queries, int sig_nbytes, const culsh_index*, int32_t* matched_dev);
 /* core::detail::query_from_matched_buckets, core/query.cuh:290-478. */
 culsh_status culsh_core_query_from_matched_buckets(culsh_ctx*, const int32_t* matched_dev, int n_queries, const culsh_index*, culsh_candidates** out);
 /* core::detail::fit_query, core/fit_query.cuh:30-55. */
