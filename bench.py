@@ -164,11 +164,49 @@ def main() -> int:
         roofline = {"kernel": proj_name, "bound": "mfma", "achieved": round(achieved, 3),
                     "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s",
                     "frac": round(achieved / PEAK_FP32_MFMA_TFLOPS, 4),
-                    # HBM bytes of the fit launch at the default size: rocprofv3 FETCH_SIZE x 2.0
-                    # (490.4 MiB) + WRITE_SIZE x 1.0 (122.1 MiB), scale factors from a 1 GiB copy
+                    # HBM bytes of the fit launch: not measured by this run (counters need rocprofv3); the
+                    # figure is the one on record for this shape in profiles/hbm_traffic_rplsh_1Mx128_T32_H16.txt
+                    # (FETCH_SIZE x 2.0 = 490.4 MiB + WRITE_SIZE x 1.0 = 122.1 MiB, factors from a 1 GiB copy)
                     "traffic": 642_300_000 if (n, nq) == (1_000_000, 10_000) else None,
+                    "traffic_source": ("profiles/hbm_traffic_rplsh_1Mx128_T32_H16.txt (rocprofv3 --pmc, an earlier "
+                                       "run of this command)" if (n, nq) == (1_000_000, 10_000) else None),
                     "work": "2*(n+q)*d*T*H flop per step over the fit and query launches",
                     "dominant_kernel_by_time": dominant}
+
+    # ---- HBM-bound kernels: algorithmic bytes of this run / HIP-event time of this run
+    # (events around every kernel: the untimed detail steps).  N = n*T items, B buckets, R raw and U unique
+    # candidates of this run's query, all read from this run's own index and result.
+    ih = fit()
+    ixa = ctx.index_arrays(ih)
+    qsig_gpu = ctx.rplsh_hash(Q, P, T, H)
+    matched = ctx.core_find_matching_buckets(qsig_gpu, ih)
+    bco = ixa["bucket_candidate_offsets"].astype(np.int64)
+    hit = matched >= 0
+    R = int((bco[matched[hit] + 1] - bco[matched[hit]]).sum())
+    B = int(ixa["n_total_buckets"])
+    lib.culsh_index_free(ih)
+    N, U = n * T, n_unique
+    W = (H + 31) // 32                       # key words per item (sign bits)
+    n_passes = (H + 7) // 8                  # 8-bit radix passes over the varying key bits
+    hbm_work = {
+        # pass 1 reads keys (rows are the identity) and writes keys + rows; later passes move both
+        "radix_scatter_kernel": (4 * W * N + (4 * W + 4) * N) + (n_passes - 1) * 2 * (4 * W + 4) * N,
+        "radix_totals_kernel": 4 * W * N,                                   # one read of the keys for all passes
+        "count_heads_kernel": 4 * W * N,                                    # sorted keys
+        "build_index_kernel": 4 * W * N + B * (4 + 4 * W),                  # sorted keys; bucket offsets + bucket keys
+        "bit_keys_to_sig_kernel": B * (4 * W + H),                          # bucket keys -> signature bytes
+        "dedup_kernel": 4 * R + 4 * U + 16 * nq,                            # candidate rows read, lists + counts/offsets written
+    }
+    roofline_kernels = []
+    for short, nbytes in hbm_work.items():
+        names = [k for k in kernels_all if short in k]
+        if not names:
+            continue
+        ms = sum(kernels_all[k] for k in names)
+        achieved = nbytes / (ms * 1e-3) / 1e9
+        roofline_kernels.append({"kernel": short, "bound": "hbm", "bytes": int(nbytes), "ms": round(ms, 4),
+                                 "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                                 "frac": round(achieved / PEAK_HBM_GBS, 4)})
 
     # ---- CPU baseline + parity on this run's own results
     cpu = None
@@ -186,8 +224,9 @@ def main() -> int:
         t2 = time.perf_counter()
         cpu_qsig = co.rplsh_hash(Q, P, T, H)
         t3 = time.perf_counter()
-        cpu_U, cpu_R = co.query_index_c(qsig, cix, keep=False)
+        cpu_c = co.query_index_c(qsig, cix, keep=True)
         t4 = time.perf_counter()
+        cpu_U, cpu_R = int(cpu_c.n_total_candidates), int(cpu_c.n_raw_candidates)
         cpu_fit_s = (t1 - t0) + (t2 - t1)
         cpu_query_s = (t3 - t2) + (t4 - t3)
         # parity: bucket table bit-exact given identical signatures; candidate totals equal
@@ -201,8 +240,14 @@ def main() -> int:
         cand = ctx.candidates_arrays(ch)
         lib.culsh_index_free(ih)
         mism = float(np.mean(cpu_sig != sig))
+        counts_ok = bool(np.array_equal(cand["counts"], cpu_c.query_candidate_counts) and
+                         np.array_equal(cand["offsets"], cpu_c.query_candidate_offsets))
+        lists_ok = bool(counts_ok and np.array_equal(cand["indices"], cpu_c.query_candidate_indices))
         parity = {"bucket_tables_bit_exact": bool(table_ok),
                   "unique_candidates_equal": bool(cand["n_total_candidates"] == cpu_U),
+                  "per_query_counts_and_offsets_equal": counts_ok,
+                  "candidate_lists_bit_exact": lists_ok,
+                  "candidate_lists_compared": int(nq),
                   "hash_bit_mismatch_vs_cpu_float": mism,
                   "raw_candidates": cpu_R, "unique_candidates": cpu_U,
                   "n_buckets": int(exp.n_total_buckets)}
@@ -211,7 +256,7 @@ def main() -> int:
                "sample": f"full workload once: fit of {n}x{d} ({cpu_fit_s:.2f} s), "
                          f"query of {nq} ({cpu_query_s:.2f} s)",
                "query_qps": round(nq / cpu_query_s, 1)}
-        if not (table_ok and parity["unique_candidates_equal"]):
+        if not (table_ok and parity["unique_candidates_equal"] and counts_ok and lists_ok):
             print("bench.py: PARITY FAILURE " + json.dumps(parity), file=sys.stderr)
             return 1
 
@@ -225,7 +270,10 @@ def main() -> int:
                    "n_samples": n, "n_features": d, "n_queries": nq, "n_hash_tables": T, "n_hashes": H},
         "fit_ms": round(fit_ms, 4), "query_ms": round(query_ms, 4),
         "query": {"value": round(query_qps, 1), "unit": "queries/s", "unique_candidates": n_unique},
-        "roofline": roofline, "cpu_baseline": cpu, "parity": parity,
+        "roofline": roofline, "roofline_kernels": roofline_kernels,
+        "roofline_kernels_note": "algorithmic HBM bytes of this run (N items, B buckets, R raw and U unique candidates "
+                                 f"= {N}, {B}, {R}, {U}) over the HIP-event time of this run's untimed detail steps",
+        "cpu_baseline": cpu, "parity": parity,
         "kernels_ms_per_step": {k: round(v, 4) for k, v in sorted(kernels_all.items())},
         "kernels_ms_per_step_note": "from extra untimed steps with HIP events around every kernel; the timed "
                                     "steps carry events around the projection launches only",

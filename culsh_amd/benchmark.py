@@ -92,21 +92,45 @@ def _mixture(torch, n, d, nq, g):
 
 
 def _zipf_sets(torch, n, d, nq, g):
-    """CSR rows of distinct column ids: Poisson(50) draws per row (at least one) from a Zipf(1.1) law
-    over d columns, duplicates inside a row removed."""
+    """CSR rows of distinct column ids: a row holds Poisson(50) columns (at least one), drawn one after the
+    other from a Zipf(1.1) law over d columns, a column that the row already holds being drawn again (so the
+    number of non-zeros is the Poisson draw itself, without duplicates)."""
     p = 1.0 / torch.arange(1, d + 1, device="cuda", dtype=torch.float64) ** 1.1
     cdf = torch.cumsum(p, 0) / p.sum()
+    block = 100_000  # rows drawn at a time
+
+    def draw_block(count):
+        k = torch.poisson(torch.full((count,), 50.0, device="cuda"), generator=g).clamp_(min=1, max=d).long()
+        m = 256  # draws per row; doubled until every row has seen enough distinct columns
+        while True:
+            cols = torch.searchsorted(cdf, torch.rand((count, m), device="cuda", generator=g, dtype=torch.float64))
+            cols.clamp_(max=d - 1)
+            # first occurrence of every column in draw order: sort (column, draw) pairs by column
+            key, _ = torch.sort(cols * m + torch.arange(m, device="cuda"), dim=1)
+            col, at = key // m, key % m
+            first = torch.ones_like(col, dtype=torch.bool)
+            first[:, 1:] = col[:, 1:] != col[:, :-1]
+            if bool((first.sum(1) >= k).all()):
+                break
+            m *= 2
+        # the k earliest first occurrences of a row are its columns
+        when = torch.where(first, at, torch.full_like(at, m))
+        when_sorted, perm = torch.sort(when, dim=1)
+        keep = torch.arange(m, device="cuda")[None, :] < k[:, None]
+        chosen = torch.where(keep, torch.gather(col, 1, perm), torch.full_like(col, d))
+        chosen, _ = torch.sort(chosen, dim=1)  # ascending columns first, the unused slots (d) behind them
+        return chosen[keep], k  # row-major: rows in order, columns ascending inside a row
 
     def rows(count):
-        nnz = torch.poisson(torch.full((count,), 50.0, device="cuda"), generator=g).clamp_(min=1).long()
-        owner = torch.repeat_interleave(torch.arange(count, device="cuda"), nnz)
-        cols = torch.searchsorted(cdf, torch.rand(int(nnz.sum()), device="cuda", generator=g, dtype=torch.float64))
-        cols.clamp_(max=d - 1)
-        pairs = torch.unique(owner * d + cols)  # sorted: rows ascending, columns ascending inside a row
-        owner, cols = pairs // d, pairs % d
+        cols, nnz = [], []
+        for start in range(0, count, block):
+            c, k = draw_block(min(block, count - start))
+            cols.append(c.to(torch.int32))
+            nnz.append(k)
+        nnz = torch.cat(nnz)
         indptr = torch.zeros(count + 1, device="cuda", dtype=torch.int64)
-        indptr[1:] = torch.cumsum(torch.bincount(owner, minlength=count), 0)
-        return DeviceCSR(cols.to(torch.int32), indptr.to(torch.int32), (count, d))
+        indptr[1:] = torch.cumsum(nnz, 0)
+        return DeviceCSR(torch.cat(cols), indptr.to(torch.int32), (count, d))
 
     return rows(n), rows(nq)
 

@@ -896,9 +896,16 @@ culsh_status query_from_spans(culsh_ctx* ctx, const int2* spans, const unsigned 
         a.out = lists;
         a.err = err;
         a.capacity = cap;
-        const void* kernel = several ? reinterpret_cast<const void*>(dedup_kernel<DD_FUSED_PASSES>)
-                                     : reinterpret_cast<const void*>(dedup_kernel<DD_FUSED>);
-        CULSH_HIP(hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes)));
+        {   // more LDS than a launch may ask for by default: allowed once per kernel and device, not per call
+            static bool allowed[2][64] = {};
+            bool& done = allowed[several ? 1 : 0][ctx->device & 63];
+            if (!done) {
+                const void* kernel = several ? reinterpret_cast<const void*>(dedup_kernel<DD_FUSED_PASSES>)
+                                             : reinterpret_cast<const void*>(dedup_kernel<DD_FUSED>);
+                CULSH_HIP(hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, ctx->lds_max));
+                done = true;
+            }
+        }
         // as many workgroups as fit on the device at once (LDS and 2048 threads per CU bound it)
         const int per_cu = static_cast<int>(std::max<size_t>(1, std::min<size_t>(2, static_cast<size_t>(ctx->lds_max) / lds_bytes)));
         const int resident = std::max(1, ctx->n_cus * per_cu);
@@ -962,10 +969,14 @@ culsh_status query_from_spans(culsh_ctx* ctx, const int2* spans, const unsigned 
         break;
     }
     if (!fused) {
-        CULSH_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(dedup_kernel<DD_COUNT>),
-                                      hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes)));
-        CULSH_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(dedup_kernel<DD_EMIT>),
-                                      hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes)));
+        static bool allowed_two_launch[64] = {};
+        if (!allowed_two_launch[ctx->device & 63]) {
+            CULSH_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(dedup_kernel<DD_COUNT>),
+                                          hipFuncAttributeMaxDynamicSharedMemorySize, ctx->lds_max));
+            CULSH_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(dedup_kernel<DD_EMIT>),
+                                          hipFuncAttributeMaxDynamicSharedMemorySize, ctx->lds_max));
+            allowed_two_launch[ctx->device & 63] = true;
+        }
         CULSH_LAUNCH(ctx, dedup_kernel<DD_COUNT>, dim3(n_queries), dim3(DD_THREADS), lds_bytes, ctx->stream, a);
         CULSH_LAUNCH_CHECK();
         CULSH_TRY(exclusive_scan_u64(ctx, out->query_candidate_counts, out->query_candidate_offsets, n_queries));

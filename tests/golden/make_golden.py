@@ -63,6 +63,7 @@ def pslsh():
     out = dict(X=X, Q=Q, P=P, b=b, T=T, H=H, window=w, sig=sig, qsig=qsig)
     out.update(index_dict("ix_", ix))
     out.update(cand_dict("q_", o.query_index(qsig, ix)))
+    out.update(cand_dict("fq_", o.fit_query(sig, H)))
     np.savez_compressed(os.path.join(HERE, "pslsh_small.npz"), **out)
 
 
@@ -85,6 +86,7 @@ def minhash():
                sig=sig, qsig=qsig)
     out.update(index_dict("ix_", ix))
     out.update(cand_dict("q_", o.query_index(qsig, ix)))
+    out.update(cand_dict("fq_", o.fit_query(sig, H)))
     np.savez_compressed(os.path.join(HERE, "minhash_small.npz"), **out)
 
 

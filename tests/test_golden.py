@@ -88,9 +88,13 @@ def test_pslsh_fixture_matches_oracle_and_brute_force(c_oracle):
     ix = o.fit_index(g["sig"], H)
     check_index(g, ix)
     check_cands(g, "q_", o.query_index(g["qsig"], ix))
+    check_cands(g, "fq_", o.fit_query(g["sig"], H))
     bi, bc, bo = brute_force_candidates(g["sig"], g["qsig"])
     np.testing.assert_array_equal(bi, g["q_indices"])
     np.testing.assert_array_equal(bo, g["q_offsets"])
+    bi, bc, bo = brute_force_candidates(g["sig"], g["sig"])
+    np.testing.assert_array_equal(bi, g["fq_indices"])
+    np.testing.assert_array_equal(bo, g["fq_offsets"])
 
 
 def test_minhash_fixture_matches_oracle_and_brute_force(c_oracle):
@@ -111,9 +115,13 @@ def test_minhash_fixture_matches_oracle_and_brute_force(c_oracle):
     ix = o.fit_index(g["sig"], H)
     check_index(g, ix)
     check_cands(g, "q_", o.query_index(g["qsig"], ix))
+    check_cands(g, "fq_", o.fit_query(g["sig"], H))
     bi, bc, bo = brute_force_candidates(g["sig"], g["qsig"])
     np.testing.assert_array_equal(bi, g["q_indices"])
     np.testing.assert_array_equal(bo, g["q_offsets"])
+    bi, bc, bo = brute_force_candidates(g["sig"], g["sig"])
+    np.testing.assert_array_equal(bi, g["fq_indices"])
+    np.testing.assert_array_equal(bo, g["fq_offsets"])
 
 
 # ------------------------------------------------------------------------------- GPU
@@ -160,7 +168,9 @@ def test_gpu_pslsh_reproduces_fixture(ctx):
     ih = ctx.pslsh_fit(g["X"], T, H, w, P=g["P"], b=g["b"])
     gpu_index_equals(ctx, ih, g)
     gpu_cands_equal(ctx.pslsh_query(g["Q"], ih), g, "q_")
+    gpu_cands_equal(ctx.pslsh_query(g["Q"], ih, batch_size=9), g, "q_")
     ctx.free_index(ih)
+    gpu_cands_equal(ctx.pslsh_fit_query(g["X"], T, H, w, P=g["P"], b=g["b"]), g, "fq_")
 
 
 @pytest.mark.gpu
@@ -173,3 +183,4 @@ def test_gpu_minhash_reproduces_fixture(ctx):
     gpu_index_equals(ctx, ih, g)
     gpu_cands_equal(ctx.minhash_query(g["qcsr_indices"], g["qcsr_indptr"], ih), g, "q_")
     ctx.free_index(ih)
+    gpu_cands_equal(ctx.minhash_fit_query(g["x_indices"], g["x_indptr"], d, T, H, A=g["A"], B=g["B"]), g, "fq_")

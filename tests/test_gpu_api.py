@@ -329,3 +329,31 @@ def test_minhash_save_load_and_fit_query(tmp_path):
     X64.indices = X64.indices.astype(np.int64)
     with pytest.raises(ValueError, match="requires int32 indices"):
         lsh.fit(X64)
+
+
+# ---------------------------------------------------------------- the reference's import name
+def test_reference_import_name_runs_the_reference_usage(tmp_path):
+    """A caller written against rishic3/cuLSH (README usage; python/tests/test_rplsh.py:145-174) runs
+    unchanged through `import culsh`: fit, query, fit_query == fit + query, save / load."""
+    from culsh import RPLSH, RPLSHModel
+    from culsh._culsh_core import Candidates
+
+    X = dense(1500, 48, np.float32, seed=3)
+    Q = X[:60]
+    lsh = RPLSH(n_hash_tables=8, n_hashes=6, seed=5)
+    model = lsh.fit(X)
+    assert isinstance(model, RPLSHModel)
+    cand = model.query(Q)
+    assert isinstance(cand, Candidates)
+    both = RPLSH(n_hash_tables=8, n_hashes=6, seed=5).fit_query(X)
+    again = model.query(X)
+    np.testing.assert_array_equal(both.get_indices(), again.get_indices())
+    np.testing.assert_array_equal(both.get_offsets(), again.get_offsets())
+    path = os.path.join(tmp_path, "model.npz")
+    model.save(path)
+    loaded = RPLSHModel.load(path)
+    np.testing.assert_array_equal(loaded.query(Q).get_indices(), cand.get_indices())
+    # every query finds itself
+    off = cand.get_offsets().astype(np.int64)
+    idx = cand.get_indices()
+    assert all(q in idx[off[q]:off[q + 1]] for q in range(len(Q)))

@@ -849,6 +849,129 @@ def test_full_size_invariants(ctx):
     ctx.free_index(ih)
 
 
+def _index_properties(ix, n, T, S):
+    """Properties of any correct index (core/fit.cuh:222-374): offsets with their terminators, every table a
+    permutation of the rows, rows ascending inside a bucket, bucket signatures strictly ascending in byte
+    order inside a table."""
+    N = n * T
+    tbo, bco = ix["table_bucket_offsets"].astype(np.int64), ix["bucket_candidate_offsets"].astype(np.int64)
+    B = int(ix["n_total_buckets"])
+    cand = ix["all_candidate_indices"]
+    assert ix["sig_nbytes"] == S and ix["n_total_candidates"] == N
+    assert tbo[0] == 0 and tbo[-1] == B and np.all(np.diff(tbo) > 0)
+    assert bco[0] == 0 and bco[-1] == N and np.all(np.diff(bco) > 0)
+    assert np.all(bco[tbo[:-1]] == np.arange(T) * n)            # a table's first bucket starts its segment
+    for t in range(T):
+        assert np.array_equal(np.bincount(cand[t * n:(t + 1) * n], minlength=n), np.ones(n, dtype=np.int64))
+    descents = np.flatnonzero(np.diff(cand.astype(np.int64)) < 0) + 1
+    assert np.all(np.isin(descents, bco))
+    # byte-lexicographic order = numeric order of the big-endian words of a signature
+    assert S % 8 == 0
+    words = ix["all_bucket_signatures"].reshape(B, S).view(">u8").astype(np.uint64)   # [B][S/8]
+    differs = words[1:] != words[:-1]
+    first = np.argmax(differs, axis=1)
+    rows_idx = np.arange(B - 1)
+    ascending = differs.any(axis=1) & (words[1:][rows_idx, first] > words[:-1][rows_idx, first])
+    ascending[tbo[1:-1] - 1] = True                              # table boundaries may descend
+    assert np.all(ascending)
+
+
+def _candidate_properties(got, n):
+    off, idx = got["offsets"].astype(np.int64), got["indices"]
+    assert off[0] == 0 and off[-1] == len(idx) and np.all(np.diff(off) >= 0)
+    assert np.array_equal(np.diff(off), got["counts"].astype(np.int64))
+    if len(idx):
+        inside = np.ones(len(idx), dtype=bool)
+        inside[off[1:-1][off[1:-1] < len(idx)]] = False          # first element of the next query
+        assert np.all((np.diff(idx.astype(np.int64)) > 0) | ~inside[1:])   # ascending and duplicate-free per query
+        assert idx.min() >= 0 and idx.max() < n
+
+
+def test_config3_full_size(ctx, c_oracle):
+    """Benchmark configuration 3 at its real size: p-stable LSH, 1,000,000 x 128 N(0,1) rows, 16 tables x 8
+    hashes, window 4 (P = a / 4, b in (0, 1]; pslsh/hash.cuh:25-47, 59-89) - some 16M buckets, rank-compressed
+    keys.  Properties on everything; the whole index and the candidate lists bit-exact against the C oracle
+    given the GPU's signatures; signatures against the float64 oracle outside the band on a sample of rows.
+    Queries: the configuration's own N(0,1) queries (hardly any candidate) and fitted rows with a little
+    noise (candidates for most)."""
+    _announce("config3_full_size")
+    from abi import assert_candidates_match, assert_index_matches
+
+    n, d, nq, T, H, w = 1_000_000, 128, 10_000, 16, 8, 4
+    rng = np.random.default_rng(303)
+    X = rng.standard_normal((n, d), dtype=np.float32)
+    Q = rng.standard_normal((nq, d), dtype=np.float32)
+    near = X[rng.integers(0, n, size=nq)] + rng.normal(0.0, 0.02, size=(nq, d)).astype(np.float32)
+    P = (rng.standard_normal((T * H, d)) / w).astype(np.float32)
+    b = (1.0 - rng.random(T * H)).astype(np.float32)             # (0, 1]
+    ih = ctx.pslsh_fit(X, T, H, w, P=P, b=b)
+    ix = ctx.index_arrays(ih)
+    _index_properties(ix, n, T, 4 * H)
+    sig = ctx.pslsh_hash(X, P, b, T, H)                           # [T][n][H] int32
+    rows = rng.integers(0, n, size=3000)
+    safe = o.pslsh_margin(X[rows], P, b, T, H) > TOL
+    assert safe.mean() > 0.999
+    np.testing.assert_array_equal(sig[:, rows][safe], o.pslsh_hash(X[rows], P, b, T, H)[safe])
+    cix = c_oracle.fit_index_c(sig, H)
+    assert_index_matches(ix, cix.to_numpy(n))
+    del sig
+    for queries, expect_hits in ((Q, False), (near, True)):
+        got = ctx.pslsh_query(queries, ih)
+        _candidate_properties(got, n)
+        qsig = ctx.pslsh_hash(queries, P, b, T, H)
+        assert_candidates_match(got, c_oracle.query_index_c(qsig, cix))
+        if expect_hits:
+            assert (got["counts"] > 0).mean() > 0.5
+    ctx.free_index(ih)
+
+
+def test_config4_full_size(ctx, c_oracle):
+    """Benchmark configuration 4 at its real size: MinHash, 1,000,000 rows over 50,000 columns, Poisson(50)
+    distinct columns per row drawn from a Zipf(1.1) law, 32 tables x 4 hashes, prime 4294967291
+    (minhash/hash.cuh:17, 69-128) - some 25M buckets, rank-coded 64-bit keys, 8 radix passes.  Signatures are
+    exact integers: the GPU's equal the oracle's on a sample of rows; the whole index and the candidate lists
+    are bit-exact against the C oracle given the signatures."""
+    _announce("config4_full_size")
+    import torch
+
+    from abi import assert_candidates_match, assert_index_matches
+    from culsh_amd.benchmark import _zipf_sets
+
+    n, d, nq, T, H = 1_000_000, 50_000, 10_000, 32, 4
+    g = torch.Generator(device="cuda")
+    g.manual_seed(404)
+    Xd, Qd = _zipf_sets(torch, n, d, nq, g)
+    xi, xp = Xd.indices.cpu().numpy(), Xd.indptr.cpu().numpy()
+    qi, qp = Qd.indices.cpu().numpy(), Qd.indptr.cpu().numpy()
+    del Xd, Qd
+    nnz = np.diff(xp)
+    assert 49.5 < nnz.mean() < 50.5 and 6.5 < nnz.std() < 7.6 and nnz.min() >= 1 and xi.max() < d   # Poisson(50)
+    starts = np.ones(len(xi), dtype=bool)
+    starts[xp[1:-1]] = False
+    assert np.all((np.diff(xi.astype(np.int64)) > 0) | ~starts[1:])   # distinct, ascending columns inside a row
+    top = np.bincount(xi, minlength=d)
+    assert top[0] > 0.99 * n and top[10] > 2 * top[100] > 4 * top[1000] > 0   # heavy head of the Zipf law: nearly every row holds column 0
+    A, B = o.generate_hash_integers(42, T * H)
+    ih = ctx.minhash_fit(xi, xp, d, T, H, seed=42, A=A, B=B)
+    ix = ctx.index_arrays(ih)
+    _index_properties(ix, n, T, 4 * H)
+    sig = ctx.minhash_compute(xi, xp, A, B, T, H)                 # [T][n][H] uint32
+    rows = np.random.default_rng(5).integers(0, n, size=2000)
+    sub_ptr = np.concatenate([[0], np.cumsum(nnz[rows])]).astype(np.int32)
+    sub_idx = np.concatenate([xi[xp[r]:xp[r + 1]] for r in rows]).astype(np.int32)
+    np.testing.assert_array_equal(sig[:, rows], o.minhash_hash(sub_idx, sub_ptr, A, B, T, H))
+    cix = c_oracle.fit_index_c(sig, H)
+    assert_index_matches(ix, cix.to_numpy(n))
+    del sig
+    got = ctx.minhash_query(qi, qp, ih)
+    _candidate_properties(got, n)
+    qsig = ctx.minhash_compute(qi, qp, A, B, T, H)
+    np.testing.assert_array_equal(qsig, c_oracle.minhash_hash(qi, qp, A, B, T, H))
+    assert_candidates_match(got, c_oracle.query_index_c(qsig, cix))
+    assert got["n_total_candidates"] > 0
+    ctx.free_index(ih)
+
+
 def test_config5_full_size_invariants(ctx):
     """Benchmark configuration 5 of the reference at its real shape (4M x 768 rows of a 1000-component Gaussian mixture on the
     unit sphere, 64 tables x 16 hashes), 20k queries in batches of 10k: the index takes 2^28 items, a
