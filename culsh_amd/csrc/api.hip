@@ -35,6 +35,8 @@ culsh_status arena_begin(culsh_ctx* ctx) {
     ctx->arena_off = 0;
     ctx->arena_live = 0;
     ctx->sort_err_dev = nullptr;  // pointed into the arena of an earlier call
+    ctx->aux_flag_dev = nullptr;  // likewise
+    ctx->aux_flag_host = 0;
     if (ctx->arena_want > ctx->arena_cap) {  // stream is idle here: every call ends with a sync
         // the new block first: a grow that fails keeps the arena there is
         const size_t want = align_up(ctx->arena_want + ctx->arena_want / 8, 1 << 20);
@@ -149,7 +151,11 @@ culsh_status read_back_pair(culsh_ctx* ctx, const uint64_t* dev_a, const uint32_
     CULSH_HIP(hipMemcpyAsync(&ctx->pinned[0], dev_a, sizeof(uint64_t), hipMemcpyDeviceToHost, ctx->stream));
     if (dev_b_or_null)
         CULSH_HIP(hipMemcpyAsync(&ctx->pinned[1], dev_b_or_null, sizeof(uint32_t), hipMemcpyDeviceToHost, ctx->stream));
+    ctx->pinned[2] = 0;
+    if (ctx->aux_flag_dev)  // a family's own flag rides along
+        CULSH_HIP(hipMemcpyAsync(&ctx->pinned[2], ctx->aux_flag_dev, sizeof(uint32_t), hipMemcpyDeviceToHost, ctx->stream));
     CULSH_HIP(hipStreamSynchronize(ctx->stream));
+    ctx->aux_flag_host = static_cast<uint32_t>(ctx->pinned[2] & 0xffffffffu);
     *a = ctx->pinned[0];
     *b = static_cast<uint32_t>(ctx->pinned[1] & 0xffffffffu);
     return CULSH_OK;
@@ -578,7 +584,7 @@ static culsh_status dense_fit_once(culsh_ctx* ctx, Family fam, const T* X, int n
 
 static culsh_status minhash_fit_once(culsh_ctx* ctx, const int32_t* indices, const int32_t* indptr, int n, int d,
                                      int nT, int H, uint64_t seed, const uint32_t* A_host, const uint32_t* B_host,
-                                     culsh_index** index_out, culsh_candidates** cands_out) {
+                                     bool plain_keys, culsh_index** index_out, culsh_candidates** cands_out) {
     CULSH_TRY(check_fit_args(ctx, indptr, n, d, nT, H, index_out ? static_cast<void*>(index_out) : static_cast<void*>(cands_out),
                              cands_out != nullptr));
     CULSH_REQUIRE((A_host == nullptr) == (B_host == nullptr), CULSH_ERR_INVALID, "hash_a and hash_b must be given together");
@@ -610,14 +616,9 @@ static culsh_status minhash_fit_once(culsh_ctx* ctx, const int32_t* indices, con
         CULSH_TRY(upload_params(ctx, B_host, TH, &ix->B));
     }
     const size_t N = static_cast<size_t>(n) * nT;
-    // rank codes instead of raw hash values where that shortens the keys (needs the row count of
-    // the CSR arrays: indptr[n], read back once)
+    // rank codes instead of raw hash values where that shortens the keys
     bool ranked = false;
-    {
-        uint32_t nnz32 = 0;
-        CULSH_TRY(read_back_u32(ctx, reinterpret_cast<const uint32_t*>(indptr) + n, 1, &nnz32));
-        CULSH_TRY(mh_build_codec(ctx, indices, static_cast<size_t>(nnz32), nT, H, d, ix.get(), &ranked));
-    }
+    if (!plain_keys) CULSH_TRY(mh_build_codec(ctx, nT, H, d, ix.get(), &ranked));
     uint32_t* keys = nullptr;
     KeyEnc enc = ENC_BE;
     int W = H;
@@ -625,7 +626,11 @@ static culsh_status minhash_fit_once(culsh_ctx* ctx, const int32_t* indices, con
         enc = ENC_MHR;
         W = ix->key_w;
         CULSH_TRY(arena_alloc_t(ctx, N * W, &keys));
-        CULSH_TRY(launch_minhash_rank(ctx, indices, indptr, n, nT, H, ix.get(), true, keys));
+        // rank codes cover column ids below n_features; the kernel flags any other id in a word that
+        // comes back with the end-of-build read-back
+        CULSH_TRY(arena_alloc_t(ctx, 1, &ctx->aux_flag_dev));
+        CULSH_HIP(hipMemsetAsync(ctx->aux_flag_dev, 0, sizeof(uint32_t), ctx->stream));
+        CULSH_TRY(launch_minhash_rank(ctx, indices, indptr, n, nT, H, ix.get(), ctx->aux_flag_dev, keys));
     } else {
         CULSH_TRY(arena_alloc_t(ctx, N * H, &keys));
         CULSH_TRY(launch_minhash(ctx, indices, indptr, ix->A, ix->B, n, nT, H, true, keys));
@@ -637,6 +642,10 @@ static culsh_status minhash_fit_once(culsh_ctx* ctx, const int32_t* indices, con
         cands->device = ctx->device;
     }
     CULSH_TRY(finish_fit(ctx, keys, n, nT, H, 4 * H, enc, W, ix.get(), cands.get()));  // minhash.cu:37
+    if (ranked && ctx->aux_flag_host) {  // a column id at or beyond n_features: these keys are void
+        CULSH_TRY(arena_end(ctx));
+        return CULSH_RETRY_PLAIN_KEYS;
+    }
     ix->n_features = d;
     ix->seed = seed;
     CULSH_TRY(arena_end(ctx));
@@ -710,9 +719,14 @@ static culsh_status dense_fit(culsh_ctx* ctx, Family fam, const T* X, int n, int
 static culsh_status minhash_fit_impl(culsh_ctx* ctx, const int32_t* indices, const int32_t* indptr, int n, int d,
                                      int nT, int H, uint64_t seed, const uint32_t* A_host, const uint32_t* B_host,
                                      culsh_index** index_out, culsh_candidates** cands_out) {
-    return with_sort_retry(ctx, [&] {
-        return minhash_fit_once(ctx, indices, indptr, n, d, nT, H, seed, A_host, B_host, index_out, cands_out);
+    culsh_status s = with_sort_retry(ctx, [&] {
+        return minhash_fit_once(ctx, indices, indptr, n, d, nT, H, seed, A_host, B_host, false, index_out, cands_out);
     });
+    if (s == CULSH_RETRY_PLAIN_KEYS)
+        s = with_sort_retry(ctx, [&] {
+            return minhash_fit_once(ctx, indices, indptr, n, d, nT, H, seed, A_host, B_host, true, index_out, cands_out);
+        });
+    return s;
 }
 
 extern "C" {
@@ -947,7 +961,7 @@ culsh_status culsh_minhash_query(culsh_ctx* ctx, const int32_t* indices, const i
     uint32_t* keys = nullptr;
     if (ix->enc == ENC_MHR) {
         CULSH_TRY(arena_alloc_t(ctx, static_cast<size_t>(nq) * T * ix->key_w, &keys));
-        CULSH_TRY(launch_minhash_rank(ctx, indices, indptr, nq, T, H, ix, false, keys));
+        CULSH_TRY(launch_minhash_rank(ctx, indices, indptr, nq, T, H, ix, nullptr, keys));
     } else {
         CULSH_TRY(arena_alloc_t(ctx, static_cast<size_t>(nq) * T * H, &keys));
         CULSH_TRY(launch_minhash(ctx, indices, indptr, ix->A, ix->B, nq, T, H, true, keys));

@@ -112,6 +112,8 @@ struct culsh_ctx {
     // chained scan of the radix sort: give-up flag of the last sort (device, arena) and the
     // switch to the unchained passes after a give-up
     uint32_t* sort_err_dev = nullptr;
+    uint32_t* aux_flag_dev = nullptr;  // a family's own flag that travels with the end-of-build read-back, or null
+    uint32_t aux_flag_host = 0;        // its value after that read-back
     bool sort_unchained = false;
     // raw candidates per query of the last query call and the shape of the index it went to (rows,
     // buckets, tables, hashes): sizes the next call's output without a host round trip (query.hip)
@@ -230,6 +232,9 @@ culsh_status read_back_pair(culsh_ctx* ctx, const uint64_t* dev_a, const uint32_
 // Internal status: the radix sort's chained scan gave up; the caller switches the context to
 // unchained passes and repeats the fit.  Never returned through the C ABI.
 constexpr culsh_status CULSH_RETRY_UNCHAINED = static_cast<culsh_status>(7);
+// Internal: a MinHash fit with rank keys met a column id at or beyond n_features; the fit is
+// repeated with plain keys, which hash any id.
+constexpr culsh_status CULSH_RETRY_PLAIN_KEYS = static_cast<culsh_status>(6);
 
 // ---------------------------------------------------------------- projection (project.hip)
 // Output modes of the projection kernels.
@@ -272,15 +277,17 @@ culsh_status launch_ps_keys_to_sig(culsh_ctx* ctx, const culsh_index* ix, size_t
 void free_ps_codec(culsh_index* ix);
 
 // ---------------------------------------------------------------- MinHash key compression (mhcodec.hip)
-// Builds the rank tables from ix->A / ix->B when that shortens the keys and every column id in
-// `indices` is below n_features `d`; then fills ix->mhc, sets ix->enc = ENC_MHR and ix->key_w, and
-// reports used = true.  May return CULSH_RETRY_UNCHAINED (its column sort is a chained radix sort).
-culsh_status mh_build_codec(culsh_ctx* ctx, const int32_t* indices, size_t nnz, int T, int H, int d, culsh_index* ix,
-                            bool* used);
-// CSR rows -> packed rank codes [T][n][ix->key_w].  `ids_below_d`: the caller has checked that every
-// column id is below the codec's n_features (a cheaper hash applies to small ids).
+// Builds the rank tables from ix->A / ix->B when that shortens the keys; then fills ix->mhc, sets
+// ix->enc = ENC_MHR and ix->key_w, and reports used = true.  Rank codes stand for column ids below
+// n_features `d` only: the fit's rank kernel flags any other id (see launch_minhash_rank).
+// May return CULSH_RETRY_UNCHAINED (its column sort is a chained radix sort).
+culsh_status mh_build_codec(culsh_ctx* ctx, int T, int H, int d, culsh_index* ix, bool* used);
+// CSR rows -> packed rank codes [T][n][ix->key_w].  `fit_flag` non-null (the fit): ids are taken to
+// be below the codec's n_features, for which a cheaper hash applies, and the word is set to 1 when
+// one is not — the keys are then wrong (never out of bounds) and the caller fits again with plain
+// keys.  Null (queries): any id is hashed as it is; ids the fit never saw match nothing.
 culsh_status launch_minhash_rank(culsh_ctx* ctx, const int32_t* indices, const int32_t* indptr, int n, int T, int H,
-                                 const culsh_index* ix, bool ids_below_d, uint32_t* keys);
+                                 const culsh_index* ix, uint32_t* fit_flag, uint32_t* keys);
 // uint32 signatures [T][rows][H] -> packed rank codes
 culsh_status launch_mh_sig_to_keys(culsh_ctx* ctx, const uint32_t* sig, size_t rows, const culsh_index* ix,
                                    uint32_t* keys);

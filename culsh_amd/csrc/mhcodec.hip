@@ -39,29 +39,6 @@ __device__ __forceinline__ uint32_t hash_mod_p_small(uint32_t a, uint32_t x, uin
     return v1 >= PRIME ? lo + 5u : lo;
 }
 
-__global__ __launch_bounds__(256) void mh_max_index_kernel(const int32_t* __restrict__ indices, size_t nnz,
-                                                          uint32_t* __restrict__ out_max) {
-    uint32_t m = 0;  // negative ids read as huge values: out of range
-    const size_t stride = static_cast<size_t>(gridDim.x) * 256;
-    const size_t tid = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
-    const size_t head = std::min(nnz, (16 - reinterpret_cast<uintptr_t>(indices) % 16) % 16 / 4);  // up to alignment
-    const uint4* v = reinterpret_cast<const uint4*>(indices + head);
-    const size_t nvec = (nnz - head) / 4;
-#pragma unroll 4
-    for (size_t i = tid; i < nvec; i += stride) {
-        const uint4 q = v[i];
-        m = max(max(m, q.x), max(max(q.y, q.z), q.w));
-    }
-    if (tid < head) m = max(m, static_cast<uint32_t>(indices[tid]));
-    const size_t tail0 = head + nvec * 4;
-    if (tail0 + tid < nnz) m = max(m, static_cast<uint32_t>(indices[tail0 + tid]));  // fewer than 4 left
-#pragma unroll
-    for (int s = 32; s > 0; s >>= 1) m = max(m, static_cast<uint32_t>(__shfl_xor(m, s, 64)));
-    // atomics on one address are served one after the other: only wavefronts that would raise the
-    // maximum issue one
-    if ((threadIdx.x & 63) == 0 && m > __atomic_load_n(out_max, __ATOMIC_RELAXED)) atomicMax(out_max, m);
-}
-
 // ainv[c] = A[c]^(p-2) mod p: the inverse of the multiplier, with which the column that produced a
 // hash value is recovered from the value (the hash is a bijection of [0, p) unless A[c] = 0 mod p)
 __global__ __launch_bounds__(256) void mh_inverse_kernel(const uint32_t* __restrict__ A, int count,
@@ -120,11 +97,21 @@ __global__ __launch_bounds__(NTHREADS) void minhash_rank_kernel(const int32_t* _
                                                                const uint32_t* __restrict__ ainv,
                                                                const uint32_t* __restrict__ rank, int n, int T, int H,
                                                                int d, int bits, int W, int th_chunk,
-                                                               uint32_t* __restrict__ out) {
+                                                               uint32_t* __restrict__ out,
+                                                               uint32_t* __restrict__ id_beyond_d) {
     extern __shared__ uint32_t stage[];  // [th_chunk][RB] codes
     const int TH = T * H;
     const int row0 = blockIdx.x * RB;
     const int rows = min(RB, n - row0);
+    if (SMALL && id_beyond_d) {
+        // The cheaper hash and the rank codes hold for ids below d only: the workgroup looks once at
+        // the ids of its rows (one contiguous stretch; negative ids read as huge) and tells the host.
+        // Every lane that sees such an id stores the same word.
+        uint32_t fmax = 0;
+        for (int j = indptr[row0] + static_cast<int>(threadIdx.x), e = indptr[row0 + rows]; j < e; j += NTHREADS)
+            fmax = max(fmax, static_cast<uint32_t>(indices[j]));
+        if (fmax >= static_cast<uint32_t>(d)) *id_beyond_d = 1u;
+    }
     for (int c0 = 0; c0 < TH; c0 += th_chunk) {
         const int nc = min(th_chunk, TH - c0);
         // (row r, hash c0 + c) -> stage[c][r]
@@ -242,50 +229,67 @@ __global__ __launch_bounds__(256) void mh_sig_to_keys_kernel(const uint32_t* __r
     if (nbits > 0) k[w++] = static_cast<uint32_t>(acc << (32 - nbits));
 }
 
-constexpr int MH_BPB = 256;  // buckets per workgroup
+// Signatures of the buckets from their rank keys.  A workgroup takes `bpb` consecutive buckets (a
+// multiple of 256 chosen by the host so that the key words fit in 16 KiB of LDS) and searches the
+// tables of its first and last bucket once; nearly every workgroup lies inside one table or across one
+// boundary, and then a bucket's table follows from one comparison.
+constexpr int MH_BPB_MIN = 256;
+
+// largest t in [lo, hi) with table_bucket_offsets[t] <= bucket
+__device__ __forceinline__ int mh_table_of(const int32_t* __restrict__ table_bucket_offsets, int lo, int hi, size_t bucket) {
+    while (hi - lo > 1) {
+        const int mid = (lo + hi) >> 1;
+        if (static_cast<size_t>(table_bucket_offsets[mid]) <= bucket) lo = mid; else hi = mid;
+    }
+    return lo;
+}
+
 __global__ __launch_bounds__(256) void mh_keys_to_sig_kernel(const uint32_t* __restrict__ keys, size_t count,
                                                             const uint64_t* __restrict__ count_dev,
                                                             const int32_t* __restrict__ table_bucket_offsets, int T,
-                                                            int H, int d, int bits, int W,
+                                                            int H, int d, int bits, int W, int bpb,
                                                             const uint32_t* __restrict__ inv,
                                                             uint32_t* __restrict__ sig) {
-    extern __shared__ uint32_t mh_lds[];  // [MH_BPB] table ids, then [MH_BPB][W] key words
-    uint32_t* tb = mh_lds;
-    uint32_t* kw = mh_lds + MH_BPB;
+    extern __shared__ uint32_t mh_lds[];  // [2] first and last table, then [bpb][W] key words
+    uint32_t* trange = mh_lds;
+    uint32_t* kw = mh_lds + 2;
     if (count_dev) count = min(count, static_cast<size_t>(*count_dev));
-    const size_t b0 = static_cast<size_t>(blockIdx.x) * MH_BPB;
+    const size_t b0 = static_cast<size_t>(blockIdx.x) * bpb;
     if (b0 >= count) return;
-    const int nb = static_cast<int>(min(static_cast<size_t>(MH_BPB), count - b0));
-    if (static_cast<int>(threadIdx.x) < nb) {
-        const size_t bucket = b0 + threadIdx.x;
-        int lo = 0, hi = T;  // largest t with table_bucket_offsets[t] <= bucket
-        while (hi - lo > 1) {
-            const int mid = (lo + hi) >> 1;
-            if (static_cast<size_t>(table_bucket_offsets[mid]) <= bucket) lo = mid; else hi = mid;
-        }
-        tb[threadIdx.x] = static_cast<uint32_t>(lo);
-    }
+    const int nb = static_cast<int>(min(static_cast<size_t>(bpb), count - b0));
+    if (threadIdx.x < 2)
+        trange[threadIdx.x] = static_cast<uint32_t>(
+            mh_table_of(table_bucket_offsets, 0, T, threadIdx.x == 0 ? b0 : b0 + static_cast<size_t>(nb) - 1));
     for (int i = threadIdx.x; i < nb * W; i += 256) kw[i] = keys[b0 * W + i];
     __syncthreads();
+    const int t_first = static_cast<int>(trange[0]), t_last = static_cast<int>(trange[1]);
+    const bool near = t_last - t_first <= 1;  // uniform over the workgroup
+    const size_t second = t_last > t_first ? static_cast<size_t>(table_bucket_offsets[t_first + 1]) : ~size_t(0);
     const uint32_t mask = (1u << bits) - 1u;
-    auto value = [&](int bl, int h) -> uint32_t {
+    auto value = [&](int bl, int t, int h) -> uint32_t {
         const uint32_t* k = kw + bl * W;
         const int o = h * bits, w0 = o >> 5, sh = o & 31;
         const unsigned long long two = (static_cast<unsigned long long>(k[w0]) << 32) | (w0 + 1 < W ? k[w0 + 1] : 0u);
         const uint32_t code = static_cast<uint32_t>(two >> (64 - sh - bits)) & mask;
-        return code < static_cast<uint32_t>(d) ? inv[static_cast<size_t>(tb[bl] * H + h) * d + code] : 0xFFFFFFFFu;
+        return code < static_cast<uint32_t>(d) ? inv[static_cast<size_t>(t * H + h) * d + code] : 0xFFFFFFFFu;
+    };
+    auto table = [&](int bl) -> int {
+        const size_t bucket = b0 + bl;
+        return near ? t_first + (bucket >= second ? 1 : 0) : mh_table_of(table_bucket_offsets, t_first, t_last + 1, bucket);
     };
     uint32_t* out = sig + b0 * H;
     if (H % 4 == 0 && reinterpret_cast<uintptr_t>(sig) % 16 == 0) {  // four hashes of a bucket per thread and store
         const int qpb = H >> 2;
         for (int q = threadIdx.x; q < nb * qpb; q += 256) {
             const int bl = q / qpb, h = (q - bl * qpb) << 2;
-            *reinterpret_cast<uint4*>(out + 4 * q) = make_uint4(value(bl, h), value(bl, h + 1), value(bl, h + 2), value(bl, h + 3));
+            const int t = table(bl);
+            *reinterpret_cast<uint4*>(out + 4 * static_cast<size_t>(q)) =
+                make_uint4(value(bl, t, h), value(bl, t, h + 1), value(bl, t, h + 2), value(bl, t, h + 3));
         }
     } else {
         for (int i = threadIdx.x; i < nb * H; i += 256) {
             const int bl = i / H;
-            out[i] = value(bl, i - bl * H);
+            out[i] = value(bl, table(bl), i - bl * H);
         }
     }
 }
@@ -299,27 +303,14 @@ void free_mh_codec(culsh_index* ix) {
     ix->mhc = MhCodec();
 }
 
-culsh_status mh_build_codec(culsh_ctx* ctx, const int32_t* indices, size_t nnz, int T, int H, int d, culsh_index* ix,
-                            bool* used) {
+culsh_status mh_build_codec(culsh_ctx* ctx, int T, int H, int d, culsh_index* ix, bool* used) {
     *used = false;
     const size_t TH = static_cast<size_t>(T) * H;
     if (d < 1 || TH * static_cast<size_t>(d) > (size_t(1) << 25) || TH > 65535) return CULSH_OK;
     int bits = 1;
     while ((1ll << bits) < static_cast<long long>(d) + 2) ++bits;
     const int W = (H * bits + 31) / 32;
-    if (W >= H || W > 64) return CULSH_OK;  // nothing to gain
-    // rank codes stand for columns below n_features only
-    if (nnz > 0) {
-        uint32_t* mx = nullptr;
-        CULSH_TRY(arena_alloc_t(ctx, 1, &mx));
-        CULSH_HIP(hipMemsetAsync(mx, 0, sizeof(uint32_t), ctx->stream));
-        const unsigned blocks = std::max(1u, std::min(4096u, div_up(nnz, 256 * 16)));
-        CULSH_LAUNCH(ctx, mh_max_index_kernel, dim3(blocks), dim3(256), 0, ctx->stream, indices, nnz, mx);
-        CULSH_LAUNCH_CHECK();
-        uint32_t max_index = 0;
-        CULSH_TRY(read_back_u32(ctx, mx, 1, &max_index));
-        if (max_index >= static_cast<uint32_t>(d)) return CULSH_OK;  // plain keys hash any column id
-    }
+    if (W >= H || W > 56) return CULSH_OK;  // nothing to gain, or more than the restore kernel keeps in LDS (256 keys of W words)
     const size_t total = TH * d;
     uint32_t *keys = nullptr, *keys_tmp = nullptr, *sorted = nullptr;
     int32_t *cols_tmp = nullptr, *cols = nullptr;
@@ -357,19 +348,21 @@ culsh_status mh_build_codec(culsh_ctx* ctx, const int32_t* indices, size_t nnz, 
 }
 
 culsh_status launch_minhash_rank(culsh_ctx* ctx, const int32_t* indices, const int32_t* indptr, int n, int T, int H,
-                                 const culsh_index* ix, bool ids_below_d, uint32_t* keys) {
+                                 const culsh_index* ix, uint32_t* fit_flag, uint32_t* keys) {
     CULSH_REQUIRE(indptr && keys && ix->mhc.rank, CULSH_ERR_INVALID, "minhash: null pointer");
     CULSH_REQUIRE(n > 0, CULSH_ERR_INVALID, "minhash: sizes must be positive");
     CULSH_REQUIRE(H <= 384, CULSH_ERR_LIMIT, "minhash: n_hashes > 384 is not supported");
     int tables_per_chunk = static_cast<int>(std::min<long long>(T, std::max(1, (12288 / RB) / H)));
     const int th_chunk = tables_per_chunk * H;
     const size_t lds = static_cast<size_t>(th_chunk) * RB * sizeof(uint32_t);
-    if (ids_below_d && ix->mhc.d <= (1 << 25))
+    if (fit_flag && ix->mhc.d <= (1 << 25))
         CULSH_LAUNCH(ctx, minhash_rank_kernel<true>, dim3((n + RB - 1) / RB), dim3(NTHREADS), lds, ctx->stream, indices,
-                     indptr, ix->A, ix->B, ix->mhc.ainv, ix->mhc.rank, n, T, H, ix->mhc.d, ix->mhc.bits, ix->key_w, th_chunk, keys);
+                     indptr, ix->A, ix->B, ix->mhc.ainv, ix->mhc.rank, n, T, H, ix->mhc.d, ix->mhc.bits, ix->key_w, th_chunk,
+                     keys, fit_flag);
     else
         CULSH_LAUNCH(ctx, minhash_rank_kernel<false>, dim3((n + RB - 1) / RB), dim3(NTHREADS), lds, ctx->stream, indices,
-                     indptr, ix->A, ix->B, ix->mhc.ainv, ix->mhc.rank, n, T, H, ix->mhc.d, ix->mhc.bits, ix->key_w, th_chunk, keys);
+                     indptr, ix->A, ix->B, ix->mhc.ainv, ix->mhc.rank, n, T, H, ix->mhc.d, ix->mhc.bits, ix->key_w, th_chunk,
+                     keys, static_cast<uint32_t*>(nullptr));
     CULSH_LAUNCH_CHECK();
     return CULSH_OK;
 }
@@ -388,11 +381,13 @@ culsh_status launch_mh_sig_to_keys(culsh_ctx* ctx, const uint32_t* sig, size_t r
 culsh_status launch_mh_keys_to_sig(culsh_ctx* ctx, const culsh_index* ix, size_t count, const uint64_t* count_dev,
                                    uint8_t* sig) {
     if (count == 0) return CULSH_OK;
-    CULSH_REQUIRE(count / MH_BPB < (1ull << 31), CULSH_ERR_LIMIT, "too many buckets");
-    const size_t lds = static_cast<size_t>(MH_BPB) * (1 + ix->key_w) * sizeof(uint32_t);
-    CULSH_LAUNCH(ctx, mh_keys_to_sig_kernel, dim3(div_up(count, MH_BPB)), dim3(256), lds, ctx->stream, ix->bucket_keys,
+    // buckets per workgroup: as many as 16 KiB of key words hold, 256 to 2048
+    const int bpb = std::max(MH_BPB_MIN, std::min(2048, (4096 / ix->key_w) / 256 * 256));
+    CULSH_REQUIRE(count / bpb < (1ull << 31), CULSH_ERR_LIMIT, "too many buckets");
+    const size_t lds = (2 + static_cast<size_t>(bpb) * ix->key_w) * sizeof(uint32_t);
+    CULSH_LAUNCH(ctx, mh_keys_to_sig_kernel, dim3(div_up(count, bpb)), dim3(256), lds, ctx->stream, ix->bucket_keys,
                  count, count_dev, ix->table_bucket_offsets, ix->n_hash_tables, ix->n_hashes, ix->mhc.d, ix->mhc.bits,
-                 ix->key_w, ix->mhc.inv, reinterpret_cast<uint32_t*>(sig));
+                 ix->key_w, bpb, ix->mhc.inv, reinterpret_cast<uint32_t*>(sig));
     CULSH_LAUNCH_CHECK();
     return CULSH_OK;
 }

@@ -160,70 +160,83 @@ __global__ __launch_bounds__(256) void ps_compress_kernel(const int32_t* __restr
     }
 }
 
-// A workgroup restores the signatures of PS_BPB consecutive buckets: the table of each bucket
-// is searched once and kept in LDS with the bucket's key words, then (bucket, hash) pairs are
-// written by consecutive threads to consecutive addresses.  With `use_lds` the launch also carries
-// 2 * H * rmax words of LDS for the value tables of two neighbouring hash tables, which cover a
-// workgroup unless it meets three tables or more.
-constexpr int PS_BPB = 256;
+// A workgroup restores the signatures of `bpb` consecutive buckets (a multiple of 256 chosen by the
+// host so that the key words fit in 16 KiB of LDS).  The tables of its first and last bucket are
+// searched once; nearly every workgroup lies inside one table or across one boundary, and then a
+// bucket's table follows from one comparison.  (bucket, hash) pairs are written by consecutive
+// threads to consecutive addresses.  With `use_lds` the launch also carries 2 * H * rmax words of
+// LDS for the value tables of two neighbouring hash tables.
+constexpr int PS_BPB_MIN = 256;
+
+// largest t in [lo, hi) with table_bucket_offsets[t] <= bucket
+__device__ __forceinline__ int ps_table_of(const int32_t* __restrict__ table_bucket_offsets, int lo, int hi, size_t bucket) {
+    while (hi - lo > 1) {
+        const int mid = (lo + hi) >> 1;
+        if (static_cast<size_t>(table_bucket_offsets[mid]) <= bucket) lo = mid; else hi = mid;
+    }
+    return lo;
+}
+
 __global__ __launch_bounds__(256) void ps_keys_to_sig_kernel(const uint32_t* __restrict__ keys, size_t count,
                                                             const uint64_t* __restrict__ count_dev,
                                                             const int32_t* __restrict__ table_bucket_offsets, int T,
-                                                            int H, int bits, int rmax, int W, int use_lds,
+                                                            int H, int bits, int rmax, int W, int use_lds, int bpb,
                                                             const int32_t* __restrict__ inv,
                                                             int32_t* __restrict__ sig,
                                                             const uint32_t* __restrict__ sort_gave_up) {
-    extern __shared__ uint32_t ps_lds[];  // [PS_BPB] table ids, [PS_BPB][W] key words, then the value tables
+    extern __shared__ uint32_t ps_lds[];  // [2] first and last table, [bpb][W] key words, then the value tables
     if (sort_gave_up && *sort_gave_up) return;  // bucket keys of a failed sort may hold ranks beyond the tables
-    uint32_t* tb = ps_lds;
-    uint32_t* kw = ps_lds + PS_BPB;
-    int32_t* lut = reinterpret_cast<int32_t*>(kw + PS_BPB * W);
+    uint32_t* trange = ps_lds;
+    uint32_t* kw = ps_lds + 2;
+    int32_t* lut = reinterpret_cast<int32_t*>(kw + static_cast<size_t>(bpb) * W);
     if (count_dev) count = min(count, static_cast<size_t>(*count_dev));
-    const size_t b0 = static_cast<size_t>(blockIdx.x) * PS_BPB;
+    const size_t b0 = static_cast<size_t>(blockIdx.x) * bpb;
     if (b0 >= count) return;
-    const int nb = static_cast<int>(min(static_cast<size_t>(PS_BPB), count - b0));
-    if (static_cast<int>(threadIdx.x) < nb) {
-        const size_t bucket = b0 + threadIdx.x;
-        int lo = 0, hi = T;  // largest t with table_bucket_offsets[t] <= bucket
-        while (hi - lo > 1) {
-            const int mid = (lo + hi) >> 1;
-            if (static_cast<size_t>(table_bucket_offsets[mid]) <= bucket) lo = mid; else hi = mid;
-        }
-        tb[threadIdx.x] = static_cast<uint32_t>(lo);
-    }
+    const int nb = static_cast<int>(min(static_cast<size_t>(bpb), count - b0));
+    if (threadIdx.x < 2)
+        trange[threadIdx.x] = static_cast<uint32_t>(
+            ps_table_of(table_bucket_offsets, 0, T, threadIdx.x == 0 ? b0 : b0 + static_cast<size_t>(nb) - 1));
     for (int i = threadIdx.x; i < nb * W; i += 256) kw[i] = keys[b0 * W + i];
     __syncthreads();
-    const int t_first = static_cast<int>(tb[0]);
-    const bool staged = use_lds && static_cast<int>(tb[nb - 1]) - t_first <= 1;  // uniform over the workgroup
+    const int t_first = static_cast<int>(trange[0]), t_last = static_cast<int>(trange[1]);
+    const bool near = t_last - t_first <= 1;  // uniform over the workgroup
+    const bool staged = use_lds && near;
     if (staged) {
-        const int words = (static_cast<int>(tb[nb - 1]) - t_first + 1) * H * rmax;  // one table's values, or two
+        const int words = (t_last - t_first + 1) * H * rmax;  // one table's values, or two
         const int32_t* src = inv + static_cast<size_t>(t_first) * H * rmax;
         for (int i = threadIdx.x; i < words; i += 256) lut[i] = src[i];
         __syncthreads();
     }
+    // first bucket of the second table (none: beyond every bucket)
+    const size_t second = t_last > t_first ? static_cast<size_t>(table_bucket_offsets[t_first + 1]) : ~size_t(0);
     const uint32_t mask = (1u << bits) - 1u;
-    auto value = [&](int bl, int h) -> int32_t {
+    auto value = [&](int bl, int t, int h) -> int32_t {
         const uint32_t* k = kw + bl * W;
         const int o = h * bits, w0 = o >> 5, sh = o & 31;
         const unsigned long long two = (static_cast<unsigned long long>(k[w0]) << 32) | (w0 + 1 < W ? k[w0 + 1] : 0u);
         const uint32_t code = static_cast<uint32_t>(two >> (64 - sh - bits)) & mask;
         if (!code) return 0;
-        const int c = static_cast<int>(tb[bl]) * H + h;
+        const int c = t * H + h;
         return staged ? lut[(c - t_first * H) * rmax + static_cast<int>(code - 1u)]
                       : inv[static_cast<size_t>(c) * rmax + (code - 1u)];
+    };
+    auto table = [&](int bl) -> int {
+        const size_t bucket = b0 + bl;
+        return near ? t_first + (bucket >= second ? 1 : 0) : ps_table_of(table_bucket_offsets, t_first, t_last + 1, bucket);
     };
     int32_t* out = sig + b0 * H;
     if (H % 4 == 0 && reinterpret_cast<uintptr_t>(sig) % 16 == 0) {  // four hashes of a bucket per thread and store
         const int qpb = H >> 2;
         for (int q = threadIdx.x; q < nb * qpb; q += 256) {
             const int bl = q / qpb, h = (q - bl * qpb) << 2;
-            *reinterpret_cast<int4*>(out + 4 * q) =
-                make_int4(value(bl, h), value(bl, h + 1), value(bl, h + 2), value(bl, h + 3));
+            const int t = table(bl);
+            *reinterpret_cast<int4*>(out + 4 * static_cast<size_t>(q)) =
+                make_int4(value(bl, t, h), value(bl, t, h + 1), value(bl, t, h + 2), value(bl, t, h + 3));
         }
     } else {
         for (int i = threadIdx.x; i < nb * H; i += 256) {
             const int bl = i / H;
-            out[i] = value(bl, i - bl * H);
+            out[i] = value(bl, table(bl), i - bl * H);
         }
     }
 }
@@ -265,7 +278,7 @@ culsh_status ps_build_codec(culsh_ctx* ctx, const int32_t* sig, int n, int T, in
     while ((1ll << bits) < rmax + 1) ++bits;  // codes 1..range, 0 reserved
     const int W = (H * bits + 31) / 32;
     if (bits > 12 || W >= H) return CULSH_OK;  // wide value ranges: keep the plain byte order keys
-    if (W > 56) return CULSH_OK;               // the restore kernel keeps PS_BPB keys of W words in LDS
+    if (W > 56) return CULSH_OK;               // the restore kernel keeps at least 256 keys of W words in LDS
 
     // one host block, one device block, one copy: vmin[TH] | range[TH] | fwd[TH][rmax] | inv[TH][rmax]
     const size_t lut = static_cast<size_t>(TH) * rmax;
@@ -327,15 +340,17 @@ culsh_status launch_ps_compress(culsh_ctx* ctx, const int32_t* sig, size_t rows,
 culsh_status launch_ps_keys_to_sig(culsh_ctx* ctx, const culsh_index* ix, size_t count, const uint64_t* count_dev,
                                    uint8_t* sig) {
     if (count == 0) return CULSH_OK;
-    CULSH_REQUIRE(count / PS_BPB < (1ull << 31), CULSH_ERR_LIMIT, "too many buckets");
     const PsCodec& pc = ix->psc;
     const size_t lut_words = 2 * static_cast<size_t>(ix->n_hashes) * pc.rmax;
     const int use_lds = lut_words <= PS_LUT_WORDS;
-    const size_t lds = (static_cast<size_t>(PS_BPB) * (1 + ix->key_w) + (use_lds ? lut_words : 0)) * sizeof(uint32_t);
+    // buckets per workgroup: as many as 16 KiB of key words hold, 256 to 2048
+    const int bpb = std::max(PS_BPB_MIN, std::min(2048, (4096 / ix->key_w) / 256 * 256));
+    CULSH_REQUIRE(count / bpb < (1ull << 31), CULSH_ERR_LIMIT, "too many buckets");
+    const size_t lds = (2 + static_cast<size_t>(bpb) * ix->key_w + (use_lds ? lut_words : 0)) * sizeof(uint32_t);
     CULSH_REQUIRE(lds <= 64 * 1024, CULSH_ERR_LIMIT, "key width too large for the signature restore kernel");
-    CULSH_LAUNCH(ctx, ps_keys_to_sig_kernel, dim3(div_up(count, PS_BPB)), dim3(256), lds, ctx->stream, ix->bucket_keys,
+    CULSH_LAUNCH(ctx, ps_keys_to_sig_kernel, dim3(div_up(count, bpb)), dim3(256), lds, ctx->stream, ix->bucket_keys,
                  count, count_dev, ix->table_bucket_offsets, ix->n_hash_tables, ix->n_hashes, pc.bits, pc.rmax,
-                 ix->key_w, use_lds, pc.inv, reinterpret_cast<int32_t*>(sig), static_cast<const uint32_t*>(ctx->sort_err_dev));
+                 ix->key_w, use_lds, bpb, pc.inv, reinterpret_cast<int32_t*>(sig), static_cast<const uint32_t*>(ctx->sort_err_dev));
     CULSH_LAUNCH_CHECK();
     return CULSH_OK;
 }

@@ -110,15 +110,17 @@ struct PassList {
 // own size: the totals do not depend on how the scatter cuts a table).
 constexpr int TOT_ITEMS = 32;
 constexpr int TOT_TILE = SORT_THREADS * TOT_ITEMS;
+constexpr int TOT_ROW = 257;  // words per histogram row
 __global__ __launch_bounds__(SORT_THREADS) void radix_totals_kernel(const uint32_t* __restrict__ keys, int n, int W,
-                                                                   PassList pl, int T,
+                                                                   PassList pl, int T, int copies,
                                                                    uint32_t* __restrict__ dtot /*[pass][T][256]*/) {
-    __shared__ uint32_t h[MAX_PASSES_PER_LAUNCH][256];
+    // Several copies of every pass's histogram, one per lane residue: lanes of one wavefront that hold
+    // the same digit (frequent with skewed keys) then add to different words, and a row of 257 words
+    // puts those words into different banks as well.
+    extern __shared__ uint32_t h[];  // [copies][pl.count][TOT_ROW]
     const int t = blockIdx.y;
-    // few passes leave room for one histogram copy per wavefront (fewer same-address atomics)
-    const int copies = pl.count <= MAX_PASSES_PER_LAUNCH / 4 ? 4 : (pl.count <= MAX_PASSES_PER_LAUNCH / 2 ? 2 : 1);
-    const int mine = (threadIdx.x >> 6) % copies;
-    for (int i = threadIdx.x; i < copies * pl.count * 256; i += SORT_THREADS) (&h[0][0])[i] = 0;
+    const int mine = static_cast<int>(threadIdx.x & 63) % copies;
+    for (int i = threadIdx.x; i < copies * pl.count * TOT_ROW; i += SORT_THREADS) h[i] = 0;
     __syncthreads();
     const uint32_t* tk = keys + static_cast<size_t>(t) * n * W;
     const int last_idx = n - 1;
@@ -137,7 +139,7 @@ __global__ __launch_bounds__(SORT_THREADS) void radix_totals_kernel(const uint32
                     kw[j] = tk[static_cast<size_t>(idx) * W + last_word];
                 }
             }
-            uint32_t* hp = h[mine * pl.count + p];
+            uint32_t* hp = h + (mine * pl.count + p) * TOT_ROW;
             const int shift = pl.shift[p];
 #pragma unroll
             for (int j = 0; j < TOT_ITEMS; ++j) {
@@ -149,7 +151,7 @@ __global__ __launch_bounds__(SORT_THREADS) void radix_totals_kernel(const uint32
     __syncthreads();
     for (int p = 0; p < pl.count; ++p) {
         uint32_t c = 0;
-        for (int r = 0; r < copies; ++r) c += h[r * pl.count + p][threadIdx.x];
+        for (int r = 0; r < copies; ++r) c += h[(r * pl.count + p) * TOT_ROW + threadIdx.x];
         if (c) atomicAdd(&dtot[(static_cast<size_t>(p) * T + t) * 256 + threadIdx.x], c);
     }
 }
@@ -550,8 +552,12 @@ culsh_status sort_tables(culsh_ctx* ctx, uint32_t* keys_in, uint32_t* keys_tmp, 
             }
             // about four workgroups per CU over all tables
             const int per_table = std::max(1, std::min((n + TOT_TILE - 1) / TOT_TILE, (4 * ctx->n_cus + T - 1) / T));
-            CULSH_LAUNCH(ctx, radix_totals_kernel, dim3(per_table, T), dim3(SORT_THREADS), 0, ctx->stream, keys_in, n, W, pl,
-                         T, dtot + static_cast<size_t>(p0) * T * 256);
+            // as many histogram copies as 60 KiB hold, eight at most
+            static const int lds_kb = [] { const char* e = std::getenv("CULSH_TOTALS_LDS_KB"); return e && *e ? std::atoi(e) : 60; }();
+            const int copies = std::max(1, std::min(8, (lds_kb * 1024) / (pl.count * TOT_ROW * 4)));
+            const size_t lds = static_cast<size_t>(copies) * pl.count * TOT_ROW * sizeof(uint32_t);
+            CULSH_LAUNCH(ctx, radix_totals_kernel, dim3(per_table, T), dim3(SORT_THREADS), lds, ctx->stream, keys_in, n, W, pl,
+                         T, copies, dtot + static_cast<size_t>(p0) * T * 256);
             CULSH_LAUNCH_CHECK();
         }
     } else {

@@ -1184,11 +1184,22 @@ def test_minhash_rank_keys_edge_cases(ctx):
     assert_candidates_match(ctx.minhash_query(qindices, qindptr, ih3), o.query_index(qsig3, exp_ix3))
     ctx.free_index(ih3)
     # a fitted row with a column id >= n_features: every id is hashed as it is (minhash/hash.cuh:97-104)
+    # (the rank kernel flags it and the fit is repeated with plain keys); ids next to the bound, beyond
+    # the range of the cheaper hash, at the top of int32, and in the last row
+    for pos, bad_id in ((7, d + 123), (0, d), (len(indices) - 1, (1 << 25) + 5), (indptr[n // 2], (1 << 31) - 1)):
+        bad = indices.copy()
+        bad[pos] = bad_id
+        sig2 = o.minhash_hash(bad, indptr, A, B, T, H)
+        ih2 = ctx.minhash_fit(bad, indptr, d, T, H, A=A, B=B)
+        exp_ix2 = o.fit_index(sig2, H)
+        assert_index_matches(ctx.index_arrays(ih2), exp_ix2)
+        assert_candidates_match(ctx.minhash_query(qindices, qindptr, ih2), o.query_index(qsig, exp_ix2))
+        ctx.free_index(ih2)
     bad = indices.copy()
-    bad[7] = d + 123
-    sig2 = o.minhash_hash(bad, indptr, A, B, T, H)
-    ih2 = ctx.minhash_fit(bad, indptr, d, T, H, A=A, B=B)
-    exp_ix2 = o.fit_index(sig2, H)
-    assert_index_matches(ctx.index_arrays(ih2), exp_ix2)
-    assert_candidates_match(ctx.minhash_query(qindices, qindptr, ih2), o.query_index(qsig, exp_ix2))
-    ctx.free_index(ih2)
+    bad[11] = d + 1
+    assert_candidates_match(ctx.minhash_fit_query(bad, indptr, d, T, H, A=A, B=B),
+                            o.fit_query(o.minhash_hash(bad, indptr, A, B, T, H), H))
+    # and a fit with rank keys straight after one that fell back: the flag does not stick
+    ih4 = ctx.minhash_fit(indices, indptr, d, T, H, A=A, B=B)
+    assert_index_matches(ctx.index_arrays(ih4), exp_ix)
+    ctx.free_index(ih4)
