@@ -373,16 +373,19 @@ static culsh_status hash_dense_to_keys(culsh_ctx* ctx, Family fam, const T* X, i
     // p-stable: int32 hashes in the reference layout first (pslsh/hash.cuh:25-47)
     int32_t* sig = nullptr;
     CULSH_TRY(arena_alloc_t(ctx, N * H, &sig));
+    int32_t* mm = nullptr;     // fit: value range of every hash function, folded by the projection where it can
+    bool mm_folded = false;
     if constexpr (std::is_same_v<T, float>) {
+        if (fit_ix && H <= 1024) CULSH_TRY(ps_minmax_prepare(ctx, nT, H, &mm));
         CULSH_TRY(launch_project_f32(ctx, X, static_cast<const float*>(P), static_cast<const float*>(b), rows, d, nT, H,
-                                     EPI_FLOOR_I32, sig));
+                                     EPI_FLOOR_I32, sig, mm, &mm_folded));
     } else {
         CULSH_TRY(launch_project_f64(ctx, X, static_cast<const double*>(P), static_cast<const double*>(b), rows, d, nT,
                                      H, EPI_FLOOR_I32, sig));
     }
     if (fit_ix) {
         bool compressed = false;
-        CULSH_TRY(ps_build_codec(ctx, sig, rows, nT, H, fit_ix, &compressed));
+        CULSH_TRY(ps_build_codec(ctx, sig, rows, nT, H, fit_ix, &compressed, mm_folded ? mm : nullptr));
         if (!compressed) { fit_ix->enc = ENC_BE; fit_ix->key_w = H; }
         ix = fit_ix;
     }

@@ -243,8 +243,13 @@ enum ProjEpilogue : int {
     EPI_SIGN_BYTES = 1,  // RPLSH, reference layout: uint8 [T][n][H]
     EPI_FLOOR_I32 = 3    // p-stable, reference layout: int32 [T][n][H]
 };
+// `minmax` (EPI_FLOOR_I32 only, may be null): [T*H][2] words preset to INT_MAX / INT_MIN.  Where the
+// kernel can (H a multiple of 4, `out` and `b` 16-byte aligned) it folds the smallest and largest
+// hash of every column into them while it stores the hashes, and says so in *minmax_folded; else
+// the caller sweeps `out` itself.
 culsh_status launch_project_f32(culsh_ctx* ctx, const float* X, const float* P, const float* b,
-                                int n, int d, int T, int H, ProjEpilogue epi, void* out);
+                                int n, int d, int T, int H, ProjEpilogue epi, void* out,
+                                int32_t* minmax = nullptr, bool* minmax_folded = nullptr);
 culsh_status launch_project_f64(culsh_ctx* ctx, const double* X, const double* P, const double* b,
                                 int n, int d, int T, int H, ProjEpilogue epi, void* out);
 
@@ -266,8 +271,12 @@ culsh_status launch_keys_to_sig(culsh_ctx* ctx, const uint32_t* keys, size_t cou
 // ---------------------------------------------------------------- p-stable key compression (pscodec.hip)
 // Measures the value range of every (table, hash) of sig [T][n][H]; when the ranges are
 // narrow, fills ix->psc, sets ix->enc = ENC_PSC and ix->key_w, and reports compressed = true.
+// `mm_folded`: the ranges when the projection has folded them already ([T*H][2] from ps_minmax_prepare),
+// else null and sig is swept here.
 culsh_status ps_build_codec(culsh_ctx* ctx, const int32_t* sig, int n, int T, int H, culsh_index* ix,
-                            bool* compressed);
+                            bool* compressed, int32_t* mm_folded = nullptr);
+// [T*H][2] range words in the arena, preset to INT_MAX / INT_MIN
+culsh_status ps_minmax_prepare(culsh_ctx* ctx, int T, int H, int32_t** mm_dev);
 // int32 hashes [T][rows][H] -> compressed key words [T][rows][ix->key_w]
 culsh_status launch_ps_compress(culsh_ctx* ctx, const int32_t* sig, size_t rows, int T, int H, const culsh_index* ix,
                                 uint32_t* keys);

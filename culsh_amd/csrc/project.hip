@@ -4,6 +4,8 @@
 // pslsh/hash.cuh:104-142): X * P^T is computed with fp32 MFMA tiles and the sign /
 // floor epilogue is applied to the accumulators in registers, so the n x (T*H)
 // projection matrix is never written to memory.
+#include <climits>
+
 #include "common.hpp"
 
 namespace culsh_amd {
@@ -24,7 +26,12 @@ struct ProjArgs {
     int n, d, T, H;
     int n_row_tiles, n_col_tiles;
     int vec_x, vec_p;  // 16-byte vector loads allowed
+    int32_t* mm;       // EPI_FLOOR_I32_MM: [T*H][2] running minimum / maximum per column
 };
+
+// p-stable epilogue that also folds every column's smallest and largest hash into ProjArgs::mm
+// (kernel-internal: callers ask for EPI_FLOOR_I32 and pass the array)
+constexpr int EPI_FLOOR_I32_MM = 4;
 
 // Column order of the sign-packing epilogue.  Columns are grouped in tiles of 32 so that
 // one wavefront ballot over a 32-column MFMA tile yields key bits directly:
@@ -75,6 +82,14 @@ __global__ __launch_bounds__(NTHREADS, (BK <= 8 ? 5 : (BK <= 16 ? 4 : 3))) void 
     __shared__ __attribute__((aligned(16))) float As[BM * PITCH];
     __shared__ __attribute__((aligned(16))) float Bs[BN * PITCH];
     __shared__ uint32_t tw[(EPI == EPI_SIGN_KEYS) ? BM * (BN / 32) : 1];
+    constexpr bool FLOOR = (EPI == EPI_FLOOR_I32 || EPI == EPI_FLOOR_I32_MM);
+    constexpr bool FOLD_MM = (EPI == EPI_FLOOR_I32_MM);
+    constexpr int MM_PITCH = BN + 4;
+    __shared__ int32_t cmin[FOLD_MM ? 8 * MM_PITCH : 1], cmax[FOLD_MM ? 8 * MM_PITCH : 1];  // [8 copies][column of the tile]
+    if (FOLD_MM) {
+        for (int i = threadIdx.x; i < 8 * MM_PITCH; i += NTHREADS) { cmin[i] = INT_MAX; cmax[i] = INT_MIN; }
+        // the barriers of the stage loop stand between this and the epilogue (n_features > 0)
+    }
 
     // Workgroup -> (row tile, column tile).  Consecutive workgroup ids are dealt round
     // robin to the 8 XCDs; ids are arranged so that all column tiles of one row tile land
@@ -260,7 +275,7 @@ __global__ __launch_bounds__(NTHREADS, (BK <= 8 ? 5 : (BK <= 16 ? 4 : 3))) void 
         // When H is a multiple of 4 those are four neighbouring hashes of one table, stored at once;
         // the 32 lanes of a half wave then cover 32 consecutive rows, H * 4 bytes apart.
         const bool quad = (H & 3) == 0 && (reinterpret_cast<uintptr_t>(a.out) & 15) == 0 &&
-                          (EPI != EPI_FLOOR_I32 || (reinterpret_cast<uintptr_t>(a.b) & 15) == 0);
+                          (!FLOOR || (reinterpret_cast<uintptr_t>(a.b) & 15) == 0);
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
             const int cb = ct * BN + wn * 64 + j * 32 + 4 * half;  // column of register 0
@@ -271,7 +286,8 @@ __global__ __launch_bounds__(NTHREADS, (BK <= 8 ? 5 : (BK <= 16 ? 4 : 3))) void 
                 if (quad) {
                     if (c0 < TH) {
                         float4 bias = make_float4(0.f, 0.f, 0.f, 0.f);
-                        if (EPI == EPI_FLOOR_I32) bias = *reinterpret_cast<const float4*>(a.b + c0);
+                        if (FLOOR) bias = *reinterpret_cast<const float4*>(a.b + c0);
+                        int4 lo = make_int4(INT_MAX, INT_MAX, INT_MAX, INT_MAX), hi = make_int4(INT_MIN, INT_MIN, INT_MIN, INT_MIN);
 #pragma unroll
                         for (int i = 0; i < 2; ++i) {
                             const int row = rt * BM + wm * 64 + i * 32 + r32;
@@ -286,12 +302,25 @@ __global__ __launch_bounds__(NTHREADS, (BK <= 8 ? 5 : (BK <= 16 ? 4 : 3))) void 
                                                        (((__float_as_uint(x3) >> 31) ^ 1u) << 24);
                                 *reinterpret_cast<uint32_t*>(static_cast<uint8_t*>(a.out) + off) = bytes;
                             } else {  // pslsh/hash.cuh:46
-                                *reinterpret_cast<int4*>(static_cast<int32_t*>(a.out) + off) =
-                                    make_int4(static_cast<int32_t>(floorf(x0 + bias.x)),
-                                              static_cast<int32_t>(floorf(x1 + bias.y)),
-                                              static_cast<int32_t>(floorf(x2 + bias.z)),
-                                              static_cast<int32_t>(floorf(x3 + bias.w)));
+                                const int4 v = make_int4(static_cast<int32_t>(floorf(x0 + bias.x)),
+                                                         static_cast<int32_t>(floorf(x1 + bias.y)),
+                                                         static_cast<int32_t>(floorf(x2 + bias.z)),
+                                                         static_cast<int32_t>(floorf(x3 + bias.w)));
+                                *reinterpret_cast<int4*>(static_cast<int32_t*>(a.out) + off) = v;
+                                if (FOLD_MM) {
+                                    lo.x = min(lo.x, v.x); lo.y = min(lo.y, v.y); lo.z = min(lo.z, v.z); lo.w = min(lo.w, v.w);
+                                    hi.x = max(hi.x, v.x); hi.y = max(hi.y, v.y); hi.z = max(hi.z, v.z); hi.w = max(hi.w, v.w);
+                                }
                             }
+                        }
+                        if (FOLD_MM) {
+                            // the 32 lanes of a half wave hold 32 rows of the same four columns; eight copies of
+                            // the ranges (one per row residue, rows of MM_PITCH words: different banks) keep the
+                            // lanes that meet at one word down to four (sixteen copies measured no faster)
+                            int32_t* mn = &cmin[(r32 & 7) * MM_PITCH + (c0 - ct * BN)];
+                            int32_t* mx = &cmax[(r32 & 7) * MM_PITCH + (c0 - ct * BN)];
+                            atomicMin(mn, lo.x); atomicMin(mn + 1, lo.y); atomicMin(mn + 2, lo.z); atomicMin(mn + 3, lo.w);
+                            atomicMax(mx, hi.x); atomicMax(mx + 1, hi.y); atomicMax(mx + 2, hi.z); atomicMax(mx + 3, hi.w);
                         }
                     }
                 } else {
@@ -299,7 +328,7 @@ __global__ __launch_bounds__(NTHREADS, (BK <= 8 ? 5 : (BK <= 16 ? 4 : 3))) void 
 #pragma unroll
                     for (int q = 0; q < 4; ++q) {
                         if (c0 + q < TH) {
-                            const float bias = (EPI == EPI_FLOOR_I32) ? a.b[c0 + q] : 0.f;
+                            const float bias = FLOOR ? a.b[c0 + q] : 0.f;
 #pragma unroll
                             for (int i = 0; i < 2; ++i) {
                                 const int row = rt * BM + wm * 64 + i * 32 + r32;
@@ -319,6 +348,22 @@ __global__ __launch_bounds__(NTHREADS, (BK <= 8 ? 5 : (BK <= 16 ? 4 : 3))) void 
                 }
                 h += 8;
                 while (h >= H) { h -= H; ++t; }
+            }
+        }
+        if (FOLD_MM) {  // the tile's ranges into the table's, again only where they would change
+            __syncthreads();
+            const int c = ct * BN + tid;
+            if (tid < BN && c < TH) {
+                int32_t lo = INT_MAX, hi = INT_MIN;
+#pragma unroll
+                for (int k = 0; k < 8; ++k) {
+                    lo = min(lo, cmin[k * MM_PITCH + tid]);
+                    hi = max(hi, cmax[k * MM_PITCH + tid]);
+                }
+                if (lo <= hi) {
+                    if (lo < a.mm[2 * c]) atomicMin(&a.mm[2 * c], lo);
+                    if (hi > a.mm[2 * c + 1]) atomicMax(&a.mm[2 * c + 1], hi);
+                }
             }
         }
     }
@@ -534,7 +579,9 @@ __global__ __launch_bounds__(NTHREADS, 2) void project_f64_kernel(ProjArgs64 a) 
 }  // namespace
 
 culsh_status launch_project_f32(culsh_ctx* ctx, const float* X, const float* P, const float* b,
-                                int n, int d, int T, int H, ProjEpilogue epi, void* out) {
+                                int n, int d, int T, int H, ProjEpilogue epi, void* out, int32_t* minmax,
+                                bool* minmax_folded) {
+    if (minmax_folded) *minmax_folded = false;
     CULSH_REQUIRE(X && P && out, CULSH_ERR_INVALID, "projection: null pointer");
     CULSH_REQUIRE(n > 0 && d > 0 && T > 0 && H > 0, CULSH_ERR_INVALID, "projection: sizes must be positive");
     const bool floor_epi = (epi == EPI_FLOOR_I32);
@@ -557,6 +604,9 @@ culsh_status launch_project_f32(culsh_ctx* ctx, const float* X, const float* P, 
     a.n_col_tiles = static_cast<int>((n_vcols + BN - 1) / BN);
     a.vec_x = (d % 4 == 0) && (reinterpret_cast<uintptr_t>(X) % 16 == 0);
     a.vec_p = (d % 4 == 0) && (reinterpret_cast<uintptr_t>(P) % 16 == 0);
+    a.mm = minmax;
+    const bool fold_mm = floor_epi && minmax && minmax_folded && H % 4 == 0 &&
+                         reinterpret_cast<uintptr_t>(out) % 16 == 0 && reinterpret_cast<uintptr_t>(b) % 16 == 0;
     const long long groups = (a.n_row_tiles + 7) / 8;
     const long long blocks = groups * 8 * a.n_col_tiles;
     CULSH_REQUIRE(blocks < (1ll << 31), CULSH_ERR_LIMIT, "projection grid too large");
@@ -570,11 +620,13 @@ culsh_status launch_project_f32(culsh_ctx* ctx, const float* X, const float* P, 
         else if (vec) CULSH_LAUNCH(ctx, (project_f32_kernel<E, true, 16, false>), grid, block, 0, ctx->stream, a);         \
         else CULSH_LAUNCH(ctx, (project_f32_kernel<E, false, 16, false>), grid, block, 0, ctx->stream, a);                 \
         break;
-    switch (epi) {
+    switch (fold_mm ? EPI_FLOOR_I32_MM : static_cast<int>(epi)) {
         PROJ_CASE(EPI_SIGN_KEYS)
         PROJ_CASE(EPI_SIGN_BYTES)
         PROJ_CASE(EPI_FLOOR_I32)
+        PROJ_CASE(EPI_FLOOR_I32_MM)
     }
+    if (fold_mm) *minmax_folded = true;
 #undef PROJ_CASE
     CULSH_LAUNCH_CHECK();
     return CULSH_OK;

@@ -248,17 +248,23 @@ void free_ps_codec(culsh_index* ix) {
     ix->psc = PsCodec();
 }
 
+culsh_status ps_minmax_prepare(culsh_ctx* ctx, int T, int H, int32_t** mm_dev) {
+    const int TH = T * H;
+    CULSH_TRY(arena_alloc_t(ctx, static_cast<size_t>(TH) * 2, mm_dev));
+    CULSH_LAUNCH(ctx, ps_minmax_reset_kernel, dim3(div_up(static_cast<size_t>(TH), 256)), dim3(256), 0, ctx->stream,
+                 *mm_dev, TH);
+    CULSH_LAUNCH_CHECK();
+    return CULSH_OK;
+}
+
 culsh_status ps_build_codec(culsh_ctx* ctx, const int32_t* sig, int n, int T, int H, culsh_index* ix,
-                            bool* compressed) {
+                            bool* compressed, int32_t* mm_folded) {
     *compressed = false;
     const int TH = T * H;
     if (H > 1024) return CULSH_OK;
-    int32_t* mm_dev = nullptr;
-    CULSH_TRY(arena_alloc_t(ctx, static_cast<size_t>(TH) * 2, &mm_dev));
-    CULSH_LAUNCH(ctx, ps_minmax_reset_kernel, dim3(div_up(static_cast<size_t>(TH), 256)), dim3(256), 0, ctx->stream,
-                 mm_dev, TH);
-    CULSH_LAUNCH_CHECK();
-    {
+    int32_t* mm_dev = mm_folded;
+    if (!mm_dev) {
+        CULSH_TRY(ps_minmax_prepare(ctx, T, H, &mm_dev));
         const size_t per_table = static_cast<size_t>(n) * H;
         const bool vec4 = H % 4 == 0 && 1024 % H == 0 && reinterpret_cast<uintptr_t>(sig) % 16 == 0;
         const unsigned bx = std::max(1u, std::min(256u, div_up(per_table, 256 * (vec4 ? 64 : 16))));

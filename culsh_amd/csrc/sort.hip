@@ -553,8 +553,7 @@ culsh_status sort_tables(culsh_ctx* ctx, uint32_t* keys_in, uint32_t* keys_tmp, 
             // about four workgroups per CU over all tables
             const int per_table = std::max(1, std::min((n + TOT_TILE - 1) / TOT_TILE, (4 * ctx->n_cus + T - 1) / T));
             // as many histogram copies as 60 KiB hold, eight at most
-            static const int lds_kb = [] { const char* e = std::getenv("CULSH_TOTALS_LDS_KB"); return e && *e ? std::atoi(e) : 60; }();
-            const int copies = std::max(1, std::min(8, (lds_kb * 1024) / (pl.count * TOT_ROW * 4)));
+            const int copies = std::max(1, std::min(8, (60 * 1024) / (pl.count * TOT_ROW * 4)));
             const size_t lds = static_cast<size_t>(copies) * pl.count * TOT_ROW * sizeof(uint32_t);
             CULSH_LAUNCH(ctx, radix_totals_kernel, dim3(per_table, T), dim3(SORT_THREADS), lds, ctx->stream, keys_in, n, W, pl,
                          T, copies, dtot + static_cast<size_t>(p0) * T * 256);
