@@ -222,9 +222,9 @@ def main() -> int:
                                  "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
                                  "frac": round(achieved / PEAK_HBM_GBS, 4)})
 
-    # ---- what a plain streaming copy reaches on this box (256 MiB -> 256 MiB, torch's copy kernel, HIP
+    # ---- what a plain streaming copy reaches on this box (1 GiB -> 1 GiB, torch's copy kernel, HIP
     # events on torch's stream): the practical ceiling next to the 8 TB/s peak
-    ca = torch.empty(1 << 26, dtype=torch.int32, device="cuda")
+    ca = torch.empty(1 << 28, dtype=torch.int32, device="cuda")
     cb = torch.empty_like(ca)
     for _ in range(3):
         cb.copy_(ca)
@@ -305,7 +305,7 @@ def main() -> int:
         "roofline_kernels_note": "algorithmic HBM bytes of this run (N items, B buckets, R raw and U unique candidates "
                                  f"= {N}, {B}, {R}, {U}) over the HIP-event time of this run's untimed detail steps",
         "hbm_copy": {"achieved": round(copy_gbs, 1), "unit": "GB/s", "frac": round(copy_gbs / PEAK_HBM_GBS, 4),
-                     "note": "plain device-to-device copy of 256 MiB (read + write bytes over time) in this run; "
+                     "note": "plain device-to-device copy of 1 GiB (read + write bytes over time) in this run; "
                              "roofline_kernels[].frac_of_copy relates each kernel to it"},
         "first_call": first_call,
         "cpu_baseline": cpu, "parity": parity,
