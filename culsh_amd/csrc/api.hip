@@ -299,18 +299,16 @@ static culsh_status upload(const T* host, size_t count, T** dev) {
     return CULSH_OK;
 }
 
-// Hash parameters go through pinned staging and an asynchronous copy on the context's stream:
-// the kernels queued behind it see the data, and the host does not wait for the copy.
-template <typename T>
-static culsh_status upload_params(culsh_ctx* ctx, const T* host, size_t count, T** dev) {
-    *dev = nullptr;
-    if (count == 0) return CULSH_OK;
-    const size_t bytes = count * sizeof(T);
-    CULSH_HIP(dev_malloc(dev, bytes));
+// Small host arrays (hash parameters, rank tables) go through pinned staging and an asynchronous copy
+// on the context's stream: the kernels queued behind it see the data, and the host does not wait for
+// the copy.  The staging area is filled from param_stage_off on, which every fit resets at its start
+// (the stream is idle then, so nothing reads the area any more).
+culsh_status upload_async(culsh_ctx* ctx, const void* host, size_t bytes, void* dev) {
+    if (bytes == 0) return CULSH_OK;
     const size_t need = ctx->param_stage_off + align_up(bytes, 256);
     if (need > ctx->param_stage_cap) {
         if (ctx->param_stage_off != 0 || bytes > (size_t(64) << 20)) {  // staging in use or not worth pinning
-            CULSH_HIP(hipMemcpy(*dev, host, bytes, hipMemcpyHostToDevice));
+            CULSH_HIP(hipMemcpy(dev, host, bytes, hipMemcpyHostToDevice));
             return CULSH_OK;
         }
         if (ctx->param_stage) (void)hipHostFree(ctx->param_stage);
@@ -320,7 +318,7 @@ static culsh_status upload_params(culsh_ctx* ctx, const T* host, size_t count, T
         if (hipHostMalloc(reinterpret_cast<void**>(&ctx->param_stage), cap, hipHostMallocDefault) != hipSuccess) {
             (void)hipGetLastError();
             ctx->param_stage = nullptr;
-            CULSH_HIP(hipMemcpy(*dev, host, bytes, hipMemcpyHostToDevice));
+            CULSH_HIP(hipMemcpy(dev, host, bytes, hipMemcpyHostToDevice));
             return CULSH_OK;
         }
         ctx->param_stage_cap = cap;
@@ -328,8 +326,16 @@ static culsh_status upload_params(culsh_ctx* ctx, const T* host, size_t count, T
     char* slot = ctx->param_stage + ctx->param_stage_off;
     std::memcpy(slot, host, bytes);
     ctx->param_stage_off += align_up(bytes, 256);
-    CULSH_HIP(hipMemcpyAsync(*dev, slot, bytes, hipMemcpyHostToDevice, ctx->stream));
+    CULSH_HIP(hipMemcpyAsync(dev, slot, bytes, hipMemcpyHostToDevice, ctx->stream));
     return CULSH_OK;
+}
+
+template <typename T>
+static culsh_status upload_params(culsh_ctx* ctx, const T* host, size_t count, T** dev) {
+    *dev = nullptr;
+    if (count == 0) return CULSH_OK;
+    CULSH_HIP(dev_malloc(dev, count * sizeof(T)));
+    return upload_async(ctx, host, count * sizeof(T), *dev);
 }
 
 // `with_query`: the fit is followed by a query of the fitted rows (fit_query), which has the query path's

@@ -223,6 +223,9 @@ void profile_collect(culsh_ctx* ctx);  // call with the stream idle
         hipLaunchKernelGGL(kernel, __VA_ARGS__);          \
     } while (0)
 
+// Copies a small host array to device memory through pinned staging, asynchronously on the context's
+// stream (api.hip); only valid inside a fit, which resets the staging area at its start.
+culsh_status upload_async(culsh_ctx* ctx, const void* host, size_t bytes, void* dev);
 // Reads `count` (<= 64) device u64/u32 words into host memory; synchronises the stream.
 culsh_status read_back_u64(culsh_ctx* ctx, const uint64_t* dev, int count, uint64_t* host);
 culsh_status read_back_u32(culsh_ctx* ctx, const uint32_t* dev, int count, uint32_t* host);

@@ -317,7 +317,7 @@ culsh_status ps_build_codec(culsh_ctx* ctx, const int32_t* sig, int n, int T, in
     pc.range = block + TH;
     pc.fwd = reinterpret_cast<uint32_t*>(block + 2 * static_cast<size_t>(TH));
     pc.inv = block + 2 * static_cast<size_t>(TH) + lut;
-    CULSH_HIP(hipMemcpy(block, host.data(), host.size() * sizeof(int32_t), hipMemcpyHostToDevice));
+    CULSH_TRY(upload_async(ctx, host.data(), host.size() * sizeof(int32_t), block));  // staged: `host` may go
     ix->enc = ENC_PSC;
     ix->key_w = W;
     *compressed = true;
