@@ -555,6 +555,12 @@ culsh_status sort_tables(culsh_ctx* ctx, uint32_t* keys_in, uint32_t* keys_tmp, 
             // as many histogram copies as 60 KiB hold, eight at most
             const int copies = std::max(1, std::min(8, (60 * 1024) / (pl.count * TOT_ROW * 4)));
             const size_t lds = static_cast<size_t>(copies) * pl.count * TOT_ROW * sizeof(uint32_t);
+            static bool configured[64] = {};  // per device: more LDS than a launch may ask for by default
+            if (lds > 48 * 1024 && !configured[ctx->device & 63]) {
+                CULSH_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(radix_totals_kernel),
+                                              hipFuncAttributeMaxDynamicSharedMemorySize, 60 * 1024));
+                configured[ctx->device & 63] = true;
+            }
             CULSH_LAUNCH(ctx, radix_totals_kernel, dim3(per_table, T), dim3(SORT_THREADS), lds, ctx->stream, keys_in, n, W, pl,
                          T, copies, dtot + static_cast<size_t>(p0) * T * 256);
             CULSH_LAUNCH_CHECK();
