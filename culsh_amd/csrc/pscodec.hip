@@ -348,9 +348,11 @@ culsh_status launch_ps_keys_to_sig(culsh_ctx* ctx, const culsh_index* ix, size_t
     if (count == 0) return CULSH_OK;
     const PsCodec& pc = ix->psc;
     const size_t lut_words = 2 * static_cast<size_t>(ix->n_hashes) * pc.rmax;
-    const int use_lds = lut_words <= PS_LUT_WORDS;
     // buckets per workgroup: as many as 16 KiB of key words hold, 256 to 2048
     const int bpb = std::max(PS_BPB_MIN, std::min(2048, (4096 / ix->key_w) / 256 * 256));
+    // the value tables go to LDS when they are small and fit beside the key words
+    const int use_lds = lut_words <= PS_LUT_WORDS &&
+                        (2 + static_cast<size_t>(bpb) * ix->key_w + lut_words) * sizeof(uint32_t) <= 64 * 1024;
     CULSH_REQUIRE(count / bpb < (1ull << 31), CULSH_ERR_LIMIT, "too many buckets");
     const size_t lds = (2 + static_cast<size_t>(bpb) * ix->key_w + (use_lds ? lut_words : 0)) * sizeof(uint32_t);
     CULSH_REQUIRE(lds <= 64 * 1024, CULSH_ERR_LIMIT, "key width too large for the signature restore kernel");

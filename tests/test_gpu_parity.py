@@ -686,6 +686,26 @@ def test_pslsh_fit_query_path(ctx, dtype):
         ctx.free_index(h)
 
 
+def test_pslsh_many_hashes_narrow_ranges(ctx):
+    """896 hashes of two or three values each: rank keys of 56 words, the widest the signature restore
+    kernel takes, with value tables that no longer fit into LDS beside them."""
+    _announce("pslsh_many_hashes")
+    n, d, T, H, nq, w = 400, 16, 2, 896, 40, 64
+    rng = np.random.default_rng(8)
+    X = rng.standard_normal((n, d)).astype(np.float32)
+    Q = X[:nq].copy()
+    P, b = o.generate_random_projections_biases(7, T * H, d, w, np.float32)
+    from abi import assert_candidates_match, assert_index_matches
+
+    sig = ctx.pslsh_hash(X, P, b, T, H)
+    assert 2 <= int(sig.max()) - int(sig.min()) + 1 <= 3
+    ih = ctx.pslsh_fit(X, T, H, w, seed=7, P=P, b=b)
+    exp_ix = o.fit_index(sig, H)
+    assert_index_matches(ctx.index_arrays(ih), exp_ix)
+    assert_candidates_match(ctx.pslsh_query(Q, ih), o.query_index(ctx.pslsh_hash(Q, P, b, T, H), exp_ix))
+    ctx.free_index(ih)
+
+
 def test_minhash_fit_query_path(ctx):
     _announce("minhash_path")
     rng = np.random.default_rng(77)
