@@ -80,12 +80,15 @@ def _copy(ptr, n, dtype):
     return np.ctypeslib.as_array(ptr, shape=(n,)).astype(dtype, copy=True)
 
 
-def rplsh_hash(X: np.ndarray, P: np.ndarray, T: int, H: int) -> np.ndarray:
+def rplsh_hash(X: np.ndarray, P: np.ndarray, T: int, H: int, blocked: bool = False) -> np.ndarray:
+    """`blocked` (fp32): the cache- and vector-blocked form, bit-identical to the plain one."""
     n, d = X.shape
     sig = np.empty((T, n, H), dtype=np.uint8)
     X = np.ascontiguousarray(X)
     P = np.ascontiguousarray(P, dtype=X.dtype)
     fn = lib().oracle_rplsh_hash_f32 if X.dtype == np.float32 else lib().oracle_rplsh_hash_f64
+    if blocked and X.dtype == np.float32:
+        fn = lib().oracle_rplsh_hash_f32_blocked
     fn(_p(X), _p(P), n, d, T, H, _p(sig))
     return sig
 

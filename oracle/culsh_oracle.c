@@ -64,6 +64,51 @@ void oracle_rplsh_hash_f32(const float* X, const float* P, int n, int d, int T, 
     }
 }
 
+/* The same function blocked for the registers and the vector units: P is repacked once into panels
+ * of CB columns ([panel][feature][CB]), and a block of RB rows x CB columns is accumulated in
+ * registers over all features.  Every output is still the sum of its products in feature order, one
+ * rounding per product and per addition (no contraction in ISO C mode), so the result equals
+ * oracle_rplsh_hash_f32 bit for bit; tests require that. */
+void oracle_rplsh_hash_f32_blocked(const float* X, const float* P, int n, int d, int T, int H,
+                                   uint8_t* sig) {
+    enum { RB = 4, CB = 16 };
+    const int TH = T * H;
+    const int panels = (TH + CB - 1) / CB;
+    float* Pp = (float*)calloc((size_t)panels * d * CB, sizeof(float));
+    if (!Pp) {  /* no scratch: the plain way */
+        oracle_rplsh_hash_f32(X, P, n, d, T, H, sig);
+        return;
+    }
+    for (int c = 0; c < TH; ++c)
+        for (int k = 0; k < d; ++k) Pp[((size_t)(c / CB) * d + k) * CB + c % CB] = P[(size_t)c * d + k];
+#pragma omp parallel for schedule(static)
+    for (int r0 = 0; r0 < n; r0 += RB) {
+        const int rows = n - r0 < RB ? n - r0 : RB;
+        const float* x[RB];
+        for (int rr = 0; rr < RB; ++rr) x[rr] = X + (size_t)(r0 + (rr < rows ? rr : 0)) * d;  /* spare rows repeat the first */
+        for (int p = 0; p < panels; ++p) {
+            const float* pp = Pp + (size_t)p * d * CB;
+            float acc[RB][CB];
+            for (int rr = 0; rr < RB; ++rr)
+                for (int j = 0; j < CB; ++j) acc[rr][j] = 0.0f;
+            for (int k = 0; k < d; ++k)
+                for (int rr = 0; rr < RB; ++rr) {
+                    const float xv = x[rr][k];
+                    for (int j = 0; j < CB; ++j) acc[rr][j] += xv * pp[(size_t)k * CB + j];
+                }
+            for (int rr = 0; rr < rows; ++rr)
+                for (int j = 0; j < CB && p * CB + j < TH; ++j) {
+                    const int c = p * CB + j;
+                    uint32_t bits;
+                    memcpy(&bits, &acc[rr][j], 4);
+                    const int t = c / H, h = c % H;
+                    sig[(size_t)t * n * H + (size_t)(r0 + rr) * H + h] = (uint8_t)((bits >> 31) ^ 1u);
+                }
+        }
+    }
+    free(Pp);
+}
+
 void oracle_rplsh_hash_f64(const double* X, const double* P, int n, int d, int T, int H,
                            uint8_t* sig) {
     const int TH = T * H;

@@ -277,6 +277,23 @@ def test_rplsh_hash_matches_reference_test_model(dtype, c_oracle):
     assert safe.mean() > 0.999
 
 
+@pytest.mark.parametrize("shape", [(1, 1, 1, 1), (7, 3, 2, 5), (1003, 37, 5, 7), (258, 128, 32, 16)])
+def test_blocked_cpu_projection_equals_the_plain_one(shape, c_oracle):
+    """The blocked projection that the CPU baseline times keeps every output's summation order, so it
+    must agree with the plain loop bit for bit: on random data, on rows and columns that do not fill a
+    block, and on the signed zeros of all-zero rows and all-zero hash vectors."""
+    n, d, T, H = shape
+    rng = np.random.default_rng(n + d)
+    X = rng.standard_normal((n, d)).astype(np.float32)
+    P = rng.standard_normal((T * H, d)).astype(np.float32)
+    X[0] = 0.0
+    P[-1] = 0.0
+    X[-1] = -np.abs(X[-1])          # x < 0 against p = 0 gives -0.0
+    plain = c_oracle.rplsh_hash(X, P, T, H)
+    np.testing.assert_array_equal(c_oracle.rplsh_hash(X, P, T, H, blocked=True), plain)
+    np.testing.assert_array_equal(plain[:, 0, :], 1)      # the zero row: +0.0 everywhere
+
+
 @pytest.mark.parametrize("dtype", [np.float32, np.float64])
 def test_pslsh_hash_matches_reference_test_model(dtype, c_oracle):
     """ref_lsh.py:275-279: floor((X @ P.T + b) / w) with b ~ U[0,w); the reference core
