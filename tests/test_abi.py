@@ -111,3 +111,38 @@ def test_minhash_generator_matches_definition():
     np.testing.assert_array_equal(A, A_ref)
     np.testing.assert_array_equal(B, B_ref)
     assert A.min() >= 1 and int(A.max()) <= o.MINHASH_PRIME - 1 and int(B.max()) <= o.MINHASH_PRIME - 1
+
+
+def test_header_is_plain_c_and_links_from_a_c_program(tmp_path):
+    """The boundary is a C ABI: the header compiles as strict C99 and as C++11, and a C program that
+    includes it links against the library and calls it (no device work: version string, and a context
+    request for a device that does not exist, which must come back as an error code)."""
+    import shutil
+    import subprocess
+
+    if not shutil.which("gcc"):
+        pytest.skip("no C compiler")
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    src = tmp_path / "host.c"
+    src.write_text(
+        '#include <stdio.h>\n#include <string.h>\n#include "culsh_amd.h"\n'
+        "int main(void) {\n"
+        "    culsh_ctx* ctx = NULL;\n"
+        '    if (strncmp(culsh_version(), "culsh_amd", 9) != 0) return 2;\n'
+        "    if (culsh_ctx_create(4096, &ctx) == CULSH_OK) return 3;\n"
+        "    if (ctx != NULL) return 4;\n"
+        '    if (culsh_last_error() == NULL || strlen(culsh_last_error()) == 0) return 5;\n'
+        '    puts("ok");\n    return 0;\n}\n')
+    inc = os.path.join(root, "include")
+    subprocess.run(["gcc", "-std=c99", "-pedantic", "-Wall", "-Wextra", "-Werror", "-I", inc, "-c", str(src),
+                    "-o", str(tmp_path / "host.o")], check=True)
+    subprocess.run(["g++", "-std=c++11", "-Wall", "-Wextra", "-Werror", "-I", inc, "-x", "c++", "-c", str(src),
+                    "-o", str(tmp_path / "host_cxx.o")], check=True)
+    libdir = os.path.join(root, "culsh_amd")
+    exe = tmp_path / "host"
+    rocm = "/opt/rocm/lib"
+    subprocess.run(["gcc", str(tmp_path / "host.o"), "-L", libdir, "-lculsh_amd", "-L", rocm,
+                    "-Wl,-rpath," + libdir, "-Wl,-rpath," + rocm, "-Wl,--allow-shlib-undefined", "-o", str(exe)],
+                   check=True)
+    out = subprocess.run([str(exe)], capture_output=True, text=True, timeout=60)
+    assert out.returncode == 0 and out.stdout.strip() == "ok", (out.returncode, out.stdout, out.stderr)
