@@ -286,6 +286,7 @@ __device__ __forceinline__ void number_pieces(uint32_t pieces, int T, uint32_t* 
     }
 }
 
+constexpr int SPARSE_WORDS = 2;  // a pass is read out through the summary when its range has this many bitmap words per row, or more
 constexpr int SPLIT_BATCH = 3;  // row bounds located per search round of split_spans
 
 // The rows of a span ascend.  For every span t < T and each of the K row bounds bound0 + k * chunk_rows
@@ -410,7 +411,8 @@ __global__ __launch_bounds__(DD_THREADS) void dedup_kernel(DedupArgs a) {
     const int T = a.T, tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int chunk_words = DD_THREADS * a.wpt;                  // multiple of 1024
     uint32_t* bm = lds;                                          // [chunk_words]
-    unsigned long long* sh_base = reinterpret_cast<unsigned long long*>(bm + chunk_words);  // [1]
+    uint32_t* sm = bm + chunk_words;                             // [chunk_words / 32] one bit per non-zero bitmap word (sparse passes)
+    unsigned long long* sh_base = reinterpret_cast<unsigned long long*>(sm + chunk_words / 32);  // [1]
     int* sh_q = reinterpret_cast<int*>(sh_base + 1);             // [2] query handed to the workgroup
     int2* tab = reinterpret_cast<int2*>(sh_base + 2);            // [DD_THREADS]
     int* s_start = reinterpret_cast<int*>(tab + DD_THREADS);     // [T]
@@ -439,7 +441,7 @@ __global__ __launch_bounds__(DD_THREADS) void dedup_kernel(DedupArgs a) {
     if (FUSED && tid == 0) *sh_q = static_cast<int>(atomicAdd(a.ticket, 1u));
     {   // the bitmap is cleared while the first loads are in flight; FUSED keeps it clean afterwards
         uint4* bm4 = reinterpret_cast<uint4*>(bm);
-        for (int i = tid; i < chunk_words / 4; i += DD_THREADS) bm4[i] = make_uint4(0u, 0u, 0u, 0u);
+        for (int i = tid; i < (chunk_words + chunk_words / 32) / 4; i += DD_THREADS) bm4[i] = make_uint4(0u, 0u, 0u, 0u);
     }
     if (FUSED) {
         __syncthreads();
@@ -513,6 +515,20 @@ __global__ __launch_bounds__(DD_THREADS) void dedup_kernel(DedupArgs a) {
         DD_TICK(0)  // setup + clear
         // Mark the rows of this pass (collect_candidates_kernel, core/query.cuh:199-237, but into
         // the bitmap instead of memory).  Rows outside [lo, lo + chunk_rows) belong to another pass.
+        // Several passes per query: a pass with few rows for its range (its pieces hold at most one row per
+        // SPARSE_WORDS bitmap words) is read out through a summary: the thread that finds a bitmap word
+        // empty also sets that word's bit in `sm`, and the read-out visits the words that have one
+        // instead of sweeping the whole range.  (Not with one pass per query: there the chained scan's
+        // look-back runs under the sweep, and without the sweep the waits for predecessors pile up and
+        // cost more than the sweep did.)
+        const bool sparse = several && static_cast<size_t>(n_pieces) * 64u * SPARSE_WORDS <= static_cast<size_t>(chunk_words);
+        auto mark_sparse = [&](int row) {
+            const uint32_t bit = static_cast<uint32_t>(row) - lo;
+            if (bit < chunk_rows) {
+                const uint32_t m = 1u << (bit & 31u), w = bit >> 5;
+                if (atomicOr(&bm[bitmap_slot(w, swap_mask)], m) == 0u) atomicOr(&sm[w >> 5], 1u << (w & 31u));
+            }
+        };
         uint32_t fresh = 0;  // COUNT: bits this thread set first
         auto mark = [&](int row) {
             const uint32_t bit = static_cast<uint32_t>(row) - lo;
@@ -525,7 +541,8 @@ __global__ __launch_bounds__(DD_THREADS) void dedup_kernel(DedupArgs a) {
                 }
             }
         };
-        walk_candidates(a.cand, s_start, s_len, s_ppref, T, n_pieces, tab, mark);
+        if (sparse) walk_candidates(a.cand, s_start, s_len, s_ppref, T, n_pieces, tab, mark_sparse);
+        else walk_candidates(a.cand, s_start, s_len, s_ppref, T, n_pieces, tab, mark);
         DD_TICK(1)  // gather
         if (MODE == DD_COUNT) {
             // a row is counted by whichever lane set its bit first
@@ -545,7 +562,18 @@ __global__ __launch_bounds__(DD_THREADS) void dedup_kernel(DedupArgs a) {
         // count is published before the line-up.  Several passes: nobody waits for the count, and the
         // line-up's own totals serve.
         uint32_t wave_total = 0;
-        for (int i = lane; !several && i < wpw / 4; i += 64) {  // in any order: contiguous reads
+        // Sparse pass: lane l owns the 32 consecutive words [32 l, 32 l + 32) of the wavefront's part and
+        // the summary word that stands for them; row order = (wave, lane, word, bit).
+        uint32_t sp_words = 0, sp_before = 0;  // this lane's summary word; rows of the lower lanes
+        if (sparse) {
+            if (lane < wpw / 32) sp_words = sm[wave * (wpw / 32) + lane];
+            uint32_t c = 0;
+            for (uint32_t left = sp_words; left; left &= left - 1u)
+                c += __popc(wbm[bitmap_slot(static_cast<uint32_t>(lane * 32 + __ffs(static_cast<int>(left)) - 1), swap_mask)]);
+            sp_before = wave_inclusive_sum_dpp(c) - c;
+            wave_total = c;
+        }
+        for (int i = lane; !sparse && !several && i < wpw / 4; i += 64) {  // in any order: contiguous reads
             const uint4 v = reinterpret_cast<const uint4*>(wbm)[i];
             wave_total += __popc(v.x) + __popc(v.y) + __popc(v.z) + __popc(v.w);
         }
@@ -579,9 +607,10 @@ __global__ __launch_bounds__(DD_THREADS) void dedup_kernel(DedupArgs a) {
         // position of the query's list for this.  A dense step (more rows than slots) is left alone.
         const uint32_t region = 64u * ew;  // words (= list slots) a step covers
         uint32_t st_total[4] = {0u, 0u, 0u, 0u};  // steps <= 4 for every geometry
+        if (sparse && several) st_total[0] = wave_sum(wave_total);
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-            if (j >= steps) break;
+            if (sparse || j >= steps) break;
             const int w0 = (j * 64 + lane) * ew;
             uint32_t* sreg = wbm + j * region;
             uint32_t words[8];
@@ -659,7 +688,24 @@ __global__ __launch_bounds__(DD_THREADS) void dedup_kernel(DedupArgs a) {
             if (last) q_next = *sh_q;
         }
         DD_TICK(2)  // count, line-up (+ look-back)
-        if (store) {
+        if (sparse) {
+            // every lane writes the rows of its own words where the lower lanes' rows end, and leaves the
+            // words and its summary word clean (also when nothing may be stored)
+            int32_t* dst = a.out + base + wave_base + sp_before;
+            const uint32_t row_base = lo + (static_cast<uint32_t>(wave * wpw + lane * 32) << 5);
+            for (uint32_t left = sp_words; left; left &= left - 1u) {
+                const uint32_t k = static_cast<uint32_t>(__ffs(static_cast<int>(left)) - 1);
+                uint32_t* word = &wbm[bitmap_slot(static_cast<uint32_t>(lane * 32) + k, swap_mask)];
+                uint32_t bits = *word;
+                *word = 0u;
+                const uint32_t r0 = row_base + (k << 5);
+                while (bits && store) {
+                    *dst++ = static_cast<int32_t>(r0 + (__ffs(static_cast<int>(bits)) - 1));
+                    bits &= bits - 1u;
+                }
+            }
+            if (sp_words) sm[wave * (wpw / 32) + lane] = 0u;
+        } else if (store) {
             int32_t* dst = a.out + base + wave_base;
             __builtin_amdgcn_wave_barrier();  // LDS accesses of one wavefront complete in order
 #pragma unroll
@@ -690,7 +736,7 @@ __global__ __launch_bounds__(DD_THREADS) void dedup_kernel(DedupArgs a) {
                 dst += st_total[j];
             }
         }
-        if (FUSED) {  // leave this wavefront's part of the bitmap clean for the next query
+        if (FUSED && !sparse) {  // leave this wavefront's part of the bitmap clean for the next query
             uint4* z = reinterpret_cast<uint4*>(wbm);
             for (int i = lane; i < wpw / 4; i += 64) z[i] = make_uint4(0u, 0u, 0u, 0u);
         }
@@ -770,7 +816,8 @@ culsh_status dedup_geometry(const culsh_ctx* ctx, const culsh_index* index, Dedu
     for (int several = 0; several < 2; ++several) {
         const size_t per_table = several ? 5 + SPLIT_BATCH : 3;
         const size_t fixed = (4 + per_table * T + 1 + 2 * DD_THREADS + 17 + (NWAVES + 1) + 8) * sizeof(uint32_t);
-        auto lds_need = [&](int w) { return static_cast<size_t>(DD_THREADS) * w * 4 + fixed; };
+        // bitmap, its summary (one bit per bitmap word), the rest
+        auto lds_need = [&](int w) { return static_cast<size_t>(DD_THREADS) * w * 4 + static_cast<size_t>(DD_THREADS) * w / 8 + fixed; };
         int wpt_max = 1;
         while (wpt_max * 2 <= wpt_limit && lds_need(wpt_max * 2) <= static_cast<size_t>(ctx->lds_max)) wpt_max *= 2;
         int wpt = 1;

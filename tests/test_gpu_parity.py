@@ -408,6 +408,40 @@ def test_core_query_bitmap_passes_long_spans_many_tables(ctx, c_oracle, monkeypa
     ctx.free_index(ih)
 
 
+def test_core_query_sparse_passes_at_full_bitmap_size(ctx, c_oracle):
+    """1.1M rows: two passes per query over the full-size bitmap (2^20 rows, eight words per lane and
+    step).  Passes that hold few rows for their range are read out through the summary of non-zero
+    words: buckets of rows that sit in one word, fill words completely, sit at both ends of a word, of
+    a lane's 32 words and of a pass, straddle the pass boundary, or are the index's last row; next to a
+    query whose passes are dense (read out by the sweep) and one without candidates."""
+    _announce("sparse_passes_full_bitmap")
+    rng = np.random.default_rng(79)
+    T, n, nq, H = 3, 1_100_000, 12, 1
+    sig = rng.integers(0, 2, size=(T, n, H)).astype(np.uint8)            # two big buckets per table: dense passes
+    edge = 1 << 20
+    groups = {
+        10: np.arange(edge - 70, edge + 70),                             # across the pass boundary, whole words
+        11: np.array([0, 31, 32, 63, 1023, 1024, edge - 1, edge, n - 1]),
+        12: np.arange(4096, 4096 + 32),                                  # exactly one word
+        13: np.array([5, 5 + 64, 5 + 2 * 64, 700_000, 700_001, n - 2]),
+        14: np.arange(edge + 1000, edge + 1000 + 300, 3),
+    }
+    for value, rows in groups.items():
+        sig[:, rows, 0] = value
+    sig[1, groups[12], 0] = 15                                            # table 1 splits one group in two
+    sig[1, groups[12][::2], 0] = 16
+    qsig = np.zeros((T, nq, H), dtype=np.uint8)
+    for i, value in enumerate([10, 11, 12, 13, 14, 15, 16, 0, 1, 200, 12, 10]):
+        qsig[:, i, 0] = value
+    qsig[2, 10, 0] = 13                                                   # different small buckets per table
+    qsig[0, 11, 0] = 1                                                    # a dense span beside sparse ones
+    ih, _ = ctx.core_fit_index(sig, H)
+    from abi import assert_candidates_match
+
+    assert_candidates_match(ctx.core_query_index(qsig, ih), c_oracle.query_index_c(qsig, c_oracle.fit_index_c(sig, H)))
+    ctx.free_index(ih)
+
+
 def test_core_query_two_launch_path(ctx, monkeypatch):
     """The count / scan / emit path (taken for row ranges beyond one bitmap pass) on a small case."""
     _announce("two_launch_path")
