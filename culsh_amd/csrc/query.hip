@@ -516,17 +516,19 @@ __global__ __launch_bounds__(DD_THREADS) void dedup_kernel(DedupArgs a) {
         // Mark the rows of this pass (collect_candidates_kernel, core/query.cuh:199-237, but into
         // the bitmap instead of memory).  Rows outside [lo, lo + chunk_rows) belong to another pass.
         // Several passes per query: a pass with few rows for its range (its pieces hold at most one row per
-        // SPARSE_WORDS bitmap words) is read out through a summary: the thread that finds a bitmap word
-        // empty also sets that word's bit in `sm`, and the read-out visits the words that have one
-        // instead of sweeping the whole range.  (Not with one pass per query: there the chained scan's
-        // look-back runs under the sweep, and without the sweep the waits for predecessors pile up and
-        // cost more than the sweep did.)
+        // SPARSE_WORDS bitmap words) is read out through a summary: every mark also sets its bitmap word's
+        // bit in `sm`, and the read-out visits the words that have one instead of sweeping the whole
+        // range.  (Not with one pass per query: there the chained scan's look-back runs under the sweep,
+        // and without the sweep the waits for predecessors pile up and cost more than the sweep did.)
         const bool sparse = several && static_cast<size_t>(n_pieces) * 64u * SPARSE_WORDS <= static_cast<size_t>(chunk_words);
         auto mark_sparse = [&](int row) {
             const uint32_t bit = static_cast<uint32_t>(row) - lo;
             if (bit < chunk_rows) {
                 const uint32_t m = 1u << (bit & 31u), w = bit >> 5;
-                if (atomicOr(&bm[bitmap_slot(w, swap_mask)], m) == 0u) atomicOr(&sm[w >> 5], 1u << (w & 31u));
+                // both without a returned value: waiting for the first one's answer to decide on the
+                // second costs more than the second
+                atomicOr(&bm[bitmap_slot(w, swap_mask)], m);
+                atomicOr(&sm[w >> 5], 1u << (w & 31u));
             }
         };
         uint32_t fresh = 0;  // COUNT: bits this thread set first
