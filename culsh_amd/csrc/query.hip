@@ -287,6 +287,7 @@ __device__ __forceinline__ void number_pieces(uint32_t pieces, int T, uint32_t* 
 }
 
 constexpr int SPARSE_WORDS = 2;  // a pass is read out through the summary when its range has this many bitmap words per row, or more
+constexpr int REG_U = 32;  // several passes: pieces per wavefront of a query whose rows stay in registers (at most 32768 rows per query)
 constexpr int SPLIT_BATCH = 3;  // row bounds located per search round of split_spans
 
 // The rows of a span ascend.  For every span t < T and each of the K row bounds bound0 + k * chunk_rows
@@ -480,6 +481,117 @@ __global__ __launch_bounds__(DD_THREADS) void dedup_kernel(DedupArgs a) {
     const uint32_t swap_mask = ew == 8 ? 4u : 0u;
 
     const unsigned long long raw_base = several ? a.raw_offsets[q] : 0ull;
+    if (several && cut) {
+        // A query with few candidates (at most REG_U pieces per wavefront) keeps its rows in registers: one
+        // piece table and one fetch for the whole query, and every pass marks the rows of its range from the
+        // registers and is read out through the summary of non-zero words.  No span is cut at the passes'
+        // row bounds and nothing is fetched twice.
+        number_pieces((static_cast<uint32_t>(sp.y) + 63u) >> 6, T, s_ppref, scratch);
+        if (tid < T) {
+            s_start[tid] = sp.x;
+            s_len[tid] = sp.y;
+        }
+        __syncthreads();
+        const uint32_t whole = s_ppref[T];
+        if (whole <= static_cast<uint32_t>(REG_U * NWAVES)) {
+            if (static_cast<uint32_t>(tid) < whole) {
+                int tl = 0, th = T;  // largest t with s_ppref[t] <= tid; that span owns the piece
+                while (th - tl > 1) {
+                    const int mid = (tl + th) >> 1;
+                    if (s_ppref[mid] <= static_cast<uint32_t>(tid)) tl = mid; else th = mid;
+                }
+                const int first = static_cast<int>(static_cast<uint32_t>(tid) - s_ppref[tl]) * 64;
+                tab[tid] = make_int2(s_start[tl] + first, min(64, s_len[tl] - first));
+            }
+            __syncthreads();
+            int rows[REG_U];
+            {
+#pragma unroll
+                for (int u0 = 0; u0 < REG_U; u0 += 16) {  // table entries of sixteen pieces, then their loads
+                    int2 ent[16];
+#pragma unroll
+                    for (int u = 0; u < 16; ++u)
+                        ent[u] = tab[min(static_cast<uint32_t>(wave + (u0 + u) * NWAVES), max(whole, 1u) - 1u)];
+#pragma unroll
+                    for (int u = 0; u < 16; ++u) {
+                        rows[u0 + u] = -1;
+                        if (static_cast<uint32_t>(wave + (u0 + u) * NWAVES) < whole && lane < ent[u].y)
+                            rows[u0 + u] = a.cand[static_cast<uint32_t>(ent[u].x + lane)];
+                    }
+                }
+            }
+            uint32_t* wbm = bm + wave * wpw;
+            unsigned int ticket_next = 0;
+            for (int chunk = 0; chunk < a.n_chunks; ++chunk) {
+                const uint32_t lo = static_cast<uint32_t>(chunk) * chunk_rows;
+                const bool last = chunk == a.n_chunks - 1;
+                if (last && tid == 0) ticket_next = atomicAdd(a.ticket, 1u);  // arrives while the rows are marked and counted
+#pragma unroll
+                for (int u = 0; u < REG_U; ++u) {
+                    const uint32_t bit = static_cast<uint32_t>(rows[u]) - lo;
+                    if (bit < chunk_rows) {  // also false for -1 (no row)
+                        const uint32_t w = bit >> 5;
+                        atomicOr(&bm[bitmap_slot(w, swap_mask)], 1u << (bit & 31u));
+                        atomicOr(&sm[w >> 5], 1u << (w & 31u));
+                    }
+                }
+                __syncthreads();
+                uint32_t sp_words = 0;
+                if (lane < wpw / 32) sp_words = sm[wave * (wpw / 32) + lane];
+                uint32_t c = 0;
+                for (uint32_t left = sp_words; left; left &= left - 1u)
+                    c += __popc(wbm[bitmap_slot(static_cast<uint32_t>(lane * 32 + __ffs(static_cast<int>(left)) - 1), swap_mask)]);
+                const uint32_t incl = wave_inclusive_sum_dpp(c);
+                if (lane == 63) wtot[wave] = incl;
+                if (last && wave == 0) {
+                    const int qn = min(static_cast<int>(__shfl(ticket_next, 0, 64)), a.n_queries);
+                    if (T <= 64 && qn < a.n_queries && lane < T) sp_next = a.spans[static_cast<size_t>(qn) * T + lane];
+                    if (lane == 0) *sh_q = qn;
+                }
+                __syncthreads();
+                uint32_t wave_base = 0, chunk_total = 0;
+#pragma unroll
+                for (int w = 0; w < NWAVES; ++w) {
+                    const uint32_t v = wtot[w];
+                    wave_base += (w < wave) ? v : 0u;
+                    chunk_total += v;
+                }
+                const uint64_t base = raw_base + running;
+                const bool store = base + chunk_total <= a.capacity;  // cannot fail with capacity = raw candidates
+                if (tid == 0) {
+                    if (!store) atomicOr(a.err, 2u);
+                    if (last) a.counts[q] = running + chunk_total;
+                }
+                if (last) q_next = *sh_q;
+                int32_t* dst = a.out + base + wave_base + (incl - c);
+                const uint32_t row_base = lo + (static_cast<uint32_t>(wave * wpw + lane * 32) << 5);
+                for (uint32_t left = sp_words; left; left &= left - 1u) {
+                    const uint32_t k = static_cast<uint32_t>(__ffs(static_cast<int>(left)) - 1);
+                    uint32_t* word = &wbm[bitmap_slot(static_cast<uint32_t>(lane * 32) + k, swap_mask)];
+                    uint32_t bits = *word;
+                    *word = 0u;
+                    const uint32_t r0 = row_base + (k << 5);
+                    while (bits && store) {
+                        *dst++ = static_cast<int32_t>(r0 + (__ffs(static_cast<int>(bits)) - 1));
+                        bits &= bits - 1u;
+                    }
+                }
+                if (sp_words) sm[wave * (wpw / 32) + lane] = 0u;
+                running += chunk_total;
+                __syncthreads();  // bitmap, summary and wtot are rewritten by the next pass
+            }
+            if (q_next >= a.n_queries) break;
+            q = q_next;
+            if (T <= 64) {
+                sp = sp_next;  // zero outside the first T lanes
+            } else {
+                sp = make_int2(0, 0);
+                if (tid < T) sp = a.spans[static_cast<size_t>(q) * T + tid];
+            }
+            continue;
+        }
+        __syncthreads();  // the general path below rewrites the piece numbering
+    }
     for (int chunk = 0; chunk < a.n_chunks; ++chunk) {
         const uint32_t lo = static_cast<uint32_t>(chunk) * chunk_rows;
         const bool last = MODE == DD_FUSED || chunk == a.n_chunks - 1;  // DD_FUSED is launched for one pass only
