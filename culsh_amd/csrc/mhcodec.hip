@@ -81,7 +81,8 @@ __global__ __launch_bounds__(256) void mh_invert_kernel(const int32_t* __restric
     inv[i] = __builtin_bswap32(sorted_keys[i]);
 }
 
-constexpr int RB = 32;  // rows per workgroup
+constexpr int RB = 32;  // rows per workgroup (RB_SMALL for launches that would otherwise leave compute units idle)
+constexpr int RB_SMALL = 8;
 constexpr int NTHREADS = 256;
 
 // MinHash of CSR rows written as packed rank codes (role of compute_minhash_kernel,
@@ -96,13 +97,13 @@ __global__ __launch_bounds__(NTHREADS) void minhash_rank_kernel(const int32_t* _
                                                                const uint32_t* __restrict__ B,
                                                                const uint32_t* __restrict__ ainv,
                                                                const uint32_t* __restrict__ rank, int n, int T, int H,
-                                                               int d, int bits, int W, int th_chunk,
+                                                               int d, int bits, int W, int th_chunk, int rb,
                                                                uint32_t* __restrict__ out,
                                                                uint32_t* __restrict__ id_beyond_d) {
-    extern __shared__ uint32_t stage[];  // [th_chunk][RB] codes
+    extern __shared__ uint32_t stage[];  // [th_chunk][rb] codes
     const int TH = T * H;
-    const int row0 = blockIdx.x * RB;
-    const int rows = min(RB, n - row0);
+    const int row0 = blockIdx.x * rb;
+    const int rows = min(rb, n - row0);
     if (SMALL && id_beyond_d) {
         // The cheaper hash and the rank codes hold for ids below d only: the workgroup looks once at
         // the ids of its rows (one contiguous stretch; negative ids read as huge) and tells the host.
@@ -148,7 +149,7 @@ __global__ __launch_bounds__(NTHREADS) void minhash_rank_kernel(const int32_t* _
             uint32_t code = static_cast<uint32_t>(d);                      // empty row: sorts last
             if (s < e) code = col < static_cast<uint32_t>(d) ? rank[static_cast<size_t>(c0 + c) * d + col]
                                                               : static_cast<uint32_t>(d) + 1u;  // matches nothing
-            stage[c * RB + r] = code;
+            stage[c * rb + r] = code;
         };
         if ((nc & 63) == 0) {
             // every wavefront works on one row at a time: saying so lets the row's column ids be fetched
@@ -173,7 +174,7 @@ __global__ __launch_bounds__(NTHREADS) void minhash_rank_kernel(const int32_t* _
             unsigned long long acc = 0;
             int nbits = 0, w = 0;
             for (int h = 0; h < H; ++h) {
-                acc = (acc << bits) | stage[(tl * H + h) * RB + r];
+                acc = (acc << bits) | stage[(tl * H + h) * rb + r];
                 nbits += bits;
                 if (nbits >= 32) {
                     k[w++] = static_cast<uint32_t>(acc >> (nbits - 32));
@@ -352,17 +353,19 @@ culsh_status launch_minhash_rank(culsh_ctx* ctx, const int32_t* indices, const i
     CULSH_REQUIRE(indptr && keys && ix->mhc.rank, CULSH_ERR_INVALID, "minhash: null pointer");
     CULSH_REQUIRE(n > 0, CULSH_ERR_INVALID, "minhash: sizes must be positive");
     CULSH_REQUIRE(H <= 384, CULSH_ERR_LIMIT, "minhash: n_hashes > 384 is not supported");
-    int tables_per_chunk = static_cast<int>(std::min<long long>(T, std::max(1, (12288 / RB) / H)));
+    // fewer rows per workgroup when 32 would give the compute units less than four workgroups each
+    const int rb = (n + RB - 1) / RB >= 4 * ctx->n_cus ? RB : RB_SMALL;
+    int tables_per_chunk = static_cast<int>(std::min<long long>(T, std::max(1, (12288 / rb) / H)));
     const int th_chunk = tables_per_chunk * H;
-    const size_t lds = static_cast<size_t>(th_chunk) * RB * sizeof(uint32_t);
+    const size_t lds = static_cast<size_t>(th_chunk) * rb * sizeof(uint32_t);
+    const dim3 grid((n + rb - 1) / rb);
     if (fit_flag && ix->mhc.d <= (1 << 25))
-        CULSH_LAUNCH(ctx, minhash_rank_kernel<true>, dim3((n + RB - 1) / RB), dim3(NTHREADS), lds, ctx->stream, indices,
-                     indptr, ix->A, ix->B, ix->mhc.ainv, ix->mhc.rank, n, T, H, ix->mhc.d, ix->mhc.bits, ix->key_w, th_chunk,
-                     keys, fit_flag);
+        CULSH_LAUNCH(ctx, minhash_rank_kernel<true>, grid, dim3(NTHREADS), lds, ctx->stream, indices, indptr, ix->A, ix->B,
+                     ix->mhc.ainv, ix->mhc.rank, n, T, H, ix->mhc.d, ix->mhc.bits, ix->key_w, th_chunk, rb, keys, fit_flag);
     else
-        CULSH_LAUNCH(ctx, minhash_rank_kernel<false>, dim3((n + RB - 1) / RB), dim3(NTHREADS), lds, ctx->stream, indices,
-                     indptr, ix->A, ix->B, ix->mhc.ainv, ix->mhc.rank, n, T, H, ix->mhc.d, ix->mhc.bits, ix->key_w, th_chunk,
-                     keys, static_cast<uint32_t*>(nullptr));
+        CULSH_LAUNCH(ctx, minhash_rank_kernel<false>, grid, dim3(NTHREADS), lds, ctx->stream, indices, indptr, ix->A, ix->B,
+                     ix->mhc.ainv, ix->mhc.rank, n, T, H, ix->mhc.d, ix->mhc.bits, ix->key_w, th_chunk, rb, keys,
+                     static_cast<uint32_t*>(nullptr));
     CULSH_LAUNCH_CHECK();
     return CULSH_OK;
 }
