@@ -1026,6 +1026,81 @@ def test_config4_full_size(ctx, c_oracle):
     ctx.free_index(ih)
 
 
+def test_item_count_just_below_2_31(ctx):
+    """n_samples * n_hash_tables = 2,097,152,000 items, the most the 32-bit offsets of the index hold
+    (limit 2^31): 2M rows x 8 features into 1000 tables x 4 hashes.  Everything is checked on the device
+    (torch as plumbing): a permutation of the rows in the first, a middle and the last table, rows
+    ascending inside buckets, offsets that end at the item count, and four queries against a brute-force
+    union over all 1000 tables computed from the stage-level signatures."""
+    import ctypes as C
+
+    import torch
+
+    from culsh_amd import _lib as L
+    from culsh_amd.abi import dev, hp, ptr
+
+    _announce("items_just_below_2_31")
+    n, d, T, H, nq = 1 << 21, 8, 1000, 4, 4
+    rng = np.random.default_rng(2031)
+    X = rng.standard_normal((n, d)).astype(np.float32)
+    P = rng.standard_normal((T * H, d)).astype(np.float32)
+    qrows = np.array([0, 123_457, n // 2 + 1, n - 1])
+    dX, dP = dev(X), dev(P)
+    dQ = dev(np.ascontiguousarray(X[qrows]))
+    lib = ctx.lib
+    ih = C.c_void_p()
+    L.check(lib.culsh_rplsh_fit_f32(ctx.h, ptr(dX), n, d, T, H, 1, hp(P), C.byref(ih)))
+    try:
+        m = L.IndexMeta()
+        L.check(lib.culsh_index_get_meta(ih, C.byref(m)))
+        N = n * T
+        assert m.n_total_candidates == N and N < 2 ** 31 and 0 < m.n_total_buckets <= T * (1 << H)
+        B = int(m.n_total_buckets)
+
+        def on_device(which, count, dtype):
+            out = torch.empty(count, dtype=dtype, device="cuda")
+            L.check(lib.culsh_index_copy_array(ctx.h, ih, which, ptr(out), out.numel() * out.element_size(), 1))
+            return out
+
+        tbo = on_device(L.ARR_TABLE_BUCKET_OFFSETS, T + 1, torch.int32).cpu().numpy().astype(np.int64)
+        assert tbo[0] == 0 and tbo[-1] == B and (np.diff(tbo) > 0).all()
+        bco = on_device(L.ARR_BUCKET_CANDIDATE_OFFSETS, B + 1, torch.int32).to(torch.int64)
+        assert int(bco[0]) == 0 and int(bco[-1]) == N and bool((bco[1:] > bco[:-1]).all())
+        # every table's buckets cover exactly its n items
+        ends = bco[torch.from_numpy(tbo).cuda()]
+        assert bool((ends == torch.arange(T + 1, device="cuda", dtype=torch.int64) * n).all())
+        cand = on_device(L.ARR_CANDIDATE_INDICES, N, torch.int32)
+        for t in (0, T // 2, T - 1):
+            rows = cand[t * n:(t + 1) * n].to(torch.int64)
+            assert int(rows.min()) == 0 and int(rows.max()) == n - 1
+            assert bool((torch.bincount(rows, minlength=n) == 1).all())              # a permutation of the rows
+            starts = torch.zeros(n, dtype=torch.bool, device="cuda")
+            b0, b1 = int(tbo[t]), int(tbo[t + 1])
+            starts[(bco[b0:b1] - t * n)] = True
+            assert bool(((rows[1:] > rows[:-1]) | starts[1:]).all())                 # ascending inside every bucket
+            del rows, starts
+        del cand
+        # four queries (rows of X) against brute force over all tables
+        sig = torch.empty(T * n * H, dtype=torch.uint8, device="cuda")
+        L.check(lib.culsh_rplsh_hash_f32(ctx.h, ptr(dX), ptr(dP), n, d, T, H, ptr(sig)))
+        sig = sig.view(T, n, H)
+        ch = C.c_void_p()
+        L.check(lib.culsh_rplsh_query_f32(ctx.h, ptr(dQ), nq, ih, -1, C.byref(ch)))
+        got = ctx.candidates_arrays(ch)
+        assert got["offsets"][0] == 0 and got["offsets"][-1] == got["n_total_candidates"]
+        for i, r in enumerate(qrows):
+            same = torch.zeros(n, dtype=torch.bool, device="cuda")
+            for t0 in range(0, T, 100):
+                part = sig[t0:t0 + 100]
+                same |= (part == part[:, r:r + 1, :]).all(dim=2).any(dim=0)
+            exp = torch.nonzero(same).flatten().cpu().numpy().astype(np.int32)
+            lo, hi = int(got["offsets"][i]), int(got["offsets"][i + 1])
+            assert got["counts"][i] == hi - lo == exp.size and r in exp
+            np.testing.assert_array_equal(got["indices"][lo:hi], exp)
+    finally:
+        lib.culsh_index_free(ih)
+
+
 def test_config5_full_size_invariants(ctx):
     """Benchmark configuration 5 of the reference at its real shape (4M x 768 rows of a 1000-component Gaussian mixture on the
     unit sphere, 64 tables x 16 hashes), 20k queries in batches of 10k: the index takes 2^28 items, a
