@@ -1101,6 +1101,24 @@ def test_item_count_just_below_2_31(ctx):
         lib.culsh_index_free(ih)
 
 
+def test_item_count_of_2_31_is_refused(ctx):
+    """One row more than the limit: refused before any device work (the rows are never read)."""
+    import ctypes as C
+
+    from culsh_amd import _lib as L
+    from culsh_amd.abi import dev, hp, ptr
+
+    _announce("items_2_31_refused")
+    T, H, d = 1024, 4, 8
+    n = (1 << 31) // T                                       # n * T = 2^31 exactly
+    tiny = dev(np.zeros((4, d), dtype=np.float32))           # stands for X: the call must not touch it
+    P = np.zeros((T * H, d), dtype=np.float32)
+    ih = C.c_void_p()
+    status = ctx.lib.culsh_rplsh_fit_f32(ctx.h, ptr(tiny), n, d, T, H, 1, hp(P), C.byref(ih))
+    assert status == L.ERR_LIMIT and not ih.value
+    assert b"2^31" in ctx.lib.culsh_last_error()
+
+
 def test_config5_full_size_invariants(ctx):
     """Benchmark configuration 5 of the reference at its real shape (4M x 768 rows of a 1000-component Gaussian mixture on the
     unit sphere, 64 tables x 16 hashes), 20k queries in batches of 10k: the index takes 2^28 items, a
