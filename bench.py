@@ -271,6 +271,21 @@ def main() -> int:
         cand = ctx.candidates_arrays(ch)
         lib.culsh_index_free(ih)
         mism = float(np.mean(cpu_sig != sig))
+        # candidate sets of the CPU's own pipeline (its float hash bits, which may differ from the GPU's
+        # inside the tolerance band) against the GPU's lists: per-query Jaccard, every query
+        if mism == 0.0 and np.array_equal(cpu_qsig, qsig):
+            jac_min = jac_mean = 1.0                      # identical signatures: the lists above are the comparison
+        else:
+            own = co.query_index_c(cpu_qsig, co.fit_index_c(cpu_sig, H), keep=True)
+            jac = np.ones(nq)
+            go, eo = cand["offsets"].astype(np.int64), own.query_candidate_offsets.astype(np.int64)
+            for i in range(nq):
+                g, e = cand["indices"][go[i]:go[i + 1]], own.query_candidate_indices[eo[i]:eo[i + 1]]
+                if g.size != e.size or not np.array_equal(g, e):
+                    inter = np.intersect1d(g, e, assume_unique=True).size
+                    union = g.size + e.size - inter
+                    jac[i] = inter / union if union else 1.0
+            jac_min, jac_mean = float(jac.min()), float(jac.mean())
         counts_ok = bool(np.array_equal(cand["counts"], cpu_c.query_candidate_counts) and
                          np.array_equal(cand["offsets"], cpu_c.query_candidate_offsets))
         lists_ok = bool(counts_ok and np.array_equal(cand["indices"], cpu_c.query_candidate_indices))
@@ -280,6 +295,8 @@ def main() -> int:
                   "candidate_lists_bit_exact": lists_ok,
                   "candidate_lists_compared": int(nq),
                   "hash_bit_mismatch_vs_cpu_float": mism,
+                  "candidate_jaccard_vs_cpu_hashed_pipeline": {"min": round(jac_min, 6), "mean": round(jac_mean, 8),
+                                                               "queries": int(nq), "required": 0.999},
                   "raw_candidates": cpu_R, "unique_candidates": cpu_U,
                   "n_buckets": int(exp.n_total_buckets)}
         cpu = {"value": round(n / cpu_fit_s / 1e6, 4), "unit": "Mvec/s", "cores": co.num_threads(),
@@ -287,7 +304,7 @@ def main() -> int:
                "sample": f"full workload once: fit of {n}x{d} ({cpu_fit_s:.2f} s), "
                          f"query of {nq} ({cpu_query_s:.2f} s)",
                "query_qps": round(nq / cpu_query_s, 1)}
-        if not (table_ok and parity["unique_candidates_equal"] and counts_ok and lists_ok):
+        if not (table_ok and parity["unique_candidates_equal"] and counts_ok and lists_ok and jac_min >= 0.999):
             print("bench.py: PARITY FAILURE " + json.dumps(parity), file=sys.stderr)
             return 1
 
