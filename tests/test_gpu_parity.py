@@ -1101,6 +1101,92 @@ def test_item_count_just_below_2_31(ctx):
         lib.culsh_index_free(ih)
 
 
+@pytest.mark.parametrize("family", ["pslsh", "minhash"])
+def test_item_count_just_below_2_31_wide_key_families(ctx, family):
+    """The same size (2^21 rows x 1000 tables) for the families with rank-compressed keys, two hashes per
+    table: index invariants on the device, and four queries against a brute-force union over all tables
+    computed from the stage-level hashes."""
+    import ctypes as C
+
+    import torch
+
+    from culsh_amd import _lib as L
+    from culsh_amd.abi import dev, hp, ptr
+
+    _announce("items_just_below_2_31", family)
+    n, T, H, nq = 1 << 21, 1000, 2, 4
+    rng = np.random.default_rng(2032)
+    qrows = np.array([1, 654_321, n // 2, n - 1])
+    lib = ctx.lib
+    ih, ch = C.c_void_p(), C.c_void_p()
+    if family == "pslsh":
+        d, w = 8, 4
+        X = rng.standard_normal((n, d)).astype(np.float32)
+        P, b = o.generate_random_projections_biases(11, T * H, d, w, np.float32)
+        dX, dP, db = dev(X), dev(P), dev(b)
+        dQ = dev(np.ascontiguousarray(X[qrows]))
+        sig = torch.empty(T * n * H, dtype=torch.int32, device="cuda")
+        L.check(lib.culsh_pslsh_hash_f32(ctx.h, ptr(dX), ptr(dP), ptr(db), n, d, T, H, ptr(sig)))
+        L.check(lib.culsh_pslsh_fit_f32(ctx.h, ptr(dX), n, d, T, H, w, 11, hp(P), hp(b), C.byref(ih)))
+        L.check(lib.culsh_pslsh_query_f32(ctx.h, ptr(dQ), nq, ih, -1, C.byref(ch)))
+    else:
+        d = 1000
+        # six distinct columns per row: base + k * stride (mod d) with 5 * stride < d, sorted per row
+        base, stride = rng.integers(0, d, size=(n, 1)), rng.integers(1, d // 6, size=(n, 1))
+        indices = np.sort((base + np.arange(6) * stride) % d, axis=1).astype(np.int32).reshape(-1)
+        indptr = (np.arange(n + 1, dtype=np.int64) * 6).astype(np.int32)
+        A, B = o.generate_hash_integers(12, T * H)
+        dI, dPtr, dA, dB = dev(indices), dev(indptr), dev(A), dev(B)
+        qi = np.concatenate([indices[indptr[r]:indptr[r + 1]] for r in qrows]).astype(np.int32)
+        qp = np.concatenate([[0], np.cumsum([indptr[r + 1] - indptr[r] for r in qrows])]).astype(np.int32)
+        dqi, dqp = dev(qi), dev(qp)
+        sig = torch.empty(T * n * H, dtype=torch.int32, device="cuda")   # uint32 values, compared for equality only
+        L.check(lib.culsh_minhash_compute(ctx.h, ptr(dI), ptr(dPtr), ptr(dA), ptr(dB), n, T, H, ptr(sig)))
+        L.check(lib.culsh_minhash_fit(ctx.h, ptr(dI), ptr(dPtr), n, d, T, H, 12, hp(A), hp(B), C.byref(ih)))
+        L.check(lib.culsh_minhash_query(ctx.h, ptr(dqi), ptr(dqp), nq, ih, C.byref(ch)))
+    try:
+        m = L.IndexMeta()
+        L.check(lib.culsh_index_get_meta(ih, C.byref(m)))
+        N, Bk = n * T, int(m.n_total_buckets)
+        assert m.n_total_candidates == N and m.sig_nbytes == 4 * H
+
+        def on_device(which, count, dtype):
+            out = torch.empty(count, dtype=dtype, device="cuda")
+            L.check(lib.culsh_index_copy_array(ctx.h, ih, which, ptr(out), out.numel() * out.element_size(), 1))
+            return out
+
+        tbo = on_device(L.ARR_TABLE_BUCKET_OFFSETS, T + 1, torch.int32).cpu().numpy().astype(np.int64)
+        bco = on_device(L.ARR_BUCKET_CANDIDATE_OFFSETS, Bk + 1, torch.int32).to(torch.int64)
+        assert tbo[0] == 0 and tbo[-1] == Bk and int(bco[0]) == 0 and int(bco[-1]) == N
+        assert bool((bco[1:] > bco[:-1]).all())
+        assert bool((bco[torch.from_numpy(tbo).cuda()] == torch.arange(T + 1, device="cuda", dtype=torch.int64) * n).all())
+        cand = on_device(L.ARR_CANDIDATE_INDICES, N, torch.int32)
+        for t in (0, T - 1):
+            rows = cand[t * n:(t + 1) * n].to(torch.int64)
+            assert bool((torch.bincount(rows, minlength=n) == 1).all())
+            starts = torch.zeros(n, dtype=torch.bool, device="cuda")
+            starts[(bco[int(tbo[t]):int(tbo[t + 1])] - t * n)] = True
+            assert bool(((rows[1:] > rows[:-1]) | starts[1:]).all())
+            del rows, starts
+        del cand
+        sig = sig.view(T, n, H)
+        got = ctx.candidates_arrays(ch)
+        ch = None
+        for i, r in enumerate(qrows):
+            same = torch.zeros(n, dtype=torch.bool, device="cuda")
+            for t0 in range(0, T, 100):
+                part = sig[t0:t0 + 100]
+                same |= (part == part[:, r:r + 1, :]).all(dim=2).any(dim=0)
+            exp = torch.nonzero(same).flatten().cpu().numpy().astype(np.int32)
+            lo, hi = int(got["offsets"][i]), int(got["offsets"][i + 1])
+            assert hi - lo == exp.size and r in exp
+            np.testing.assert_array_equal(got["indices"][lo:hi], exp)
+    finally:
+        if ch:
+            lib.culsh_candidates_free(ch)
+        lib.culsh_index_free(ih)
+
+
 def test_item_count_of_2_31_is_refused(ctx):
     """One row more than the limit: refused before any device work (the rows are never read)."""
     import ctypes as C
