@@ -3,6 +3,7 @@
 
 #include <hip/hip_runtime.h>
 
+#include <atomic>
 #include <cstdarg>
 #include <cstdint>
 #include <cstdio>
@@ -30,6 +31,14 @@ struct Status {
             return (e_ == hipErrorOutOfMemory) ? CULSH_ERR_NOMEM : CULSH_ERR_HIP;         \
         }                                                                                 \
     } while (0)
+
+// "Done once per device" flags.  Contexts are used by one host thread each, but two threads with a
+// context each may reach the same flag together: doing the step twice is harmless, a torn flag is not.
+struct PerDeviceOnce {
+    std::atomic<bool> done[64] = {};
+    bool is_set(int device) const { return done[device & 63].load(std::memory_order_acquire); }
+    void set(int device) { done[device & 63].store(true, std::memory_order_release); }
+};
 
 #define CULSH_TRY(expr)                    \
     do {                                   \

@@ -1058,13 +1058,13 @@ culsh_status query_from_spans(culsh_ctx* ctx, const int2* spans, const unsigned 
         a.err = err;
         a.capacity = cap;
         {   // more LDS than a launch may ask for by default: allowed once per kernel and device, not per call
-            static bool allowed[2][64] = {};
-            bool& done = allowed[several ? 1 : 0][ctx->device & 63];
-            if (!done) {
+            static PerDeviceOnce allowed[2];
+            PerDeviceOnce& done = allowed[several ? 1 : 0];
+            if (!done.is_set(ctx->device)) {
                 const void* kernel = several ? reinterpret_cast<const void*>(dedup_kernel<DD_FUSED_PASSES>)
                                              : reinterpret_cast<const void*>(dedup_kernel<DD_FUSED>);
                 CULSH_HIP(hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, ctx->lds_max));
-                done = true;
+                done.set(ctx->device);
             }
         }
         // as many workgroups as fit on the device at once (LDS and 2048 threads per CU bound it)
@@ -1130,13 +1130,13 @@ culsh_status query_from_spans(culsh_ctx* ctx, const int2* spans, const unsigned 
         break;
     }
     if (!fused) {
-        static bool allowed_two_launch[64] = {};
-        if (!allowed_two_launch[ctx->device & 63]) {
+        static PerDeviceOnce allowed_two_launch;
+        if (!allowed_two_launch.is_set(ctx->device)) {
             CULSH_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(dedup_kernel<DD_COUNT>),
                                           hipFuncAttributeMaxDynamicSharedMemorySize, ctx->lds_max));
             CULSH_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(dedup_kernel<DD_EMIT>),
                                           hipFuncAttributeMaxDynamicSharedMemorySize, ctx->lds_max));
-            allowed_two_launch[ctx->device & 63] = true;
+            allowed_two_launch.set(ctx->device);
         }
         CULSH_LAUNCH(ctx, dedup_kernel<DD_COUNT>, dim3(n_queries), dim3(DD_THREADS), lds_bytes, ctx->stream, a);
         CULSH_LAUNCH_CHECK();

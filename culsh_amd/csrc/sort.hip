@@ -438,11 +438,11 @@ namespace {
 template <int KW, bool CHAINED, int THREADS, int ITEMS, typename... Args>
 culsh_status launch_scatter(culsh_ctx* ctx, dim3 grid, Args... args) {
     constexpr size_t lds = scatter_lds_bytes(KW, TileShape{THREADS, ITEMS});
-    static bool configured[64] = {};  // per device: more LDS than a launch may ask for by default
-    if (lds > 48 * 1024 && !configured[ctx->device & 63]) {
+    static PerDeviceOnce configured;  // more LDS than a launch may ask for by default
+    if (lds > 48 * 1024 && !configured.is_set(ctx->device)) {
         CULSH_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(radix_scatter_kernel<KW, CHAINED, THREADS, ITEMS>),
                                       hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)));
-        configured[ctx->device & 63] = true;
+        configured.set(ctx->device);
     }
     {
         static const char* const names[2][5] = {
@@ -555,11 +555,11 @@ culsh_status sort_tables(culsh_ctx* ctx, uint32_t* keys_in, uint32_t* keys_tmp, 
             // as many histogram copies as 60 KiB hold, eight at most
             const int copies = std::max(1, std::min(8, (60 * 1024) / (pl.count * TOT_ROW * 4)));
             const size_t lds = static_cast<size_t>(copies) * pl.count * TOT_ROW * sizeof(uint32_t);
-            static bool configured[64] = {};  // per device: more LDS than a launch may ask for by default
-            if (lds > 48 * 1024 && !configured[ctx->device & 63]) {
+            static PerDeviceOnce configured;  // more LDS than a launch may ask for by default
+            if (lds > 48 * 1024 && !configured.is_set(ctx->device)) {
                 CULSH_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(radix_totals_kernel),
                                               hipFuncAttributeMaxDynamicSharedMemorySize, 60 * 1024));
-                configured[ctx->device & 63] = true;
+                configured.set(ctx->device);
             }
             CULSH_LAUNCH(ctx, radix_totals_kernel, dim3(per_table, T), dim3(SORT_THREADS), lds, ctx->stream, keys_in, n, W, pl,
                          T, copies, dtot + static_cast<size_t>(p0) * T * 256);

@@ -1372,6 +1372,49 @@ def test_objects_cross_contexts(ctx):
     ctx.free_index(ih2)
 
 
+def test_contexts_on_host_threads(c_oracle):
+    """One context per host thread: four threads fit and query at the same time (ctypes releases the
+    interpreter lock during a call, so the library's calls, the block cache and the kernels with
+    their waits between workgroups really overlap), each on its own data and several times over, and
+    every result is the oracle's."""
+    _announce("contexts_on_host_threads")
+    import threading
+    from abi import Ctx, assert_candidates_match, assert_index_matches
+
+    shapes = [(4, 70000, 300, 2), (6, 9000, 200, 3), (2, 150000, 64, 2), (33, 3000, 100, 4)]  # T, n, nq, H
+    cases = []
+    for i, (T, n, nq, H) in enumerate(shapes):
+        rng = np.random.default_rng(500 + i)
+        sig = random_sigs(rng, T, n, H, "rplsh")
+        qsig = random_sigs(rng, T, nq, H, "rplsh")
+        cix = c_oracle.fit_index_c(sig, H)
+        cases.append((sig, qsig, H, n, cix.to_numpy(n), c_oracle.query_index_c(qsig, cix)))
+    failures = []
+    start = threading.Barrier(len(cases))
+
+    def work(case):
+        sig, qsig, H, n, exp_ix, exp_cand = case
+        try:
+            c = Ctx(0)
+            start.wait(timeout=60)
+            for _ in range(6):
+                ih, _ = c.core_fit_index(sig, H)
+                assert_index_matches(c.index_arrays(ih), exp_ix)
+                assert_candidates_match(c.core_query_index(qsig, ih), exp_cand)
+                c.free_index(ih)
+            c.close()
+        except BaseException as e:  # reported by the main thread
+            failures.append(repr(e))
+
+    threads = [threading.Thread(target=work, args=(case,)) for case in cases]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join(timeout=100)
+    assert not any(t.is_alive() for t in threads), "a thread did not finish"
+    assert not failures, failures
+
+
 def test_minhash_rank_keys_edge_cases(ctx):
     """MinHash keys are stored as column ranks when every fitted column id is below n_features.
     Checked against the oracle: query rows whose minimum comes from a column >= n_features (they
