@@ -1273,7 +1273,13 @@ culsh_status culsh_index_load(culsh_ctx* ctx, culsh_kind kind, int is_double, co
     ix->seed = seed;
     ix->enc = enc;
     ix->key_w = key_words(enc, S);
-    CULSH_TRY(upload(cand, static_cast<size_t>(n_total_candidates), &ix->all_candidate_indices));
+    {   // readable behind its end, see CAND_PAD
+        const size_t count = static_cast<size_t>(n_total_candidates);
+        if (count) {  // empty array -> nullptr (array_utils.cuh:34-36)
+            CULSH_HIP(dev_malloc(&ix->all_candidate_indices, (count + CAND_PAD) * sizeof(int32_t)));
+            CULSH_HIP(hipMemcpy(ix->all_candidate_indices, cand, count * sizeof(int32_t), hipMemcpyHostToDevice));
+        }
+    }
     CULSH_TRY(upload(bsig, static_cast<size_t>(n_total_buckets) * S, &ix->all_bucket_signatures));
     CULSH_TRY(upload(bco, static_cast<size_t>(n_total_buckets) + 1, &ix->bucket_candidate_offsets));
     CULSH_TRY(upload(tbo, static_cast<size_t>(T) + 1, &ix->table_bucket_offsets));

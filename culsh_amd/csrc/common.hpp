@@ -124,10 +124,13 @@ struct culsh_ctx {
     uint32_t* aux_flag_dev = nullptr;  // a family's own flag that travels with the end-of-build read-back, or null
     uint32_t aux_flag_host = 0;        // its value after that read-back
     bool sort_unchained = false;
-    // raw candidates per query of the last query call and the shape of the index it went to (rows,
-    // buckets, tables, hashes): sizes the next call's output without a host round trip (query.hip)
-    uint64_t raw_guess_key = 0;
-    double raw_guess_per_query = 0.0;
+    // raw and distinct candidates per query of the last query calls, by the shape of the index they
+    // went to (rows, buckets, tables, hashes): sizes the next call's output on an index of that shape
+    // without a host round trip (query.hip).  A few shapes are kept, so that a caller who alternates
+    // between indices keeps the short path on each.
+    struct QueryGuess { uint64_t key = 0; double raw_per_query = 0.0, uniq_per_query = 0.0; };
+    QueryGuess query_guess[8];
+    int query_guess_next = 0;  // slot the next unknown shape replaces
     int lds_max = 0;                     // max LDS bytes per workgroup
     int n_cus = 0;
     // per-kernel timing with HIP events on `stream` (off unless enabled)
@@ -357,6 +360,37 @@ culsh_status query_from_matched(culsh_ctx* ctx, const int32_t* matched, int n_qu
 // lookup + candidate retrieval from key words [T][n_queries][key_w]
 culsh_status query_from_keys(culsh_ctx* ctx, const uint32_t* q_keys, int n_queries, const culsh_index* index,
                              culsh_candidates* out);
+
+// Elements that can be read (not used) behind the last one of an index's all_candidate_indices: the
+// query kernels fetch whole 64-row pieces.
+constexpr size_t CAND_PAD = 64;
+
+// ---------------------------------------------------------------- sparse de-duplication (dedup_sparse.hip)
+// One launch that turns the queries' bucket spans into packed ascending duplicate-free lists through a
+// two-level bitmap whose cost follows the candidates, not the row range.
+struct SparseDedupArgs {
+    const void* spans;            // int2 [n_queries][T] (start, length) in `cand`
+    const int32_t* cand;          // all_candidate_indices
+    int32_t* out;                 // candidate indices, `capacity` elements
+    uint64_t* counts;             // [n_queries] (written)
+    uint64_t* offsets;            // [n_queries + 1] (written)
+    unsigned long long* state;    // [n_queries] words of the chained scan, zero before the launch
+    unsigned int* err;            // bit 0: the chained scan gave up, bit 1: `out` too small
+    unsigned int* ticket;         // next query to hand out, zero before the launch
+    unsigned long long capacity;
+    int T, n_queries;
+    int l1_per_thread;            // level-1 words per thread (SparseDedupGeometry)
+    int cap;                      // level-2 entries (SparseDedupGeometry)
+    int spin_limit;               // polls of an unpublished predecessor before giving up
+    unsigned long long* ticks;    // optional [workgroups][8] phase timers (wall clock ticks of thread 0), or null
+};
+struct SparseDedupGeometry {
+    int l1_per_thread = 0, cap = 0;
+    size_t lds_bytes = 0;
+};
+// false when level 1 of `n_rows` rows leaves no room for level 2 in LDS; cap_limit > 0 lowers `cap` (tests)
+bool sparse_dedup_geometry(const culsh_ctx* ctx, int n_rows, int T, int cap_limit, SparseDedupGeometry* g);
+culsh_status launch_dedup_sparse(culsh_ctx* ctx, const SparseDedupArgs& a, const SparseDedupGeometry& g);
 
 // ---------------------------------------------------------------- scans (scan.hip)
 // Exclusive prefix sum of `n` u64 values; out[n] receives the total (out has n+1 slots).

@@ -331,7 +331,7 @@ culsh_status fit_index_from_keys(culsh_ctx* ctx, uint32_t* keys, int n, int T, i
     int32_t* rows_out = nullptr;
     CULSH_TRY(arena_alloc_t(ctx, N * W, &keys_tmp));
     CULSH_TRY(arena_alloc_t(ctx, N, &rows_tmp));
-    CULSH_HIP(dev_malloc(&rows_out, N * sizeof(int32_t)));
+    CULSH_HIP(dev_malloc(&rows_out, (N + CAND_PAD) * sizeof(int32_t)));  // readable behind its end, see CAND_PAD
     index->all_candidate_indices = rows_out;  // owned by the index from here on (freed with it)
     uint32_t* sorted = nullptr;
     uint32_t bits_vary[64];

@@ -25,11 +25,10 @@
 
 #include "block_utils.hpp"
 #include "common.hpp"
+#include "dedup_common.hpp"
 
 namespace culsh_amd {
 namespace {
-
-constexpr int DD_THREADS = 1024;
 
 // Bits to drop from a key's first word to get its directory entry: the entry is made of the
 // KEY_DIR_BITS bits from the highest bit that the largest first word has set.
@@ -219,72 +218,6 @@ __global__ __launch_bounds__(256) void close_gaps_kernel(const int32_t* __restri
     for (uint64_t i = threadIdx.x; i < count; i += 256) to[i] = from[i];
 }
 
-constexpr int NWAVES = DD_THREADS / 64;
-constexpr int WALK_U = 16;  // pieces in flight per wavefront
-
-// Visits every row id of the query's spans.  The spans are cut into pieces of up to 64
-// consecutive ids (a piece never crosses a span boundary), pieces are dealt round-robin to
-// the wavefronts, and a wavefront reads a piece with one load per lane.  Where piece p
-// starts is looked up once per piece (one binary search per thread over the spans'
-// piece counts, all pieces of a round in parallel) and kept in `tab`, so the per-lane
-// work is an add, a compare and the load.  `f` is also called with -1, for the lanes beyond a
-// piece's end, and must ignore it.  Contains barriers: all threads must call it.
-template <typename F>
-__device__ __forceinline__ void walk_candidates(const int32_t* __restrict__ cand, const int* s_start,
-                                                const int* s_len, const uint32_t* s_ppref, int T,
-                                                uint32_t n_pieces, int2* tab, F&& f) {
-    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // the same in every lane: kept in a scalar register
-    for (uint32_t r0 = 0; r0 < n_pieces; r0 += DD_THREADS) {
-        const uint32_t pc = r0 + static_cast<uint32_t>(tid);
-        if (pc < n_pieces) {
-            int tl = 0, th = T;  // largest t with s_ppref[t] <= pc; that span owns the piece
-            while (th - tl > 1) {
-                const int mid = (tl + th) >> 1;
-                if (s_ppref[mid] <= pc) tl = mid; else th = mid;
-            }
-            const int first = static_cast<int>(pc - s_ppref[tl]) * 64;
-            tab[tid] = make_int2(s_start[tl] + first, min(64, s_len[tl] - first));
-        }
-        __syncthreads();
-        const uint32_t here = min(static_cast<uint32_t>(DD_THREADS), n_pieces - r0);
-        for (uint32_t p0 = wave; p0 < here; p0 += NWAVES * WALK_U) {
-            // table entries of all pieces first (one LDS round trip instead of one per piece), then the loads
-            int rows[WALK_U];
-            int2 ent[WALK_U];
-#pragma unroll
-            for (int u = 0; u < WALK_U; ++u) ent[u] = tab[min(p0 + u * NWAVES, here - 1u)];
-#pragma unroll
-            for (int u = 0; u < WALK_U; ++u) {
-                const uint32_t pi = p0 + u * NWAVES;
-                rows[u] = -1;
-                if (pi < here && lane < ent[u].y) rows[u] = cand[static_cast<uint32_t>(ent[u].x + lane)];  // unsigned: no sign extension per load
-            }
-#pragma unroll
-            for (int u = 0; u < WALK_U; ++u) f(rows[u]);  // -1 where the lane has no row: f tells by its range check
-        }
-        __syncthreads();  // tab is rewritten by the next round
-    }
-}
-
-// Piece numbering of the spans handed to walk_candidates: s_ppref[t] = pieces of the spans before t,
-// s_ppref[T] = all pieces.  `pieces` is the piece count of span threadIdx.x (0 beyond the T-th thread).
-// Up to 64 spans sit in the first wavefront, which then does it alone, without a barrier; all threads
-// must call it, and a barrier has to follow before s_ppref is read.
-__device__ __forceinline__ void number_pieces(uint32_t pieces, int T, uint32_t* s_ppref, uint32_t* scratch) {
-    const int tid = threadIdx.x;
-    if (T <= 64) {
-        if (tid < 64) {
-            const uint32_t incl = wave_inclusive_sum_dpp(pieces);
-            if (tid < T) s_ppref[tid] = incl - pieces;
-            if (tid == 63) s_ppref[T] = incl;
-        }
-    } else {
-        uint32_t total;
-        const uint32_t ex = block_exclusive_sum(pieces, scratch, &total);
-        if (tid < T) s_ppref[tid] = ex;
-        if (tid == 0) s_ppref[T] = total;
-    }
-}
 
 constexpr int SPARSE_WORDS = 2;  // a pass is read out through the summary when its range has this many bitmap words per row, or more
 constexpr int REG_U = 32;  // several passes: pieces per wavefront of a query whose rows stay in registers (at most 32768 rows per query)
@@ -335,45 +268,6 @@ struct DedupArgs {
     unsigned long long* ticks;  // optional [n_queries][8] phase timers (wall clock ticks of thread 0), or null
 };
 
-// Chained scan over the queries' counts.  A published word holds a 2-bit tag and a value:
-// tag 1 = this query's count, tag 2 = sum of the counts of queries 0..q.  The caller (one
-// full wavefront) has published its count; here it sums its predecessors' counts back to
-// the nearest running sum, then publishes its own running sum.  Workgroups start in index order, so the
-// lowest unfinished query never waits on one that has not started; the poll count is
-// bounded all the same and a give-up is reported through `err`.
-constexpr unsigned long long TAG_COUNT = 1ull << 62, TAG_SUM = 2ull << 62, TAG_VALUE = TAG_COUNT - 1ull;
-
-__device__ __forceinline__ unsigned long long look_back(unsigned long long* state, int q, unsigned long long total,
-                                                        int spin_limit, unsigned int* err) {
-    const int lane = threadIdx.x & 63;
-    unsigned long long excl = 0;
-    int hi = q;  // queries [0, hi) are not accounted for yet
-    int polls = 0;
-    bool gave_up = false;
-    while (hi > 0) {
-        const int idx = hi - 1 - lane;  // lane 0 looks at the nearest predecessor
-        const unsigned long long v =
-            idx >= 0 ? __hip_atomic_load(&state[idx], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : TAG_SUM;
-        const unsigned tag = static_cast<unsigned>(v >> 62);
-        const unsigned long long has_sum = __ballot(tag == 2u), unpublished = __ballot(tag == 0u);
-        const int f = has_sum ? __ffsll(static_cast<long long>(has_sum)) - 1 : 64;  // nearest running sum
-        const unsigned long long needed = f >= 63 ? ~0ull : ((2ull << f) - 1ull);  // lanes 0..f
-        if (unpublished & needed) {
-            if (++polls > spin_limit) { gave_up = true; break; }
-            __builtin_amdgcn_s_sleep(2);
-            continue;
-        }
-        excl += wave_sum((lane <= f) ? (v & TAG_VALUE) : 0ull);
-        if (f < 64) break;
-        hi -= 64;
-    }
-    if (gave_up) {
-        if (lane == 0) atomicOr(err, 1u);
-        excl = 0;
-    }
-    if (lane == 0) __hip_atomic_store(&state[q], TAG_SUM | (excl + total), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    return excl;
-}
 
 // Where bitmap word `w` sits in LDS.  With eight words per lane and step a lane reads two 16-byte
 // halves at a lane stride of 32 bytes, and sixteen neighbouring lanes would hit every bank twice per
@@ -948,9 +842,10 @@ culsh_status dedup_geometry(const culsh_ctx* ctx, const culsh_index* index, Dedu
 
 // The zero-initialised words a query needs, in one block cleared by one memset:
 // [0] raw candidate total, [1] error flags (low half) and ticket counter (high half),
-// [2 .. 2 + n_queries) the published words of the chained scan (one pass only).
+// [2 .. 2 + n_queries) the published words of the chained scan (kernels that pack the lists themselves).
 culsh_status alloc_query_words(culsh_ctx* ctx, int n_queries, const DedupGeometry& g, unsigned long long** words) {
-    const size_t count = 2 + (g.n_chunks == 1 ? static_cast<size_t>(n_queries) : 0);
+    (void)g;
+    const size_t count = 2 + static_cast<size_t>(n_queries);
     CULSH_TRY(arena_alloc_t(ctx, count, words));
     CULSH_HIP(hipMemsetAsync(*words, 0, count * sizeof(unsigned long long), ctx->stream));
     return CULSH_OK;
@@ -997,20 +892,47 @@ culsh_status query_from_spans(culsh_ctx* ctx, const int2* spans, const unsigned 
     bool fused = env_int("CULSH_DEDUP_TWO_PASS", 0) == 0;
     const bool several = n_chunks > 1;
     uint64_t U = 0;
-    // The output is sized by the number of raw candidates R.  One pass per query: when the previous call
-    // went to an index of the same shape (the same index, or one fitted again), its raw candidates per query (plus a quarter) size this call's output and
-    // R is read back together with the result, one host round trip instead of two; the kernel does not
-    // write beyond the capacity, and a call that would have is redone with R known.
-    // CULSH_QUERY_RAW_GUESS (tests): raw candidates per query to assume, 0 = never guess.
+    // Which kernel.  Row ranges of one bitmap pass: the bitmap kernel.  Larger ones: the two-level
+    // kernel (dedup_sparse.hip) when its level 1 fits and a query's distinct rows are expected to fit
+    // its level 2, else the bitmap kernel with several passes per query.
+    // CULSH_DEDUP_SPARSE (tests, tuning): 0 = never, 1 = whenever the geometry allows; CULSH_DEDUP_SPARSE_CAP
+    // lowers the number of level-2 entries.
+    enum Path { P_FUSED, P_PASSES, P_SPARSE };
+    SparseDedupGeometry sg;
+    const int sparse_knob = env_int("CULSH_DEDUP_SPARSE", -1);
+    const bool sparse_ok = sparse_knob != 0 && sparse_dedup_geometry(ctx, n, T, env_int("CULSH_DEDUP_SPARSE_CAP", 0), &sg);
+    auto choose_path = [&](double raw_per_query, double uniq_per_query) {  // uniq_per_query < 0: not known
+        if (sparse_ok && sparse_knob == 1) return P_SPARSE;
+        if (!several) return P_FUSED;
+        if (!sparse_ok) return P_PASSES;
+        const bool fits = uniq_per_query >= 0.0 ? uniq_per_query <= 0.9 * sg.cap : raw_per_query <= 4.0 * sg.cap;
+        return fits ? P_SPARSE : P_PASSES;
+    };
+    // The output is sized by the number of raw candidates R, an upper bound of the result.  When an
+    // earlier call went to an index of the same shape (the same index, or one fitted again), its
+    // distinct candidates per query (plus a quarter) size this call's output and R is read back together
+    // with the result, one host round trip instead of two; the kernels do not write beyond the
+    // capacity, and a call that would have is redone with R known.
+    // CULSH_QUERY_RAW_GUESS (tests): candidates per query to assume, 0 = never guess.
     const int forced_guess = env_int("CULSH_QUERY_RAW_GUESS", -1);
-    const uint64_t shape = (static_cast<uint64_t>(index->n_total_candidates) << 32 ^ static_cast<uint64_t>(index->n_total_buckets)) *
-                               0x9E3779B97F4A7C15ull +
-                           (static_cast<uint64_t>(T) << 20 ^ static_cast<uint64_t>(index->n_hashes));
-    double guess = forced_guess >= 0 ? static_cast<double>(forced_guess)
-                                     : (ctx->raw_guess_key == shape ? ctx->raw_guess_per_query : 0.0);
+    const uint64_t shape = ((static_cast<uint64_t>(index->n_total_candidates) << 32 ^ static_cast<uint64_t>(index->n_total_buckets)) *
+                                0x9E3779B97F4A7C15ull +
+                            (static_cast<uint64_t>(T) << 20 ^ static_cast<uint64_t>(index->n_hashes))) | 1ull;
+    culsh_ctx::QueryGuess* slot = nullptr;
+    for (auto& s : ctx->query_guess)
+        if (s.key == shape) slot = &s;
+    double guess_raw = forced_guess >= 0 ? static_cast<double>(forced_guess) : (slot ? slot->raw_per_query : 0.0);
+    double guess_uniq = forced_guess >= 0 ? static_cast<double>(forced_guess) : (slot ? slot->uniq_per_query : 0.0);
+    if (!slot) {
+        slot = &ctx->query_guess[ctx->query_guess_next];
+        ctx->query_guess_next = (ctx->query_guess_next + 1) % static_cast<int>(sizeof(ctx->query_guess) / sizeof(ctx->query_guess[0]));
+        *slot = culsh_ctx::QueryGuess();
+    }
     for (int attempt = 0; fused && attempt < 2; ++attempt) {
         const uint64_t bound = static_cast<uint64_t>(n_queries) * static_cast<uint64_t>(n);
-        const bool guessed = attempt == 0 && !several && guess > 0.0;
+        bool guessed = attempt == 0 && guess_raw > 0.0;
+        Path path = guessed ? choose_path(guess_raw, guess_uniq) : P_FUSED;
+        if (path == P_PASSES) guessed = false;  // lists at raw-count spacing: R sizes the output
         unsigned long long* words = const_cast<unsigned long long*>(raw_total);
         uint64_t R = 0;
         if (attempt == 1) {  // the guess was too small: R is known by now, the kernel's words start from zero again
@@ -1020,27 +942,30 @@ culsh_status query_from_spans(culsh_ctx* ctx, const int2* spans, const unsigned 
             CULSH_TRY(read_back_u64(ctx, reinterpret_cast<const uint64_t*>(raw_total), 1, &R));  // host sync 1 of 2
         }
         if (!guessed) {
-            ctx->raw_guess_key = shape;
-            ctx->raw_guess_per_query = static_cast<double>(R) / n_queries;
+            path = choose_path(static_cast<double>(R) / n_queries, -1.0);
+            slot->key = shape;
+            slot->raw_per_query = static_cast<double>(R) / n_queries;
         }
         if (!guessed && R == 0) {  // no query matched any bucket (query.cuh:358-365: counts/offsets stay, indices stay null)
             CULSH_HIP(hipMemsetAsync(out->query_candidate_counts, 0, static_cast<size_t>(n_queries) * sizeof(uint64_t), ctx->stream));
             CULSH_HIP(hipMemsetAsync(out->query_candidate_offsets, 0, (static_cast<size_t>(n_queries) + 1) * sizeof(uint64_t), ctx->stream));
             out->n_total_candidates = 0;
             out->query_candidate_indices = nullptr;
+            slot->uniq_per_query = 0.0;
             return CULSH_OK;
         }
-        // One pass: lists are packed by a chained scan over the queries; a query holds at most n
-        // distinct rows, which bounds the output when buckets overlap heavily.  Several passes: list q
-        // starts at the sum of the raw counts of the queries before it, and the gaps are closed below.
-        const uint64_t cap = several ? R
-                             : guessed ? std::min<uint64_t>(bound, static_cast<uint64_t>(guess * n_queries * 1.25) + 1024)
+        // Packed lists (bitmap kernel with one pass, two-level kernel): a chained scan over the queries
+        // places them; a query holds at most n distinct rows, which bounds the output when buckets
+        // overlap heavily.  Several bitmap passes: list q starts at the sum of the raw counts of the
+        // queries before it, and the gaps are closed below.
+        const uint64_t cap = path == P_PASSES ? R
+                             : guessed ? std::min<uint64_t>(bound, static_cast<uint64_t>(guess_uniq * n_queries * 1.25) + 1024)
                                        : std::min<uint64_t>(R, bound);
         unsigned int* err = reinterpret_cast<unsigned int*>(words + 1);  // [0] error flags, [1] ticket counter
         a.state = words + 2;
         a.ticket = err + 1;
         uint64_t* raw_offsets = nullptr;
-        if (several) {
+        if (path == P_PASSES) {
             uint64_t* raw_counts = nullptr;
             CULSH_TRY(arena_alloc_t(ctx, static_cast<size_t>(n_queries), &raw_counts));
             CULSH_TRY(arena_alloc_t(ctx, static_cast<size_t>(n_queries) + 1, &raw_offsets));
@@ -1057,27 +982,47 @@ culsh_status query_from_spans(culsh_ctx* ctx, const int2* spans, const unsigned 
         a.out = lists;
         a.err = err;
         a.capacity = cap;
-        {   // more LDS than a launch may ask for by default: allowed once per kernel and device, not per call
-            static PerDeviceOnce allowed[2];
-            PerDeviceOnce& done = allowed[several ? 1 : 0];
-            if (!done.is_set(ctx->device)) {
-                const void* kernel = several ? reinterpret_cast<const void*>(dedup_kernel<DD_FUSED_PASSES>)
-                                             : reinterpret_cast<const void*>(dedup_kernel<DD_FUSED>);
-                CULSH_HIP(hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, ctx->lds_max));
-                done.set(ctx->device);
+        if (path == P_SPARSE) {
+            SparseDedupArgs s;
+            s.spans = spans;
+            s.cand = a.cand;
+            s.out = lists;
+            s.counts = a.counts;
+            s.offsets = a.offsets;
+            s.state = a.state;
+            s.err = err;
+            s.ticket = a.ticket;
+            s.capacity = cap;
+            s.T = T;
+            s.n_queries = n_queries;
+            s.l1_per_thread = sg.l1_per_thread;
+            s.cap = sg.cap;
+            s.spin_limit = a.spin_limit;
+            s.ticks = ticks_dev;
+            CULSH_TRY(launch_dedup_sparse(ctx, s, sg));
+        } else {
+            {   // more LDS than a launch may ask for by default: allowed once per kernel and device, not per call
+                static PerDeviceOnce allowed[2];
+                PerDeviceOnce& done = allowed[path == P_PASSES ? 1 : 0];
+                if (!done.is_set(ctx->device)) {
+                    const void* kernel = path == P_PASSES ? reinterpret_cast<const void*>(dedup_kernel<DD_FUSED_PASSES>)
+                                                          : reinterpret_cast<const void*>(dedup_kernel<DD_FUSED>);
+                    CULSH_HIP(hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, ctx->lds_max));
+                    done.set(ctx->device);
+                }
             }
+            // as many workgroups as fit on the device at once (LDS and 2048 threads per CU bound it)
+            const int per_cu = static_cast<int>(std::max<size_t>(1, std::min<size_t>(2, static_cast<size_t>(ctx->lds_max) / lds_bytes)));
+            const int resident = std::max(1, ctx->n_cus * per_cu);
+            if (path == P_PASSES)
+                CULSH_LAUNCH(ctx, dedup_kernel<DD_FUSED_PASSES>, dim3(std::min(n_queries, resident)), dim3(DD_THREADS),
+                             lds_bytes, ctx->stream, a);
+            else
+                CULSH_LAUNCH(ctx, dedup_kernel<DD_FUSED>, dim3(std::min(n_queries, resident)), dim3(DD_THREADS), lds_bytes,
+                             ctx->stream, a);
+            CULSH_LAUNCH_CHECK();
         }
-        // as many workgroups as fit on the device at once (LDS and 2048 threads per CU bound it)
-        const int per_cu = static_cast<int>(std::max<size_t>(1, std::min<size_t>(2, static_cast<size_t>(ctx->lds_max) / lds_bytes)));
-        const int resident = std::max(1, ctx->n_cus * per_cu);
-        if (several)
-            CULSH_LAUNCH(ctx, dedup_kernel<DD_FUSED_PASSES>, dim3(std::min(n_queries, resident)), dim3(DD_THREADS),
-                         lds_bytes, ctx->stream, a);
-        else
-            CULSH_LAUNCH(ctx, dedup_kernel<DD_FUSED>, dim3(std::min(n_queries, resident)), dim3(DD_THREADS), lds_bytes,
-                         ctx->stream, a);
-        CULSH_LAUNCH_CHECK();
-        if (several) CULSH_TRY(exclusive_scan_u64(ctx, out->query_candidate_counts, out->query_candidate_offsets, n_queries));
+        if (path == P_PASSES) CULSH_TRY(exclusive_scan_u64(ctx, out->query_candidate_counts, out->query_candidate_offsets, n_queries));
         CULSH_HIP(hipMemcpyAsync(&ctx->pinned[0], out->query_candidate_offsets + n_queries, sizeof(uint64_t),
                                  hipMemcpyDeviceToHost, ctx->stream));
         CULSH_HIP(hipMemcpyAsync(&ctx->pinned[1], err, sizeof(unsigned int), hipMemcpyDeviceToHost, ctx->stream));
@@ -1087,13 +1032,13 @@ culsh_status query_from_spans(culsh_ctx* ctx, const int2* spans, const unsigned 
         U = ctx->pinned[0];
         const unsigned int e = static_cast<unsigned int>(ctx->pinned[1] & 0xffffffffu);
         if (guessed) {
-            ctx->raw_guess_key = shape;
-            ctx->raw_guess_per_query = static_cast<double>(ctx->pinned[2]) / n_queries;
+            slot->key = shape;
+            slot->raw_per_query = static_cast<double>(ctx->pinned[2]) / n_queries;
         }
         if (guessed && e == 2u) {  // the guess was too small and nothing else went wrong: once more with R
             dev_free(lists);
             out->query_candidate_indices = nullptr;
-            guess = 0.0;
+            guess_raw = 0.0;
             continue;
         }
         if (e != 0) {  // never seen; the two-launch path below needs no cooperation between workgroups
@@ -1103,7 +1048,9 @@ culsh_status query_from_spans(culsh_ctx* ctx, const int2* spans, const unsigned 
         } else if (U == 0) {
             dev_free(lists);
             out->query_candidate_indices = nullptr;
-        } else if (several) {
+            slot->uniq_per_query = 0.0;
+        } else if (path == P_PASSES) {
+            slot->uniq_per_query = static_cast<double>(U) / n_queries;
             int32_t* packed = nullptr;
             CULSH_HIP(dev_malloc(&packed, U * sizeof(int32_t)));
             out->query_candidate_indices = packed;
@@ -1117,15 +1064,19 @@ culsh_status query_from_spans(culsh_ctx* ctx, const int2* spans, const unsigned 
             if (err_copy == hipSuccess) err_copy = hipStreamSynchronize(ctx->stream);
             dev_free(lists);
             CULSH_HIP(err_copy);
-        } else if (U <= cap / 2 && (cap - U) * sizeof(int32_t) > (size_t(16) << 20)) {
-            // heavy overlap between tables: hand out an exact-size array instead of the bound
-            int32_t* exact = nullptr;
-            CULSH_HIP(dev_malloc(&exact, U * sizeof(int32_t)));
-            out->query_candidate_indices = exact;
-            hipError_t err_copy = hipMemcpyAsync(exact, lists, U * sizeof(int32_t), hipMemcpyDeviceToDevice, ctx->stream);
-            if (err_copy == hipSuccess) err_copy = hipStreamSynchronize(ctx->stream);
-            dev_free(lists);
-            CULSH_HIP(err_copy);
+        } else {
+            slot->uniq_per_query = static_cast<double>(U) / n_queries;
+            if (U < cap - cap / 4 && (cap - U) * sizeof(int32_t) > (size_t(1) << 20)) {
+                // more than a quarter of the block would stay unused (tables that overlap, a first call
+                // sized by the raw candidates): hand out an exact-size array instead
+                int32_t* exact = nullptr;
+                CULSH_HIP(dev_malloc(&exact, U * sizeof(int32_t)));
+                out->query_candidate_indices = exact;
+                hipError_t err_copy = hipMemcpyAsync(exact, lists, U * sizeof(int32_t), hipMemcpyDeviceToDevice, ctx->stream);
+                if (err_copy == hipSuccess) err_copy = hipStreamSynchronize(ctx->stream);
+                dev_free(lists);
+                CULSH_HIP(err_copy);
+            }
         }
         break;
     }
@@ -1159,6 +1110,10 @@ culsh_status query_from_spans(culsh_ctx* ctx, const int2* spans, const unsigned 
         CULSH_HIP(hipMemcpy(all.data(), ticks_dev, all.size() * sizeof(uint64_t), hipMemcpyDeviceToHost));
         uint64_t tk[8] = {0, 0, 0, 0, 0, 0, 0, 0};
         for (size_t i = 0; i < all.size(); ++i) tk[i & 7] += all[i];
+        if (sparse_ok)
+            fprintf(stderr, "[two-level trace, if taken] set-up %llu level-1 %llu look-back+copy-out %llu rank %llu level-2 %llu count %llu line-up %llu tail %llu\n",
+                    (unsigned long long)tk[0], (unsigned long long)tk[1], (unsigned long long)tk[2], (unsigned long long)tk[3],
+                    (unsigned long long)tk[4], (unsigned long long)tk[5], (unsigned long long)tk[6], (unsigned long long)tk[7]);
         fprintf(stderr, "[dedup trace] wpt=%d chunks=%d fused=%d | setup %llu gather %llu count %llu store %llu (ticks) | popc %llu line-up %llu look-back %llu barrier %llu\n",
                 wpt, n_chunks, int(fused), (unsigned long long)tk[0], (unsigned long long)tk[1],
                 (unsigned long long)tk[2], (unsigned long long)tk[3], (unsigned long long)tk[4],

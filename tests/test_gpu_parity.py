@@ -442,6 +442,83 @@ def test_core_query_sparse_passes_at_full_bitmap_size(ctx, c_oracle):
     ctx.free_index(ih)
 
 
+@pytest.mark.parametrize("cap", [0, 64, 8])
+@pytest.mark.parametrize("n", [3000, 70_000])
+def test_core_query_two_level_bitmap(ctx, c_oracle, monkeypatch, n, cap):
+    """The de-duplication kernel for queries with few candidates for the row range, forced on a small
+    index: one bit per block of 32 rows, the non-empty blocks ranked, one word of row bits per ranked
+    block.  Rows at both ends of a block, of a level-1 word (1024 rows) and of the index; a bucket of
+    consecutive rows (blocks filled completely: a read-out step with more rows than its place holds is
+    stored from registers); queries without candidates; tables that repeat each other's rows.  With a
+    level 2 of 64 or 8 entries the queries take many rank ranges (counted first, then stored)."""
+    _announce("two_level_bitmap", n, cap)
+    monkeypatch.setenv("CULSH_DEDUP_SPARSE", "1")
+    if cap:
+        monkeypatch.setenv("CULSH_DEDUP_SPARSE_CAP", str(cap))
+    rng = np.random.default_rng(1000 + n + cap)
+    T, nq, H = 7, 300, 2
+    sig = rng.integers(0, 12, size=(T, n, H)).astype(np.uint8)             # ~n/144 rows per bucket
+    edges = np.array([0, 31, 32, 63, 1023, 1024, 1055, n - 33, n - 32, n - 1])
+    sig[:, edges, 0] = 50
+    run = np.arange(n // 2, n // 2 + 1500)                                  # 1500 consecutive rows: full blocks
+    sig[:3, run, :] = 60
+    sig[3:, run[::2], :] = 60                                               # other tables hold half of them
+    qsig = rng.integers(0, 12, size=(T, nq, H)).astype(np.uint8)
+    qsig[:, ::7, :] = 200                                                   # no candidates
+    qsig[:, 1::7, 0] = 50                                                   # the edge rows (only)
+    qsig[:, 2::7, :] = 60                                                   # the dense run
+    qsig[:2, 3::7, :] = 60                                                  # dense run in two tables, random buckets in the rest
+    ih, _ = ctx.core_fit_index(sig, H)
+    from abi import assert_candidates_match
+
+    exp = c_oracle.query_index_c(qsig, c_oracle.fit_index_c(sig, H))
+    assert_candidates_match(ctx.core_query_index(qsig, ih), exp)
+    assert_candidates_match(ctx.core_query_index(qsig, ih), exp)            # output sized from the first call
+    ctx.free_index(ih)
+
+
+@pytest.mark.parametrize("T,n,nq", [(100, 5000, 150), (1, 2_200_000, 40), (5, 2_200_000, 64)])
+def test_core_query_two_level_bitmap_shapes(ctx, c_oracle, monkeypatch, T, n, nq):
+    """The two-level kernel with more tables than a wavefront has lanes, with one table, and on a row
+    range of more than 2^20 rows (several level-1 words per thread), where it is chosen without being
+    forced; the last row of the index is a candidate."""
+    _announce("two_level_bitmap_shapes", T, n)
+    if n < (1 << 20):
+        monkeypatch.setenv("CULSH_DEDUP_SPARSE", "1")
+    rng = np.random.default_rng(T + n)
+    H = 2
+    sig = rng.integers(0, 60, size=(T, n, H)).astype(np.uint8)
+    sig[:, n - 1, :] = 100
+    sig[:, n // 3, :] = 100
+    qsig = rng.integers(0, 60, size=(T, nq, H)).astype(np.uint8)
+    qsig[:, 5, :] = 100
+    qsig[:, 6, :] = 255
+    ih, _ = ctx.core_fit_index(sig, H)
+    from abi import assert_candidates_match
+
+    exp = c_oracle.query_index_c(qsig, c_oracle.fit_index_c(sig, H))
+    for _ in range(2):                                                      # second call: output sized from the first
+        assert_candidates_match(ctx.core_query_index(qsig, ih), exp)
+    ctx.free_index(ih)
+
+
+def test_core_query_two_level_bitmap_look_back_gives_up(ctx, monkeypatch):
+    """The two-level kernel with no polls allowed in its chained scan: the call is redone with the
+    count / scan / emit launches."""
+    _announce("two_level_give_up")
+    monkeypatch.setenv("CULSH_DEDUP_SPARSE", "1")
+    monkeypatch.setenv("CULSH_DEDUP_SPIN_LIMIT", "0")
+    rng = np.random.default_rng(15)
+    T, n, nq, H = 6, 5000, 3000, 2
+    sig = random_sigs(rng, T, n, H, "rplsh")
+    qsig = random_sigs(rng, T, nq, H, "rplsh")
+    ih, _ = ctx.core_fit_index(sig, H)
+    from abi import assert_candidates_match
+
+    assert_candidates_match(ctx.core_query_index(qsig, ih), o.query_index(qsig, o.fit_index(sig, H)))
+    ctx.free_index(ih)
+
+
 def test_core_query_two_launch_path(ctx, monkeypatch):
     """The count / scan / emit path (taken for row ranges beyond one bitmap pass) on a small case."""
     _announce("two_launch_path")
