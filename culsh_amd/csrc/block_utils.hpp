@@ -40,6 +40,11 @@ __device__ __forceinline__ uint32_t wave_inclusive_sum_dpp(uint32_t v) {
     return static_cast<uint32_t>(x);
 }
 
+// Sum over the 64 lanes, in every lane, without LDS traffic (DPP scan, then the last lane's value).
+__device__ __forceinline__ uint32_t wave_sum_dpp(uint32_t v) {
+    return static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(wave_inclusive_sum_dpp(v)), 63));
+}
+
 // Exclusive prefix sum over the workgroup (blockDim.x a multiple of 64, at most 1024).
 // `scratch` holds 17 words of type T in LDS.  Returns this thread's exclusive prefix and
 // stores the workgroup total in *total.  Contains three barriers; all threads must call it.

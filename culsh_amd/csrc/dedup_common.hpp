@@ -67,28 +67,36 @@ __device__ __forceinline__ void walk_candidates(const int32_t* __restrict__ cand
 // longer count how many younger loads may stay in flight at a use and would wait for all of them.
 // `f` is called for the lanes that hold a row only (never with -1).
 // THREADS: size of the workgroup (a multiple of 64); `tab` holds THREADS entries.
+// `kept` (optional): the caller's copy of the wavefront's table entries.  A walk of a single round
+// (n_pieces <= THREADS) leaves them there, and a later walk over the same spans that is handed them
+// back skips the piece table and its barrier (`reuse` = true; the caller places a barrier between the
+// walks if the work of `f` needs one).
 template <int THREADS, typename F>
 __device__ __forceinline__ void stream_candidates(const int32_t* __restrict__ cand, const int* s_start,
                                                   const int* s_len, const uint32_t* s_ppref, int T,
-                                                  uint32_t n_pieces, int2* tab, F&& f) {
+                                                  uint32_t n_pieces, int2* tab, F&& f, int2* kept = nullptr,
+                                                  bool reuse = false) {
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     for (uint32_t r0 = 0; r0 < n_pieces; r0 += THREADS) {
-        const uint32_t pc = r0 + static_cast<uint32_t>(tid);
-        if (pc < n_pieces) {
-            int tl = 0, th = T;  // largest t with s_ppref[t] <= pc; that span owns the piece
-            while (th - tl > 1) {
-                const int mid = (tl + th) >> 1;
-                if (s_ppref[mid] <= pc) tl = mid; else th = mid;
-            }
-            const int first = static_cast<int>(pc - s_ppref[tl]) * 64;
-            tab[tid] = make_int2(s_start[tl] + first, min(64, s_len[tl] - first));
-        }
-        __syncthreads();
         const uint32_t here = min(static_cast<uint32_t>(THREADS), n_pieces - r0);
         int2 mine = make_int2(0, 0);  // length 0: no such piece
-        {
+        if (reuse) {
+            mine = *kept;
+        } else {
+            const uint32_t pc = r0 + static_cast<uint32_t>(tid);
+            if (pc < n_pieces) {
+                int tl = 0, th = T;  // largest t with s_ppref[t] <= pc; that span owns the piece
+                while (th - tl > 1) {
+                    const int mid = (tl + th) >> 1;
+                    if (s_ppref[mid] <= pc) tl = mid; else th = mid;
+                }
+                const int first = static_cast<int>(pc - s_ppref[tl]) * 64;
+                tab[tid] = make_int2(s_start[tl] + first, min(64, s_len[tl] - first));
+            }
+            __syncthreads();
             const uint32_t pi = static_cast<uint32_t>(wave + lane * (THREADS / 64));
             if (pi < here) mine = tab[pi];
+            if (kept) *kept = mine;
         }
         const int nk = here > static_cast<uint32_t>(wave) ? static_cast<int>((here - wave + THREADS / 64 - 1) / (THREADS / 64)) : 0;  // pieces of this wavefront, <= 64
         auto fetch = [&](int k) {  // k < 64, the same in all lanes

@@ -162,24 +162,25 @@ __global__ __launch_bounds__(DD_THREADS) void dedup_sparse_kernel(SparseDedupArg
         SP_TICK(0)  // set-up
 
         // Level 1: every candidate row marks its block.
+        int2 kept = make_int2(0, 0);  // this lane's piece table entry, for the second walk
+        const bool one_round = n_pieces <= static_cast<uint32_t>(DD_THREADS);
         stream_candidates<DD_THREADS>(a.cand, s_start, s_len, s_ppref, T, n_pieces, tab, [&](int row) {
             const uint32_t blk = static_cast<uint32_t>(row) >> 5;
             atomicOr(&l1[blk >> 5].x, 1u << (blk & 31u));
-        });
+        }, &kept);
         if (n_pieces == 0) __syncthreads();  // (no barrier inside the walk then)
         SP_TICK(1)  // level-1 marks
 
-        // The previous query's list leaves now: its count was published a level-1 walk ago.
-        if (pending) flush_pending();
-        SP_TICK(2)  // look-back and copy-out of the previous query
-
-        // Rank: thread `tid` owns the level-1 words [tid * k1, tid * k1 + k1).
+        // Rank: thread `tid` owns the level-1 words [tid * k1, tid * k1 + k1).  Under it the previous
+        // query's list leaves: its count was published a level-1 walk ago, so the first wavefront's
+        // look-back finds the earlier counts in place; every wavefront then stores its part of the list.
         uint32_t mine = 0;
         for (int j = 0; j < k1; ++j) mine += __popc(l1[tid * k1 + j].x);
         uint32_t n_blocks = 0, before = 0;
         {
             const uint32_t incl = wave_inclusive_sum_dpp(mine);
             if (lane == 63) scratch[wave] = incl;
+            if (pending && wave == 0) place_list(pend_q, pend_total);
             __syncthreads();
 #pragma unroll
             for (int w = 0; w < NWAVES; ++w) {
@@ -193,10 +194,15 @@ __global__ __launch_bounds__(DD_THREADS) void dedup_sparse_kernel(SparseDedupArg
                 l1[tid * k1 + j].y = run;
                 run += __popc(l1[tid * k1 + j].x);
             }
+            if (pending) {
+                const unsigned long long base = *sh_base;
+                copy_out(pend_pw, pend_step, a.out + base + pend_wave_base, base != ~0ull);
+                pending = false;
+            }
         }
-        __syncthreads();  // the prefix words are in place (and scratch may be rewritten)
+        __syncthreads();  // the prefix words are in place, level 2 is clean, scratch and *sh_base may be rewritten
         const uint32_t n_pass = n_blocks <= cap ? 1u : (n_blocks + cap - 1u) / cap;
-        SP_TICK(3)  // rank
+        SP_TICK(3)  // rank, look-back and copy-out of the previous query
         // Level 2, rank range that starts at p0: a row finds its block's rank and sets its bit in the
         // block's entry; the same 64-bit OR leaves the block number there (every row of a block ORs
         // the same number into a word that was zero).
@@ -208,7 +214,7 @@ __global__ __launch_bounds__(DD_THREADS) void dedup_sparse_kernel(SparseDedupArg
                 if (r < cap)
                     atomicOr(reinterpret_cast<unsigned long long*>(&pb[r]),
                              (static_cast<unsigned long long>(1u << (static_cast<uint32_t>(row) & 31u)) << 32) | blk);
-            });
+            }, &kept, one_round);
             if (n_pieces == 0) __syncthreads();
         };
 
@@ -267,7 +273,7 @@ __global__ __launch_bounds__(DD_THREADS) void dedup_sparse_kernel(SparseDedupArg
                 c[j] = __popc(bits[j][0]) + __popc(bits[j][1]) + __popc(bits[j][2]) + __popc(bits[j][3]);
                 wave_total += c[j];
             }
-            wave_total = wave_sum(wave_total);
+            wave_total = wave_sum_dpp(wave_total);
             if (lane == 0) wtot[wave] = wave_total;
             unsigned int ticket_next = 0;
             if (last && tid == 0) ticket_next = atomicAdd(a.ticket, 1u);  // arrives while the rows are lined up
