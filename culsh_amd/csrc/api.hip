@@ -338,15 +338,15 @@ static culsh_status upload_params(culsh_ctx* ctx, const T* host, size_t count, T
     return upload_async(ctx, host, count * sizeof(T), *dev);
 }
 
-// `with_query`: the fit is followed by a query of the fitted rows (fit_query), which has the query path's
-// limit on the number of tables; refused here, before any device work.
-static culsh_status check_fit_args(culsh_ctx* ctx, const void* X, int n, int d, int T, int H, void* out,
-                                   bool with_query = false) {
+// More than CULSH_MAX_TABLES tables are refused by every fit (and by culsh_index_load), before any device
+// work: the query kernels give every table of a query a thread of one workgroup, so such an index could be
+// built and saved but never queried.  (The reference has no stated bound; its kernels are written for tens
+// of tables, core/fit.cuh:59-68.)
+static culsh_status check_fit_args(culsh_ctx* ctx, const void* X, int n, int d, int T, int H, void* out) {
     CULSH_REQUIRE(ctx && X && out, CULSH_ERR_INVALID, "null argument");
     CULSH_REQUIRE(n > 0 && d > 0, CULSH_ERR_INVALID, "n_samples and n_features must be positive");
     CULSH_REQUIRE(T > 0 && H > 0, CULSH_ERR_INVALID, "n_hash_tables and n_hashes must be positive");
-    CULSH_REQUIRE(T <= 65535, CULSH_ERR_LIMIT, "n_hash_tables > 65535 is not supported");
-    CULSH_REQUIRE(!with_query || T <= 1024, CULSH_ERR_LIMIT, "fit_query: n_hash_tables > 1024 is not supported");
+    CULSH_REQUIRE(T <= CULSH_MAX_TABLES, CULSH_ERR_LIMIT, "n_hash_tables > 1024 is not supported");
     CULSH_REQUIRE(static_cast<long long>(n) * T < (1ll << 31), CULSH_ERR_LIMIT,
                   "n_samples * n_hash_tables must be below 2^31 (int32 candidate positions)");
     return CULSH_OK;
@@ -521,8 +521,7 @@ template <typename T>
 static culsh_status dense_fit_once(culsh_ctx* ctx, Family fam, const T* X, int n, int d, int nT, int H, int window,
                               uint64_t seed, const T* P_host, const T* b_host, culsh_index** index_out,
                               culsh_candidates** cands_out) {
-    CULSH_TRY(check_fit_args(ctx, X, n, d, nT, H, index_out ? static_cast<void*>(index_out) : static_cast<void*>(cands_out),
-                             cands_out != nullptr));
+    CULSH_TRY(check_fit_args(ctx, X, n, d, nT, H, index_out ? static_cast<void*>(index_out) : static_cast<void*>(cands_out)));
     if (fam == FAM_PSLSH) {
         CULSH_REQUIRE(window > 0, CULSH_ERR_INVALID, "window_size must be positive");
         CULSH_REQUIRE((P_host == nullptr) == (b_host == nullptr), CULSH_ERR_INVALID,
@@ -594,8 +593,7 @@ static culsh_status dense_fit_once(culsh_ctx* ctx, Family fam, const T* X, int n
 static culsh_status minhash_fit_once(culsh_ctx* ctx, const int32_t* indices, const int32_t* indptr, int n, int d,
                                      int nT, int H, uint64_t seed, const uint32_t* A_host, const uint32_t* B_host,
                                      bool plain_keys, culsh_index** index_out, culsh_candidates** cands_out) {
-    CULSH_TRY(check_fit_args(ctx, indptr, n, d, nT, H, index_out ? static_cast<void*>(index_out) : static_cast<void*>(cands_out),
-                             cands_out != nullptr));
+    CULSH_TRY(check_fit_args(ctx, indptr, n, d, nT, H, index_out ? static_cast<void*>(index_out) : static_cast<void*>(cands_out)));
     CULSH_REQUIRE((A_host == nullptr) == (B_host == nullptr), CULSH_ERR_INVALID, "hash_a and hash_b must be given together");
     ArenaScope scope(ctx);
     CULSH_TRY(scope.begin_status);
@@ -1140,7 +1138,7 @@ culsh_status culsh_core_query_from_matched_buckets(culsh_ctx* ctx, const int32_t
 
 static culsh_status core_fit_query_once(culsh_ctx* ctx, const void* X_sig, int n, int T, int H, int S,
                                   culsh_candidates** out) {
-    CULSH_TRY(check_fit_args(ctx, X_sig, n, 1, T, H, out, true));
+    CULSH_TRY(check_fit_args(ctx, X_sig, n, 1, T, H, out));
     CULSH_REQUIRE(S > 0 && S <= 256, CULSH_ERR_INVALID, "sig_nbytes must be in [1, 256]");
     ArenaScope scope(ctx);
     CULSH_TRY(scope.begin_status);
@@ -1228,6 +1226,7 @@ culsh_status culsh_index_load(culsh_ctx* ctx, culsh_kind kind, int is_double, co
                       kind == CULSH_KIND_CORE, CULSH_ERR_INVALID, "unknown index kind");
     CULSH_REQUIRE(n_total_candidates >= 0 && n_total_buckets >= 0 && T > 0 && H > 0 && S > 0 && d >= 0,
                   CULSH_ERR_INVALID, "bad index metadata");
+    CULSH_REQUIRE(T <= CULSH_MAX_TABLES, CULSH_ERR_LIMIT, "n_hash_tables > 1024 is not supported");
     CULSH_REQUIRE(S <= 256, CULSH_ERR_LIMIT, "sig_nbytes > 256 is not supported");
     CULSH_REQUIRE((n_total_candidates == 0 || cand) && (n_total_buckets == 0 || bsig) && bco && tbo,
                   CULSH_ERR_INVALID, "missing index array");
@@ -1312,11 +1311,80 @@ culsh_status culsh_index_load(culsh_ctx* ctx, culsh_kind kind, int is_double, co
         CULSH_TRY(upload(static_cast<const uint32_t*>(param0), TH, &ix->A));
         CULSH_TRY(upload(static_cast<const uint32_t*>(param1), TH, &ix->B));
     }
+    // The key form a fit would have chosen, so that a loaded model runs the same lookup as a fitted one
+    // (bindings.cu:407-476 loads into the same Index type that fit returns).  p-stable: the value ranges
+    // come from the bucket signatures themselves (every fitted row sits in a bucket, so they are the
+    // fit's ranges).  MinHash: the rank tables depend on hash_a / hash_b / n_features only; a bucket
+    // value that is no column's hash (the fit met column ids beyond n_features and kept plain keys) sends
+    // the index back to plain keys.
+    bool compact = false;
+    if (kind == CULSH_KIND_PSLSH && n_total_buckets > 0 && H <= 1024) {
+        std::vector<int32_t> mm(2 * TH);
+        const int32_t* values = reinterpret_cast<const int32_t*>(bsig);
+        for (int t = 0; t < T; ++t) {
+            int32_t* m = mm.data() + 2 * static_cast<size_t>(t) * H;
+            for (int h = 0; h < H; ++h) { m[2 * h] = INT32_MAX; m[2 * h + 1] = INT32_MIN; }
+            for (int b = tbo[t]; b < tbo[t + 1]; ++b) {
+                const int32_t* v = values + static_cast<size_t>(b) * H;
+                for (int h = 0; h < H; ++h) {
+                    m[2 * h] = std::min(m[2 * h], v[h]);
+                    m[2 * h + 1] = std::max(m[2 * h + 1], v[h]);
+                }
+            }
+            for (int h = 0; h < H; ++h)
+                if (m[2 * h] > m[2 * h + 1]) m[2 * h] = m[2 * h + 1] = 0;  // a table without buckets
+        }
+        ctx->param_stage_off = 0;  // the rank tables go up through the pinned staging area (stream idle here)
+        CULSH_TRY(ps_build_codec_from_ranges(ctx, mm.data(), T, H, ix.get(), &compact));
+    } else if (kind == CULSH_KIND_MINHASH && n_total_buckets > 0) {
+        culsh_status st = mh_build_codec(ctx, T, H, d, ix.get(), &compact);
+        if (st == CULSH_RETRY_UNCHAINED) {  // its column sort gave up on the chained scan: once more without
+            free_mh_codec(ix.get());
+            ctx->sort_unchained = true;
+            st = mh_build_codec(ctx, T, H, d, ix.get(), &compact);
+        }
+        CULSH_REQUIRE(st != CULSH_RETRY_UNCHAINED, CULSH_ERR_INTERNAL, "radix sort: chained scan gave up twice");
+        CULSH_TRY(st);
+    }
     CULSH_HIP(dev_malloc(&ix->bucket_keys, std::max<size_t>(1, static_cast<size_t>(n_total_buckets) * ix->key_w) * 4));
-    CULSH_TRY(launch_sig_to_keys(ctx, ix->all_bucket_signatures, n_total_buckets, S, enc, ix->key_w, ix->bucket_keys));
+    if (compact) {
+        uint32_t* unknown = nullptr;
+        CULSH_TRY(arena_alloc_t(ctx, 1, &unknown));
+        CULSH_HIP(hipMemsetAsync(unknown, 0, sizeof(uint32_t), ctx->stream));
+        for (int t = 0; t < T; ++t) {  // the tables hold different numbers of buckets: one launch each
+            const size_t first = static_cast<size_t>(tbo[t]), count = static_cast<size_t>(tbo[t + 1] - tbo[t]);
+            uint32_t* keys = ix->bucket_keys + first * ix->key_w;
+            if (kind == CULSH_KIND_PSLSH)
+                CULSH_TRY(launch_ps_compress(ctx, reinterpret_cast<const int32_t*>(ix->all_bucket_signatures) + first * H, count,
+                                             1, H, ix.get(), keys, t));
+            else
+                CULSH_TRY(launch_mh_sig_to_keys(ctx, reinterpret_cast<const uint32_t*>(ix->all_bucket_signatures) + first * H,
+                                                count, ix.get(), keys, 1, t, unknown));
+        }
+        uint32_t any_unknown = 0;
+        CULSH_TRY(read_back_u32(ctx, unknown, 1, &any_unknown));
+        if (any_unknown) {
+            free_mh_codec(ix.get());
+            ix->enc = ENC_BE;
+            ix->key_w = key_words(ENC_BE, S);
+            dev_free(ix->bucket_keys);
+            ix->bucket_keys = nullptr;
+            CULSH_HIP(dev_malloc(&ix->bucket_keys, std::max<size_t>(1, static_cast<size_t>(n_total_buckets) * ix->key_w) * 4));
+            compact = false;
+        }
+    }
+    if (!compact)
+        CULSH_TRY(launch_sig_to_keys(ctx, ix->all_bucket_signatures, n_total_buckets, S, ix->enc, ix->key_w, ix->bucket_keys));
     CULSH_TRY(build_key_directory(ctx, ix.get(), static_cast<size_t>(n_total_buckets)));
     CULSH_TRY(arena_end(ctx));
     *out = ix.release();
+    return CULSH_OK;
+}
+
+culsh_status culsh_index_key_form(const culsh_index* ix, int32_t* key_words_out, int32_t* encoding) {
+    CULSH_REQUIRE(ix && key_words_out && encoding, CULSH_ERR_INVALID, "null argument");
+    *key_words_out = ix->key_w;
+    *encoding = static_cast<int32_t>(ix->enc);
     return CULSH_OK;
 }
 

@@ -292,9 +292,12 @@ culsh_status ps_build_codec(culsh_ctx* ctx, const int32_t* sig, int n, int T, in
                             bool* compressed, int32_t* mm_folded = nullptr);
 // [T*H][2] range words in the arena, preset to INT_MAX / INT_MIN
 culsh_status ps_minmax_prepare(culsh_ctx* ctx, int T, int H, int32_t** mm_dev);
-// int32 hashes [T][rows][H] -> compressed key words [T][rows][ix->key_w]
+// The same from value ranges on the host: mm[2c] / mm[2c + 1] = smallest / largest hash of column c = t * H + h.
+culsh_status ps_build_codec_from_ranges(culsh_ctx* ctx, const int32_t* mm, int T, int H, culsh_index* ix, bool* compressed);
+// int32 hashes [T][rows][H] -> compressed key words [T][rows][ix->key_w]; the T tables of `sig` are the
+// index's tables t0 .. t0 + T - 1
 culsh_status launch_ps_compress(culsh_ctx* ctx, const int32_t* sig, size_t rows, int T, int H, const culsh_index* ix,
-                                uint32_t* keys);
+                                uint32_t* keys, int t0 = 0);
 // ix->bucket_keys -> little-endian int32 signatures of the buckets (needs table_bucket_offsets)
 culsh_status launch_ps_keys_to_sig(culsh_ctx* ctx, const culsh_index* ix, size_t count, const uint64_t* count_dev,
                                    uint8_t* sig);
@@ -312,9 +315,11 @@ culsh_status mh_build_codec(culsh_ctx* ctx, int T, int H, int d, culsh_index* ix
 // keys.  Null (queries): any id is hashed as it is; ids the fit never saw match nothing.
 culsh_status launch_minhash_rank(culsh_ctx* ctx, const int32_t* indices, const int32_t* indptr, int n, int T, int H,
                                  const culsh_index* ix, uint32_t* fit_flag, uint32_t* keys);
-// uint32 signatures [T][rows][H] -> packed rank codes
+// uint32 signatures [T][rows][H] -> packed rank codes; T < 0: all tables of the index, else the T tables
+// t0 .. t0 + T - 1.  unknown_flag (device, may be null) is set to 1 when a value is no column's hash
+// (its code then matches nothing).
 culsh_status launch_mh_sig_to_keys(culsh_ctx* ctx, const uint32_t* sig, size_t rows, const culsh_index* ix,
-                                   uint32_t* keys);
+                                   uint32_t* keys, int T = -1, int t0 = 0, uint32_t* unknown_flag = nullptr);
 // ix->bucket_keys -> little-endian uint32 signatures of the buckets (needs table_bucket_offsets)
 culsh_status launch_mh_keys_to_sig(culsh_ctx* ctx, const culsh_index* ix, size_t count, const uint64_t* count_dev,
                                    uint8_t* sig);
@@ -360,6 +365,10 @@ culsh_status query_from_matched(culsh_ctx* ctx, const int32_t* matched, int n_qu
 // lookup + candidate retrieval from key words [T][n_queries][key_w]
 culsh_status query_from_keys(culsh_ctx* ctx, const uint32_t* q_keys, int n_queries, const culsh_index* index,
                              culsh_candidates* out);
+
+// Most hash tables an index may have (every fit, load and query checks it): the query kernels give each
+// table of a query one thread of a workgroup.
+constexpr int CULSH_MAX_TABLES = 1024;
 
 // Elements that can be read (not used) behind the last one of an index's all_candidate_indices: the
 // query kernels fetch whole 64-row pieces.

@@ -191,12 +191,14 @@ __global__ __launch_bounds__(NTHREADS) void minhash_rank_kernel(const int32_t* _
 // uint32 signatures [T][rows][H] (reference layout) -> packed rank codes.  A value is looked
 // up among the sorted hash values of its hash function (rank = position).
 __global__ __launch_bounds__(256) void mh_sig_to_keys_kernel(const uint32_t* __restrict__ sig, size_t rows, int T,
-                                                            int H, int d, int bits, int W,
+                                                            int H, int d, int bits, int W, int t0,
                                                             const uint32_t* __restrict__ inv,
-                                                            uint32_t* __restrict__ keys) {
+                                                            uint32_t* __restrict__ keys,
+                                                            uint32_t* __restrict__ unknown_flag) {
     const size_t item = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
     if (item >= rows * T) return;
-    const int t = static_cast<int>(item / rows);
+    const int t = t0 + static_cast<int>(item / rows);  // t0: number of the first table of `sig`
+    bool unknown = false;  // a value that is no column's hash (unknown_flag, may be null, is set to 1 then)
     const uint32_t* s = sig + item * H;
     uint32_t* k = keys + item * W;
     unsigned long long acc = 0;
@@ -218,6 +220,7 @@ __global__ __launch_bounds__(256) void mh_sig_to_keys_kernel(const uint32_t* __r
                 if (mk == key) { code = static_cast<uint32_t>(mid); break; }
                 if (mk < key) lo = mid + 1; else hi = mid - 1;
             }
+            unknown |= code == static_cast<uint32_t>(d) + 1u;
         }
         acc = (acc << bits) | code;
         nbits += bits;
@@ -228,6 +231,7 @@ __global__ __launch_bounds__(256) void mh_sig_to_keys_kernel(const uint32_t* __r
         }
     }
     if (nbits > 0) k[w++] = static_cast<uint32_t>(acc << (32 - nbits));
+    if (unknown && unknown_flag) *unknown_flag = 1u;
 }
 
 // Signatures of the buckets from their rank keys.  A workgroup takes `bpb` consecutive buckets (a
@@ -371,12 +375,13 @@ culsh_status launch_minhash_rank(culsh_ctx* ctx, const int32_t* indices, const i
 }
 
 culsh_status launch_mh_sig_to_keys(culsh_ctx* ctx, const uint32_t* sig, size_t rows, const culsh_index* ix,
-                                   uint32_t* keys) {
-    const size_t items = rows * ix->n_hash_tables;
+                                   uint32_t* keys, int T, int t0, uint32_t* unknown_flag) {
+    if (T < 0) T = ix->n_hash_tables;
+    const size_t items = rows * T;
     if (items == 0) return CULSH_OK;
     CULSH_REQUIRE(items / 256 < (1ull << 31), CULSH_ERR_LIMIT, "too many items");
-    CULSH_LAUNCH(ctx, mh_sig_to_keys_kernel, dim3(div_up(items, 256)), dim3(256), 0, ctx->stream, sig, rows,
-                 ix->n_hash_tables, ix->n_hashes, ix->mhc.d, ix->mhc.bits, ix->key_w, ix->mhc.inv, keys);
+    CULSH_LAUNCH(ctx, mh_sig_to_keys_kernel, dim3(div_up(items, 256)), dim3(256), 0, ctx->stream, sig, rows, T,
+                 ix->n_hashes, ix->mhc.d, ix->mhc.bits, ix->key_w, t0, ix->mhc.inv, keys, unknown_flag);
     CULSH_LAUNCH_CHECK();
     return CULSH_OK;
 }

@@ -125,7 +125,7 @@ __device__ __forceinline__ void ps_compress_item(const int32_t* __restrict__ s, 
 // one table (all but T - 1 of them) looks ranks up there.
 template <bool VEC4>
 __global__ __launch_bounds__(256) void ps_compress_kernel(const int32_t* __restrict__ sig, size_t rows, int T, int H,
-                                                         int bits, int rmax, int W, int use_lds,
+                                                         int bits, int rmax, int W, int use_lds, int t0,
                                                          const int32_t* __restrict__ vmin,
                                                          const int32_t* __restrict__ range,
                                                          const uint32_t* __restrict__ fwd,
@@ -134,8 +134,8 @@ __global__ __launch_bounds__(256) void ps_compress_kernel(const int32_t* __restr
     const size_t items = rows * T;
     const size_t item0 = static_cast<size_t>(blockIdx.x) * 256;
     const size_t item = item0 + threadIdx.x;
-    const int t_first = static_cast<int>(item0 / rows);
-    const int t_last = static_cast<int>(min(item0 + 255, items - 1) / rows);
+    const int t_first = t0 + static_cast<int>(item0 / rows);  // t0: number of the first table of `sig`
+    const int t_last = t0 + static_cast<int>(min(item0 + 255, items - 1) / rows);
     const bool staged = use_lds && t_first == t_last;  // uniform over the workgroup
     if (staged) {
         const int lut = H * rmax;
@@ -154,7 +154,7 @@ __global__ __launch_bounds__(256) void ps_compress_kernel(const int32_t* __restr
         const int32_t* lv = reinterpret_cast<const int32_t*>(ps_lut + H * rmax);
         ps_compress_item<VEC4>(s, k, H, bits, rmax, ps_lut, lv, lv + H);
     } else {
-        const int t = static_cast<int>(item / rows);
+        const int t = t0 + static_cast<int>(item / rows);
         ps_compress_item<VEC4>(s, k, H, bits, rmax, fwd + static_cast<size_t>(t) * H * rmax, vmin + t * H,
                                range + t * H);
     }
@@ -277,7 +277,13 @@ culsh_status ps_build_codec(culsh_ctx* ctx, const int32_t* sig, int n, int T, in
     std::vector<int32_t> mm(static_cast<size_t>(TH) * 2);
     CULSH_HIP(hipMemcpyAsync(mm.data(), mm_dev, mm.size() * sizeof(int32_t), hipMemcpyDeviceToHost, ctx->stream));
     CULSH_HIP(hipStreamSynchronize(ctx->stream));
+    return ps_build_codec_from_ranges(ctx, mm.data(), T, H, ix, compressed);
+}
 
+culsh_status ps_build_codec_from_ranges(culsh_ctx* ctx, const int32_t* mm, int T, int H, culsh_index* ix, bool* compressed) {
+    *compressed = false;
+    const int TH = T * H;
+    if (H > 1024) return CULSH_OK;
     long long rmax = 1;
     for (int c = 0; c < TH; ++c) rmax = std::max(rmax, static_cast<long long>(mm[2 * c + 1]) - mm[2 * c] + 1);
     int bits = 1;
@@ -325,7 +331,7 @@ culsh_status ps_build_codec(culsh_ctx* ctx, const int32_t* sig, int n, int T, in
 }
 
 culsh_status launch_ps_compress(culsh_ctx* ctx, const int32_t* sig, size_t rows, int T, int H, const culsh_index* ix,
-                                uint32_t* keys) {
+                                uint32_t* keys, int t0) {
     const size_t items = rows * T;
     if (items == 0) return CULSH_OK;
     CULSH_REQUIRE(items / 256 < (1ull << 31), CULSH_ERR_LIMIT, "too many items");
@@ -335,10 +341,10 @@ culsh_status launch_ps_compress(culsh_ctx* ctx, const int32_t* sig, size_t rows,
     const size_t lds = use_lds ? (lut_words + 2 * static_cast<size_t>(H)) * sizeof(uint32_t) : 0;
     if (H % 4 == 0 && reinterpret_cast<uintptr_t>(sig) % 16 == 0)
         CULSH_LAUNCH(ctx, ps_compress_kernel<true>, dim3(div_up(items, 256)), dim3(256), lds, ctx->stream, sig, rows, T,
-                     H, pc.bits, pc.rmax, ix->key_w, use_lds, pc.vmin, pc.range, pc.fwd, keys);
+                     H, pc.bits, pc.rmax, ix->key_w, use_lds, t0, pc.vmin, pc.range, pc.fwd, keys);
     else
         CULSH_LAUNCH(ctx, ps_compress_kernel<false>, dim3(div_up(items, 256)), dim3(256), lds, ctx->stream, sig, rows, T,
-                     H, pc.bits, pc.rmax, ix->key_w, use_lds, pc.vmin, pc.range, pc.fwd, keys);
+                     H, pc.bits, pc.rmax, ix->key_w, use_lds, t0, pc.vmin, pc.range, pc.fwd, keys);
     CULSH_LAUNCH_CHECK();
     return CULSH_OK;
 }

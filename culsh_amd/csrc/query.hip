@@ -1123,7 +1123,8 @@ culsh_status query_from_spans(culsh_ctx* ctx, const int2* spans, const unsigned 
 }
 
 culsh_status check_query_args(int n_queries, const culsh_index* index) {
-    CULSH_REQUIRE(index->n_hash_tables <= DD_THREADS, CULSH_ERR_LIMIT, "query: n_hash_tables > 1024 is not supported");
+    static_assert(CULSH_MAX_TABLES <= DD_THREADS, "one thread per table");
+    CULSH_REQUIRE(index->n_hash_tables <= CULSH_MAX_TABLES, CULSH_ERR_LIMIT, "query: n_hash_tables > 1024 is not supported");
     CULSH_REQUIRE(n_queries > 0, CULSH_ERR_INVALID, "query: n_queries must be positive");
     CULSH_REQUIRE(index->n_total_candidates / index->n_hash_tables > 0, CULSH_ERR_INVALID, "query: empty index");
     return CULSH_OK;

@@ -17,7 +17,8 @@
  *     (the reference binding synchronises the same way, bindings.cu:41,68,97).
  *   - Objects are not thread-safe; one context per host thread.
  *   - Limits: n_samples * n_hash_tables < 2^31 (int32 candidate positions, as
- *     core/index.cuh:32), n_hash_tables <= 65535.
+ *     core/index.cuh:32); n_hash_tables <= 1024 for every fit, load and query (refused with
+ *     CULSH_ERR_LIMIT before any device work: a query gives each table one thread of a workgroup).
  *
  * Citations are file:line in the reference checkout (cuda/culsh/src/... unless noted).
  */
@@ -195,6 +196,11 @@ culsh_status culsh_core_fit_query(culsh_ctx*, const void* X_sig_dev, int n_sampl
 
 /* ---- index object ------------------------------------------------------------------------ */
 culsh_status culsh_index_get_meta(const culsh_index*, culsh_index_meta* out);
+/* Internal form of the lookup keys (no counterpart in the reference; for tests and tuning): 32-bit words
+ * per bucket key, and how a signature becomes a key: 0 = its bytes, big-endian word by word, 1 = one bit per
+ * RPLSH hash, 2 = p-stable hashes as ranks among the values seen at fit time, 3 = MinHash values as ranks
+ * of their columns.  A loaded index gets the form a fit of the same data would have chosen. */
+culsh_status culsh_index_key_form(const culsh_index*, int32_t* key_words, int32_t* encoding);
 /* Number of elements / element size of one of the index's arrays (0 elements when absent). */
 culsh_status culsh_index_array_info(const culsh_index*, culsh_array which, uint64_t* n_elems, uint32_t* elem_size);
 /* Copies an array to the host (getters of bindings.cu:341-378) or to a device buffer. */

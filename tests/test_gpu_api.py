@@ -331,6 +331,63 @@ def test_minhash_save_load_and_fit_query(tmp_path):
         lsh.fit(X64)
 
 
+def _key_form(index):
+    """(key words per bucket, encoding) of an index object of the extension-module surface."""
+    import ctypes as C
+
+    w, enc = C.c_int32(), C.c_int32()
+    from culsh_amd import _lib as L
+
+    L.check(index._lib.culsh_index_key_form(index._h, C.byref(w), C.byref(enc)))
+    return w.value, enc.value
+
+
+def test_loaded_models_look_buckets_up_like_fitted_ones(tmp_path):
+    """A model that comes back from `load` runs the same bucket lookup as the one `fit` returned: the
+    loaded index has the fitted index's key form (p-stable hashes as ranks of the values seen at fit
+    time, 8 words -> 2; MinHash values as ranks of their columns, 4 words -> 2; RPLSH one bit per hash)
+    and returns the same candidates, also for queries whose hashes no fitted row has.  A MinHash model
+    fitted on column ids at or beyond n_features keeps plain keys on both sides."""
+    from culsh_amd import MinHashLSH, MinHashLSHModel, PStableLSH, PStableLSHModel, RPLSH, RPLSHModel
+
+    X = dense(3000, 32, np.float32, seed=11)
+    Q = np.concatenate([X[:150], 40.0 * dense(50, 32, np.float32, seed=12)])     # far-away queries: unseen hash values
+    for est, cls, words, enc in ((PStableLSH(n_hash_tables=6, n_hashes=8, window_size=4, seed=3), PStableLSHModel, 2, 2),
+                                 (RPLSH(n_hash_tables=6, n_hashes=40, seed=3), RPLSHModel, 2, 1)):
+        model = est.fit(X)
+        path = os.path.join(tmp_path, cls.__name__ + ".npz")
+        model.save(path)
+        loaded = cls.load(path)
+        assert _key_form(model.index) == _key_form(loaded.index)
+        assert _key_form(model.index)[1] == enc and _key_form(model.index)[0] <= words
+        a, b = model.query(Q), loaded.query(Q)
+        np.testing.assert_array_equal(a.get_indices(), b.get_indices())
+        np.testing.assert_array_equal(a.get_offsets(), b.get_offsets())
+        assert a.get_counts()[:150].min() >= 1
+    S = sparse(2000, 300, 0.04)
+    lsh = MinHashLSH(n_hash_tables=8, n_hashes=4, seed=9)
+    model = lsh.fit(S)
+    path = os.path.join(tmp_path, "mh.npz")
+    model.save(path)
+    loaded = MinHashLSHModel.load(path)
+    assert _key_form(model.index) == (2, 3) == _key_form(loaded.index)                # 4 x 9 bits
+    a, b = model.query(S[:200]), loaded.query(S[:200])
+    np.testing.assert_array_equal(a.get_indices(), b.get_indices())
+    np.testing.assert_array_equal(a.get_offsets(), b.get_offsets())
+    # column ids beyond n_features: the fit falls back to plain keys, and so does the load
+    wide, wide_q = S.copy(), S[:200].copy()
+    wide.indices = (wide.indices + 5).astype(np.int32)                                 # ids up to 304 >= 300 = n_features
+    wide_q.indices = (wide_q.indices + 5).astype(np.int32)
+    model = lsh.fit(wide)
+    path = os.path.join(tmp_path, "mh_wide.npz")
+    model.save(path)
+    loaded = MinHashLSHModel.load(path)
+    assert _key_form(model.index) == (4, 0) == _key_form(loaded.index)
+    a, b = model.query(wide_q), loaded.query(wide_q)
+    np.testing.assert_array_equal(a.get_indices(), b.get_indices())
+    np.testing.assert_array_equal(a.get_offsets(), b.get_offsets())
+
+
 # ---------------------------------------------------------------- the reference's import name
 def test_reference_import_name_runs_the_reference_usage(tmp_path):
     """A caller written against rishic3/cuLSH (README usage; python/tests/test_rplsh.py:145-174) runs

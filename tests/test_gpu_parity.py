@@ -197,14 +197,40 @@ def test_fit_after_sort_gives_up_touches_nothing_it_should_not(c_oracle, monkeyp
         own.close()
 
 
-def test_fit_query_refuses_more_than_1024_tables_up_front(ctx):
-    """The query path handles up to 1024 tables; fit_query says so before it hashes or sorts anything."""
+def test_more_than_1024_tables_are_refused_up_front(ctx):
+    """The query path handles up to 1024 tables (one thread of a workgroup per table), so no index with
+    more is ever built: fit, fit_query and load of every family say so before they hash, sort or copy
+    anything, instead of handing out an index that no query accepts."""
+    import ctypes as C
+
+    from abi import hp
+    from culsh_amd import _lib as L
+
     sig = np.zeros((1025, 4, 1), dtype=np.uint8)
     with pytest.raises(RuntimeError, match="1024"):
         ctx.core_fit_query(sig, 1)
+    with pytest.raises(RuntimeError, match="1024"):
+        ctx.core_fit_index(sig, 1)
     X = np.zeros((4, 8), dtype=np.float32)
     with pytest.raises(RuntimeError, match="1024"):
         ctx.rplsh_fit_query(X, 1025, 1)
+    with pytest.raises(RuntimeError, match="1024"):
+        ctx.rplsh_fit(X, 1025, 1)
+    with pytest.raises(RuntimeError, match="1024"):
+        ctx.pslsh_fit(X, 1025, 1, 4)
+    indptr = np.arange(5, dtype=np.int32)
+    with pytest.raises(RuntimeError, match="1024"):
+        ctx.minhash_fit(np.zeros(4, np.int32), indptr, 8, 1025, 1)
+    # a saved index with 1025 tables of one bucket each
+    T, n = 1025, 2
+    cand = np.tile(np.arange(n, dtype=np.int32), T)
+    bsig = np.zeros(T, dtype=np.uint8)
+    bco = (np.arange(T + 1) * n).astype(np.int32)
+    tbo = np.arange(T + 1, dtype=np.int32)
+    ih = C.c_void_p()
+    rc = ctx.lib.culsh_index_load(ctx.h, L.KIND_CORE, 0, hp(cand), hp(bsig), hp(bco), hp(tbo), None, None,
+                                  T * n, T, T, 1, 1, 0, 0, C.byref(ih))
+    assert rc == L.ERR_LIMIT and b"1024" in ctx.lib.culsh_last_error()
 
 
 def test_core_fit_index_single_bucket_per_table(ctx):
@@ -553,7 +579,7 @@ def test_core_query_after_look_back_gives_up(ctx, monkeypatch):
 @pytest.mark.parametrize("T,n,nq,H", [(90, 3000, 400, 3), (1024, 300, 40, 2)])
 def test_core_query_more_than_64_tables(ctx, T, n, nq, H):
     """More tables than a wavefront has lanes (the spans of the next query are then not prefetched),
-    up to the most a query supports (one thread per table); one more is an error, not a wrong answer."""
+    up to the most an index may have (one thread per table)."""
     _announce("many_tables", T)
     rng = np.random.default_rng(6)
     sig = random_sigs(rng, T, n, H, "rplsh")
@@ -563,12 +589,6 @@ def test_core_query_more_than_64_tables(ctx, T, n, nq, H):
 
     assert_candidates_match(ctx.core_query_index(qsig, ih), o.query_index(qsig, o.fit_index(sig, H)))
     ctx.free_index(ih)
-    if T == 1024:
-        too_many = rng.integers(0, 2, size=(T + 1, 20, 1), dtype=np.uint8)
-        ih2, _ = ctx.core_fit_index(too_many, 1)
-        with pytest.raises(RuntimeError, match="n_hash_tables > 1024"):
-            ctx.core_query_index(too_many[:, :5], ih2)
-        ctx.free_index(ih2)
 
 
 def test_core_query_tables_that_overlap_completely(ctx, c_oracle):
