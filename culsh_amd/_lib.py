@@ -95,6 +95,7 @@ PROTOTYPES = {
     "culsh_core_query_from_matched_buckets": [_P, _P, _I, _P, _PP],
     "culsh_core_fit_query": [_P, _P, _I, _I, _I, _I, _PP],
     "culsh_index_get_meta": [_P, C.POINTER(IndexMeta)],
+    "culsh_debug_arena_state": [_P, C.POINTER(C.c_uint64)],
     "culsh_index_key_form": [_P, C.POINTER(C.c_int32), C.POINTER(C.c_int32)],
     "culsh_index_array_info": [_P, _I, C.POINTER(C.c_uint64), C.POINTER(C.c_uint32)],
     "culsh_index_copy_array": [_P, _P, _I, _P, _U64, _I],
@@ -107,6 +108,7 @@ PROTOTYPES = {
 _SPECIAL = {
     "culsh_last_error": (C.c_char_p, []),
     "culsh_version": (C.c_char_p, []),
+    "culsh_debug_allocation_calls": (C.c_uint64, []),
     "culsh_ctx_destroy": (None, [_P]),
     "culsh_memory_trim": (None, []),
     "culsh_ctx_stream": (_P, [_P]),

@@ -15,6 +15,9 @@
 
 namespace culsh_amd {
 
+std::atomic<uint64_t> g_allocation_calls{0};
+
+
 // ---------------------------------------------------------------- errors
 static thread_local std::string g_last_error;
 
@@ -41,11 +44,40 @@ culsh_status arena_begin(culsh_ctx* ctx) {
         // the new block first: a grow that fails keeps the arena there is
         const size_t want = align_up(ctx->arena_want + ctx->arena_want / 8, 1 << 20);
         void* p = nullptr;
-        if (hipMalloc(&p, want) == hipSuccess) {
-            if (ctx->arena) (void)hipFree(ctx->arena);
+        count_allocation_call();
+        hipError_t grown = hipMalloc(&p, want);
+        if (grown != hipSuccess && ctx->arena) {
+            // both blocks do not fit side by side: the stream is idle and nothing in the old one is
+            // live, so it goes first and the new one is tried once more
+            (void)hipGetLastError();
+            count_allocation_call();
+            (void)hipFree(ctx->arena);
+            const size_t old_cap = ctx->arena_cap;
+            ctx->arena = nullptr;
+            ctx->arena_cap = 0;
+            count_allocation_call();
+            grown = hipMalloc(&p, want);
+            if (grown != hipSuccess) {  // not even alone: back to the size that did fit
+                (void)hipGetLastError();
+                void* old = nullptr;
+                count_allocation_call();
+                if (hipMalloc(&old, old_cap) == hipSuccess) {
+                    ctx->arena = static_cast<char*>(old);
+                    ctx->arena_cap = old_cap;
+                } else {
+                    (void)hipGetLastError();
+                }
+            }
+        }
+        if (grown == hipSuccess) {
+            if (ctx->arena) {  // (the grow fitted beside it)
+                count_allocation_call();
+                (void)hipFree(ctx->arena);
+            }
             ctx->arena = static_cast<char*>(p);
             ctx->arena_cap = want;
         } else {
+            ++ctx->arena_grow_failures;  // visible through culsh_debug_arena_state
             (void)hipGetLastError();  // what does not fit falls back to per-allocation blocks
         }
     }
@@ -66,8 +98,10 @@ culsh_status arena_alloc(culsh_ctx* ctx, size_t bytes, void** out) {
         return CULSH_OK;
     }
     void* p = nullptr;
+    count_allocation_call();
     CULSH_HIP(hipMalloc(&p, bytes));
     ctx->overflow.push_back(p);
+    ++ctx->arena_overflow_blocks;
     *out = p;
     return CULSH_OK;
 }
@@ -96,7 +130,7 @@ StageTimer::StageTimer(culsh_ctx* c, const char* name) : ctx(c) {
         if (!c->prof_pool.empty()) {
             e = c->prof_pool.back();
             c->prof_pool.pop_back();
-        } else if (hipEventCreate(&e) != hipSuccess) {
+        } else if (count_allocation_call(), hipEventCreate(&e) != hipSuccess) {
             (void)hipGetLastError();
             return;
         }
@@ -128,7 +162,10 @@ void profile_collect(culsh_ctx* ctx) {
 culsh_status arena_end(culsh_ctx* ctx) {
     hipError_t e = hipStreamSynchronize(ctx->stream);
     if (e == hipSuccess) profile_collect(ctx);
-    for (void* p : ctx->overflow) (void)hipFree(p);
+    for (void* p : ctx->overflow) {
+        count_allocation_call();
+        (void)hipFree(p);
+    }
     ctx->overflow.clear();
     if (e != hipSuccess) {
         set_error("stream synchronize failed: %s", hipGetErrorString(e));
@@ -315,6 +352,7 @@ culsh_status upload_async(culsh_ctx* ctx, const void* host, size_t bytes, void* 
         ctx->param_stage = nullptr;
         ctx->param_stage_cap = 0;
         const size_t cap = std::max<size_t>(size_t(1) << 20, 2 * align_up(bytes, 256));
+        count_allocation_call();
         if (hipHostMalloc(reinterpret_cast<void**>(&ctx->param_stage), cap, hipHostMallocDefault) != hipSuccess) {
             (void)hipGetLastError();
             ctx->param_stage = nullptr;
@@ -512,6 +550,10 @@ static culsh_status finish_fit(culsh_ctx* ctx, uint32_t* keys, int n, int T, int
     int32_t* item_to_bucket = nullptr;
     if (cands_or_null) CULSH_TRY(arena_alloc_t(ctx, static_cast<size_t>(n) * T, &item_to_bucket));
     CULSH_TRY(fit_index_from_keys(ctx, keys, n, T, H, S, enc, W, item_to_bucket, ix));
+    // A family's own flag has come back with the end-of-build read-back (MinHash rank keys: a column id
+    // at or beyond n_features).  The keys are void then; the caller fits again with plain keys, and the
+    // query of the fitted rows is not run on an index that is about to be dropped.
+    if (ctx->aux_flag_host) return CULSH_RETRY_PLAIN_KEYS;
     if (cands_or_null)  // core/fit_query.cuh:46-50
         CULSH_TRY(query_from_matched(ctx, item_to_bucket, n, ix, cands_or_null));
     return CULSH_OK;
@@ -648,10 +690,13 @@ static culsh_status minhash_fit_once(culsh_ctx* ctx, const int32_t* indices, con
         CULSH_REQUIRE(cands, CULSH_ERR_NOMEM, "host allocation failed");
         cands->device = ctx->device;
     }
-    CULSH_TRY(finish_fit(ctx, keys, n, nT, H, 4 * H, enc, W, ix.get(), cands.get()));  // minhash.cu:37
-    if (ranked && ctx->aux_flag_host) {  // a column id at or beyond n_features: these keys are void
-        CULSH_TRY(arena_end(ctx));
-        return CULSH_RETRY_PLAIN_KEYS;
+    {
+        const culsh_status st = finish_fit(ctx, keys, n, nT, H, 4 * H, enc, W, ix.get(), cands.get());  // minhash.cu:37
+        if (st == CULSH_RETRY_PLAIN_KEYS) {  // a column id at or beyond n_features: these keys are void
+            CULSH_TRY(arena_end(ctx));
+            return CULSH_RETRY_PLAIN_KEYS;
+        }
+        CULSH_TRY(st);
     }
     ix->n_features = d;
     ix->seed = seed;
@@ -791,12 +836,9 @@ culsh_status culsh_ctx_create(int device, culsh_ctx** out) {
         return CULSH_ERR_NOMEM;
     }
     ctx->pinned = static_cast<uint64_t*>(pinned);
-    const culsh_status scratch_status = static_scratch_init(device);
-    if (scratch_status != CULSH_OK) {
-        (void)hipHostFree(pinned);
-        (void)hipStreamDestroy(ctx->stream);
-        return scratch_status;
-    }
+    // The workspace of the entry point that allocates nothing.  If its address cannot be had, only that
+    // entry point is affected (it reports the missing workspace); everything else works without it.
+    if (static_scratch_init(device) != CULSH_OK) (void)hipGetLastError();
     *out = ctx.release();
     return CULSH_OK;
 }
@@ -810,7 +852,10 @@ void culsh_ctx_destroy(culsh_ctx* ctx) {
     }
     profile_collect(ctx);
     for (hipEvent_t e : ctx->prof_pool) (void)hipEventDestroy(e);
-    for (void* p : ctx->overflow) (void)hipFree(p);
+    for (void* p : ctx->overflow) {
+        count_allocation_call();
+        (void)hipFree(p);
+    }
     if (ctx->arena) (void)hipFree(ctx->arena);
     if (ctx->pinned) (void)hipHostFree(ctx->pinned);
     if (ctx->param_stage) (void)hipHostFree(ctx->param_stage);
@@ -1378,6 +1423,17 @@ culsh_status culsh_index_load(culsh_ctx* ctx, culsh_kind kind, int is_double, co
     CULSH_TRY(build_key_directory(ctx, ix.get(), static_cast<size_t>(n_total_buckets)));
     CULSH_TRY(arena_end(ctx));
     *out = ix.release();
+    return CULSH_OK;
+}
+
+uint64_t culsh_debug_allocation_calls(void) { return g_allocation_calls.load(std::memory_order_relaxed); }
+
+culsh_status culsh_debug_arena_state(const culsh_ctx* ctx, uint64_t out[4]) {
+    CULSH_REQUIRE(ctx && out, CULSH_ERR_INVALID, "null argument");
+    out[0] = ctx->arena_cap;
+    out[1] = ctx->arena_off;
+    out[2] = ctx->arena_overflow_blocks;
+    out[3] = ctx->arena_grow_failures;
     return CULSH_OK;
 }
 

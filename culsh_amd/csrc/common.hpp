@@ -105,6 +105,8 @@ struct culsh_ctx {
     size_t arena_live = 0;               // bytes handed out and not rewound in this call (arena + overflow)
     size_t arena_want = 0;               // high-water mark of arena_live
     std::vector<void*> overflow;         // freed at the end of the call
+    uint64_t arena_overflow_blocks = 0;  // blocks that did not fit the arena, over the context's life
+    uint64_t arena_grow_failures = 0;    // grows of the arena that found no memory (the calls went on with overflow blocks)
     uint64_t* pinned = nullptr;          // 64 x u64 pinned host words for D2H scalars
     // pinned staging for hash parameters on their way to the device (grown on demand); calls end
     // with the stream idle, so a call may reuse it from the start
@@ -181,6 +183,12 @@ struct culsh_candidates {
 };
 
 namespace culsh_amd {
+
+// Calls into the HIP allocator made by this library in this process (hipMalloc, hipHostMalloc, hipFree,
+// hipEventCreate): what culsh_debug_allocation_calls reports, so that a test can tell that a call
+// allocated nothing.
+extern std::atomic<uint64_t> g_allocation_calls;
+inline void count_allocation_call() { g_allocation_calls.fetch_add(1, std::memory_order_relaxed); }
 
 // ---------------------------------------------------------------- object memory (pool.hip)
 // Device blocks owned by index / candidate objects; freed blocks are cached for reuse.

@@ -45,6 +45,7 @@ void evict(Pool& p, size_t keep) {
                 biggest = &kv.second;
         if (!biggest) break;
         auto it = std::prev(biggest->end());
+        count_allocation_call();
         (void)hipFree(it->second);
         p.cached_bytes -= it->first;
         biggest->erase(it);
@@ -73,10 +74,12 @@ hipError_t dev_malloc(void** out, size_t bytes) {
         p.cached_bytes -= sz;
         fl.erase(it);
     } else {
+        count_allocation_call();
         e = hipMalloc(out, sz);
         if (e != hipSuccess) {  // give the cache back and try once more
             (void)hipGetLastError();
             evict(p, 0);
+            count_allocation_call();
             e = hipMalloc(out, sz);
             if (e != hipSuccess) return e;
         }
@@ -91,12 +94,14 @@ void dev_free(void* ptr) {
     std::lock_guard<std::mutex> lock(p.mu);
     auto it = p.live.find(ptr);
     if (it == p.live.end()) {  // not from dev_malloc
+        count_allocation_call();
         (void)hipFree(ptr);
         return;
     }
     const Pool::Live meta = it->second;
     p.live.erase(it);
     if (meta.size > p.limit) {
+        count_allocation_call();
         (void)hipFree(ptr);
         return;
     }

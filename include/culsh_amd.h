@@ -175,8 +175,10 @@ culsh_status culsh_core_fit_index(culsh_ctx*, const void* X_sig_dev, int n_sampl
 culsh_status culsh_core_query_index(culsh_ctx*, const void* Q_sig_dev, int n_queries, int sig_nbytes, const culsh_index*, culsh_candidates** out);
 /* find_matching_buckets_kernel, core/query.cuh:72-101: int32 matched_dev[n_queries * T]. */
 culsh_status culsh_core_find_matching_buckets(culsh_ctx*, const void* Q_sig_dev, int n_queries, int sig_nbytes, const culsh_index*, int32_t* matched_dev);
-/* The same lookup for callers that cannot allocate (code under HIP graph capture, tight serving loops,
- * harnesses that forbid hipMalloc).  No counterpart in the reference.  The key words of the queries,
+/* The same lookup for callers that cannot allocate (tight serving loops, harnesses that forbid hipMalloc,
+ * code that must not allocate because a HIP graph is being captured elsewhere in the process; the call
+ * itself still sets the current device and checks the launch status, and has not been run on a capturing
+ * stream).  No counterpart in the reference.  The key words of the queries,
  * which culsh_core_find_matching_buckets keeps in the context's scratch arena, live in a workspace that
  * is part of the library's device image (CULSH_STATIC_SCRATCH_WORDS 32-bit words per GPU, held until the
  * process ends); the call makes no hipMalloc / hipFree, creates no events and does not wait for the
@@ -196,6 +198,14 @@ culsh_status culsh_core_fit_query(culsh_ctx*, const void* X_sig_dev, int n_sampl
 
 /* ---- index object ------------------------------------------------------------------------ */
 culsh_status culsh_index_get_meta(const culsh_index*, culsh_index_meta* out);
+/* Debugging aids (no counterpart in the reference).  culsh_debug_allocation_calls: how often this
+ * library has called the HIP allocator in this process (hipMalloc, hipHostMalloc, hipFree,
+ * hipEventCreate): unchanged across a call means the call allocated nothing.  culsh_debug_arena_state:
+ * out[0] = bytes of the context's scratch arena, out[1] = bytes of it in use, out[2] = scratch blocks
+ * that did not fit the arena so far, out[3] = grows of the arena that found no memory (such calls go on
+ * with separate blocks and the next call tries again). */
+uint64_t culsh_debug_allocation_calls(void);
+culsh_status culsh_debug_arena_state(const culsh_ctx*, uint64_t out[4]);
 /* Internal form of the lookup keys (no counterpart in the reference; for tests and tuning): 32-bit words
  * per bucket key, and how a signature becomes a key: 0 = its bytes, big-endian word by word, 1 = one bit per
  * RPLSH hash, 2 = p-stable hashes as ranks among the values seen at fit time, 3 = MinHash values as ranks

@@ -331,7 +331,7 @@ def test_core_query_wide_row_range(ctx, c_oracle, n):
 
 
 def test_core_query_output_sized_from_previous_call(ctx, monkeypatch):
-    """A second query call on an index sizes its output from the first call's raw candidates per query
+    """A second query call on an index sizes its output from the first call's distinct candidates per query
     and reads the true number back afterwards.  Calls whose queries bring fewer, as many, and far more
     candidates than the call before (the last overflows the guessed size and is redone), then forced
     guesses of one candidate per query and of more than the index holds, and a call without any match."""
@@ -350,6 +350,19 @@ def test_core_query_output_sized_from_previous_call(ctx, monkeypatch):
     none = np.full((T, 50, H), 200, np.uint8)
     for qsig in (few, few, many, few, none, few, many[:, :10], many):
         assert_candidates_match(ctx.core_query_index(qsig, ih), o.query_index(qsig, exp_ix))
+    # A second index of another shape, queried in turns with the first: the sizes are remembered per
+    # index shape, so each keeps its own (the first one's large-bucket queries must not size the
+    # second one's output, nor the other way round), and every call matches the oracle.
+    T2, n2 = 3, 7000
+    sig2 = rng.integers(0, 4, size=(T2, n2, H)).astype(np.uint8)          # ~440 rows per bucket
+    ih2, _ = ctx.core_fit_index(sig2, H)
+    exp_ix2 = o.fit_index(sig2, H)
+    q2 = rng.integers(0, 4, size=(T2, 200, H)).astype(np.uint8)
+    for _ in range(3):
+        assert_candidates_match(ctx.core_query_index(many, ih), o.query_index(many, exp_ix))
+        assert_candidates_match(ctx.core_query_index(q2, ih2), o.query_index(q2, exp_ix2))
+        assert_candidates_match(ctx.core_query_index(few, ih), o.query_index(few, exp_ix))
+    ctx.free_index(ih2)
     for forced in ("1", "100000000", "0"):
         monkeypatch.setenv("CULSH_QUERY_RAW_GUESS", forced)
         for qsig in (many, none, few):

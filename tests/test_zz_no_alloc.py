@@ -50,6 +50,53 @@ def test_static_lookup_matches_allocating_lookup(ctx, kind):
     ctx.free_index(ih)
 
 
+@pytest.mark.parametrize("kind", ["rplsh", "pslsh"])
+def test_static_lookup_allocates_nothing(ctx, kind):
+    """Around the static call nothing moves that an allocation would move: the library's count of calls
+    into the HIP allocator (hipMalloc, hipHostMalloc, hipFree, hipEventCreate), the context's scratch
+    arena (size, bytes in use, blocks beside it) and the device's free memory.  Also with per-kernel
+    timing switched on (the allocating lookup then takes events from a pool or creates them), and for
+    two calls issued back to back without a wait in between, followed by one culsh_ctx_synchronize."""
+    import ctypes as C
+
+    import torch
+
+    from abi import dev, ptr
+    from culsh_amd import _lib as L
+
+    print("[case] static lookup allocates nothing", kind, flush=True)
+    rng = np.random.default_rng(99)
+    T, n, H = 5, 3000, 3
+    sig = _sigs(rng, T, n, H, kind)
+    ih, _ = ctx.core_fit_index(sig, H)
+    exp_ix = o.fit_index(sig, H)
+    qa, qb = _sigs(rng, T, 400, H, kind), _sigs(rng, T, 150, H, kind)
+    qa[:, :200] = sig[:, rng.integers(0, n, 200)]
+    qb[:, :75] = sig[:, rng.integers(0, n, 75)]
+    S = qa.dtype.itemsize * H
+    da, db = dev(qa.view(np.uint8).reshape(-1)), dev(qb.view(np.uint8).reshape(-1))
+    ma = torch.empty(400 * T, dtype=torch.int32, device="cuda")
+    mb = torch.empty(150 * T, dtype=torch.int32, device="cuda")
+    torch.cuda.synchronize()
+
+    def state():
+        arena = (C.c_uint64 * 4)()
+        L.check(ctx.lib.culsh_debug_arena_state(ctx.h, arena))
+        return int(ctx.lib.culsh_debug_allocation_calls()), tuple(arena), torch.cuda.mem_get_info()[0]
+
+    for timing in (0, 1):
+        L.check(ctx.lib.culsh_profile_enable(ctx.h, timing))
+        before = state()
+        L.check(ctx.lib.culsh_core_find_matching_buckets_static(ctx.h, ptr(da), 400, S, ih, ptr(ma)))
+        L.check(ctx.lib.culsh_core_find_matching_buckets_static(ctx.h, ptr(db), 150, S, ih, ptr(mb)))   # no wait in between
+        ctx.synchronize()
+        assert state() == before
+        np.testing.assert_array_equal(ma.cpu().numpy(), o.find_matching_buckets(qa, exp_ix))
+        np.testing.assert_array_equal(mb.cpu().numpy(), o.find_matching_buckets(qb, exp_ix))
+    L.check(ctx.lib.culsh_profile_enable(ctx.h, 0))
+    ctx.free_index(ih)
+
+
 def test_static_lookup_after_family_fit(ctx):
     """An index whose keys are compressed ranks (p-stable fit): the static lookup converts query
     signatures with the index's tables, as the allocating one does."""
@@ -78,7 +125,7 @@ def test_static_lookup_refuses_sizes_beyond_the_workspace(ctx):
     from culsh_amd import _lib as L
 
     rng = np.random.default_rng(1)
-    T, n, H = 2, 100, 40                        # 40 sign bytes -> 2 key words per signature
+    T, n, H = 2, 100, 40                        # 40 opaque bytes -> 10 key words per signature
     sig = rng.integers(0, 2, size=(T, n, H), dtype=np.uint8)
     ih, _ = ctx.core_fit_index(sig, H)
     nq = (1 << 20) // (T * 10) + 1              # opaque byte keys: 10 words each
