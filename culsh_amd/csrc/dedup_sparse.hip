@@ -259,7 +259,8 @@ __global__ __launch_bounds__(DD_THREADS) void dedup_sparse_kernel(SparseDedupArg
             const uint32_t pw = ((m + NWAVES - 1u) / NWAVES + (SP_STEP - 1u)) & ~static_cast<uint32_t>(SP_STEP - 1);
             const int steps = static_cast<int>(pw / SP_STEP);  // <= SP_MAX_STEPS
             uint32_t blk[SP_MAX_STEPS][4], bits[SP_MAX_STEPS][4], c[SP_MAX_STEPS];
-            uint32_t wave_total = 0;
+            unsigned int ticket_next = 0;
+            if (last && tid == 0) ticket_next = atomicAdd(a.ticket, 1u);  // arrives while the rows are lined up
 #pragma unroll
             for (int j = 0; j < SP_MAX_STEPS; ++j) {
                 uint4 v0 = make_uint4(0u, 0u, 0u, 0u), v1 = make_uint4(0u, 0u, 0u, 0u);
@@ -271,26 +272,7 @@ __global__ __launch_bounds__(DD_THREADS) void dedup_sparse_kernel(SparseDedupArg
                 blk[j][0] = v0.x; bits[j][0] = v0.y; blk[j][1] = v0.z; bits[j][1] = v0.w;
                 blk[j][2] = v1.x; bits[j][2] = v1.y; blk[j][3] = v1.z; bits[j][3] = v1.w;
                 c[j] = __popc(bits[j][0]) + __popc(bits[j][1]) + __popc(bits[j][2]) + __popc(bits[j][3]);
-                wave_total += c[j];
             }
-            wave_total = wave_sum_dpp(wave_total);
-            if (lane == 0) wtot[wave] = wave_total;
-            unsigned int ticket_next = 0;
-            if (last && tid == 0) ticket_next = atomicAdd(a.ticket, 1u);  // arrives while the rows are lined up
-            __syncthreads();
-            uint32_t wave_base = 0, chunk_total = 0;
-#pragma unroll
-            for (int w = 0; w < NWAVES; ++w) {
-                const uint32_t v = wtot[w];
-                wave_base += (w < wave) ? v : 0u;
-                chunk_total += v;
-            }
-            wave_base = __builtin_amdgcn_readfirstlane(wave_base);
-            chunk_total = __builtin_amdgcn_readfirstlane(chunk_total);
-            if (n_pass == 1 && tid == 0)  // published before the line-up, so that later queries can go on
-                __hip_atomic_store(&a.state[q], TAG_COUNT | static_cast<unsigned long long>(chunk_total),
-                                   __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            SP_TICK(5)  // load, count, barrier
             // Line-up: a step's entries are in registers, which frees their place (two words per entry):
             // the rows are written there in list order, ready for full-width stores.  A step with more
             // rows than its place holds stays as it is.
@@ -314,14 +296,29 @@ __global__ __launch_bounds__(DD_THREADS) void dedup_sparse_kernel(SparseDedupArg
                     }
                 }
             }
+            if (lane == 0) wtot[wave] = st_total[0] + st_total[1] + st_total[2] + st_total[3];
             if (last && wave == 0) {
                 const int qn = min(static_cast<int>(__shfl(ticket_next, 0, 64)), a.n_queries);
                 if (T <= 64 && qn < a.n_queries && lane < T) sp_next = spans[static_cast<size_t>(qn) * T + lane];
                 if (lane == 0) *sh_q = qn;
             }
-            SP_TICK(6)  // line-up
+            SP_TICK(5)  // load, line-up
+            __syncthreads();  // all rows are lined up; the wavefronts' totals and *sh_q are in place
+            uint32_t wave_base = 0, chunk_total = 0;
+#pragma unroll
+            for (int w = 0; w < NWAVES; ++w) {
+                const uint32_t v = wtot[w];
+                wave_base += (w < wave) ? v : 0u;
+                chunk_total += v;
+            }
+            wave_base = __builtin_amdgcn_readfirstlane(wave_base);
+            chunk_total = __builtin_amdgcn_readfirstlane(chunk_total);
             if (n_pass == 1) {
-                // the list leaves after the next query's level-1 walk (or after the last query)
+                // The count is published now; the list leaves after the next query's level-1 walk (or after
+                // the last query), when the look-back finds the earlier queries' counts in place.
+                if (tid == 0)
+                    __hip_atomic_store(&a.state[q], TAG_COUNT | static_cast<unsigned long long>(chunk_total),
+                                       __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                 pending = true;
                 pend_q = q;
                 pend_pw = pw;
@@ -329,14 +326,13 @@ __global__ __launch_bounds__(DD_THREADS) void dedup_sparse_kernel(SparseDedupArg
                 pend_wave_base = wave_base;
 #pragma unroll
                 for (int j = 0; j < SP_MAX_STEPS; ++j) pend_step[j] = st_total[j];
-                __syncthreads();  // *sh_q is in place
             } else {
-                __syncthreads();  // all rows are lined up, *sh_q is in place
                 const unsigned long long base = *sh_base;
                 copy_out(pw, st_total, a.out + base + running + wave_base, base != ~0ull);
                 running += chunk_total;
                 __syncthreads();  // level 2 and wtot are rewritten by the next rank range / query
             }
+            SP_TICK(6)  // totals
             if (last) q_next = *sh_q;
         }
         if (q_next >= a.n_queries) break;

@@ -1111,7 +1111,7 @@ culsh_status query_from_spans(culsh_ctx* ctx, const int2* spans, const unsigned 
         uint64_t tk[8] = {0, 0, 0, 0, 0, 0, 0, 0};
         for (size_t i = 0; i < all.size(); ++i) tk[i & 7] += all[i];
         if (sparse_ok)
-            fprintf(stderr, "[two-level trace, if taken] set-up %llu level-1 %llu look-back+copy-out %llu rank %llu level-2 %llu count %llu line-up %llu tail %llu\n",
+            fprintf(stderr, "[two-level trace, if taken] set-up %llu level-1 %llu (unused) %llu rank+look-back+copy-out %llu level-2 %llu line-up %llu totals %llu tail %llu\n",
                     (unsigned long long)tk[0], (unsigned long long)tk[1], (unsigned long long)tk[2], (unsigned long long)tk[3],
                     (unsigned long long)tk[4], (unsigned long long)tk[5], (unsigned long long)tk[6], (unsigned long long)tk[7]);
         fprintf(stderr, "[dedup trace] wpt=%d chunks=%d fused=%d | setup %llu gather %llu count %llu store %llu (ticks) | popc %llu line-up %llu look-back %llu barrier %llu\n",
