@@ -9,7 +9,8 @@ namespace culsh_amd {
 
 constexpr int DD_THREADS = 1024;
 constexpr int NWAVES = DD_THREADS / 64;
-constexpr int WALK_U = 8;  // pieces in flight per wavefront
+constexpr int WALK_U = 16;   // pieces in flight per wavefront (walk_candidates)
+constexpr int STREAM_U = 8;  // pieces in flight per wavefront (stream_candidates)
 
 // Visits every row id of the query's spans.  The spans are cut into pieces of up to 64
 // consecutive ids (a piece never crosses a span boundary), pieces are dealt round-robin to
@@ -55,9 +56,9 @@ __device__ __forceinline__ void walk_candidates(const int32_t* __restrict__ cand
     }
 }
 
-// The same visit with loads that never drain: a wavefront keeps WALK_U pieces in flight and, as soon as
-// it has taken a piece's rows out of their register, fetches the piece WALK_U places further on into
-// it, so the walk costs one memory latency plus the work per piece instead of one latency per WALK_U
+// The same visit with loads that never drain: a wavefront keeps STREAM_U pieces in flight and, as soon as
+// it has taken a piece's rows out of their register, fetches the piece STREAM_U places further on into
+// it, so the walk costs one memory latency plus the work per piece instead of one latency per STREAM_U
 // pieces.  Lane l holds the table entry of the wavefront's l-th piece of the round (one LDS read per
 // round); a piece's start and length reach the scalar registers through v_readlane, so a load is a
 // scalar base plus the lane's fixed offset and costs no vector arithmetic.  Every load is issued
@@ -103,16 +104,18 @@ __device__ __forceinline__ void stream_candidates(const int32_t* __restrict__ ca
             const int32_t* piece = cand + static_cast<uint32_t>(__builtin_amdgcn_readlane(mine.x, k));
             return piece[lane];
         };
-        int rows[WALK_U];
+        int rows[STREAM_U];
 #pragma unroll
-        for (int u = 0; u < WALK_U; ++u) rows[u] = fetch(u);
-        for (int k0 = 0; k0 < nk; k0 += WALK_U) {
+        for (int u = 0; u < STREAM_U; ++u) rows[u] = fetch(u);
+        for (int k0 = 0; k0 < nk; k0 += STREAM_U) {
 #pragma unroll
-            for (int u = 0; u < WALK_U; ++u) {
-                const int row = rows[u];
+            for (int u = 0; u < STREAM_U; ++u) {
+                // the rows are used up before their register takes the next load: fetched into another
+                // register while these are still needed, they would have to be copied back at the end of
+                // every round of the loop, and the copies wait for all loads in flight
                 const int len = __builtin_amdgcn_readlane(mine.y, k0 + u);  // 0 beyond the wavefront's last piece
-                rows[u] = fetch((k0 + WALK_U + u) & 63);
-                if (lane < len) f(row);
+                if (lane < len) f(rows[u]);
+                rows[u] = fetch((k0 + STREAM_U + u) & 63);
             }
         }
         __syncthreads();  // tab is rewritten by the next round
