@@ -453,24 +453,40 @@ __global__ void shift_offsets_kernel(const uint64_t* __restrict__ src, uint64_t*
 
 // One pre-sized result instead of the reference's re-allocation per batch
 // (Candidates::merge, core/candidates.cuh:139-197); same contents.
+// `lists` (may be null): an array of `lists_cap` elements that already holds, at its final place, the lists of
+// the parts marked lists_in_place.  It becomes the result's array when everything fits; `*lists` is taken over
+// or freed here either way.
 static culsh_status concat_candidates(culsh_ctx* ctx, const std::vector<culsh_candidates*>& parts,
-                                      culsh_candidates* out) {
+                                      culsh_candidates* out, int32_t** lists = nullptr, uint64_t lists_cap = 0) {
     size_t nq = 0;
     uint64_t total = 0;
     for (auto* p : parts) { nq += p->n_queries; total += p->n_total_candidates; }
+    int32_t* placed = lists ? *lists : nullptr;  // owned here from now on
+    if (lists) *lists = nullptr;
+    struct Guard { int32_t* p; ~Guard() { dev_free(p); } } guard{placed};
     CULSH_REQUIRE(nq < (1ull << 31), CULSH_ERR_LIMIT, "too many queries");
     out->n_queries = static_cast<int>(nq);
     out->n_total_candidates = total;
     CULSH_HIP(dev_malloc(&out->query_candidate_counts, std::max<size_t>(1, nq) * sizeof(uint64_t)));
     CULSH_HIP(dev_malloc(&out->query_candidate_offsets, (nq + 1) * sizeof(uint64_t)));
-    if (total) CULSH_HIP(dev_malloc(&out->query_candidate_indices, total * sizeof(int32_t)));
+    const bool keep = placed && total > 0 && total <= lists_cap;  // the pre-filled array is the result's
+    if (keep) {
+        out->query_candidate_indices = placed;
+        guard.p = nullptr;
+    } else if (total) {
+        CULSH_HIP(dev_malloc(&out->query_candidate_indices, total * sizeof(int32_t)));
+    }
     size_t q0 = 0;
     uint64_t c0 = 0;
     CULSH_HIP(hipMemsetAsync(out->query_candidate_offsets, 0, sizeof(uint64_t), ctx->stream));
     for (auto* p : parts) {
-        if (p->n_total_candidates)
-            CULSH_HIP(hipMemcpyAsync(out->query_candidate_indices + c0, p->query_candidate_indices,
-                                     p->n_total_candidates * sizeof(int32_t), hipMemcpyDeviceToDevice, ctx->stream));
+        if (p->n_total_candidates) {
+            const int32_t* src = p->lists_in_place ? (placed ? placed + c0 : nullptr) : p->query_candidate_indices;
+            CULSH_REQUIRE(src, CULSH_ERR_INTERNAL, "a batch's candidate lists are missing");
+            if (!(keep && p->lists_in_place))
+                CULSH_HIP(hipMemcpyAsync(out->query_candidate_indices + c0, src, p->n_total_candidates * sizeof(int32_t),
+                                         hipMemcpyDeviceToDevice, ctx->stream));
+        }
         if (p->n_queries) {
             CULSH_HIP(hipMemcpyAsync(out->query_candidate_counts + q0, p->query_candidate_counts,
                                      p->n_queries * sizeof(uint64_t), hipMemcpyDeviceToDevice, ctx->stream));
@@ -483,13 +499,14 @@ static culsh_status concat_candidates(culsh_ctx* ctx, const std::vector<culsh_ca
         q0 += p->n_queries;
         c0 += p->n_total_candidates;
     }
+    if (guard.p) CULSH_HIP(hipStreamSynchronize(ctx->stream));  // copies out of the array that the guard frees
     return CULSH_OK;
 }
 
 // query over key words that are already in the arena
 static culsh_status query_keys(culsh_ctx* ctx, const uint32_t* q_keys, int nq, const culsh_index* ix,
-                               culsh_candidates* out) {
-    return query_from_keys(ctx, q_keys, nq, ix, out);
+                               culsh_candidates* out, int32_t* lists_dst = nullptr, uint64_t lists_cap = 0) {
+    return query_from_keys(ctx, q_keys, nq, ix, out, lists_dst, lists_cap);
 }
 
 template <typename T>
@@ -514,6 +531,13 @@ static culsh_status dense_query(culsh_ctx* ctx, Family fam, const T* Q, int nq, 
     const int d = ix->n_features, nT = ix->n_hash_tables, H = ix->n_hashes;
     if (batch_size <= 0 || batch_size >= nq) batch_size = nq;  // rplsh.cu:190-192
     std::vector<CandPtr> parts;
+    // The batches' lists go straight into one array, sized after the first batch by what it found per
+    // query (plus 15 %): the first batch's lists are copied there once, later batches write theirs behind
+    // what is there already; a batch that does not fit gets an array of its own and everything is put
+    // together at the end, as for the reference's merge.
+    struct Lists { int32_t* p = nullptr; ~Lists() { dev_free(p); } } lists;
+    uint64_t lists_cap = 0, lists_used = 0;
+    bool contiguous = true;  // all lists so far are (or can be put) in `lists` one behind the other
     for (int start = 0; start < nq; start += batch_size) {
         const int bn = std::min(batch_size, nq - start);
         const ArenaMark mark = arena_mark(ctx);
@@ -524,7 +548,27 @@ static culsh_status dense_query(culsh_ctx* ctx, Family fam, const T* Q, int nq, 
         CandPtr part(new (std::nothrow) culsh_candidates());
         CULSH_REQUIRE(part, CULSH_ERR_NOMEM, "host allocation failed");
         part->device = ctx->device;
-        CULSH_TRY(query_keys(ctx, keys, bn, ix, part.get()));
+        const bool room = lists.p && contiguous && lists_used < lists_cap;
+        CULSH_TRY(query_keys(ctx, keys, bn, ix, part.get(), room ? lists.p + lists_used : nullptr,
+                             room ? lists_cap - lists_used : 0));
+        const uint64_t found = part->n_total_candidates;
+        if (start == 0 && bn < nq && found > 0) {
+            const double per_query = static_cast<double>(found) / bn;
+            lists_cap = static_cast<uint64_t>(per_query * nq * 1.15) + 4096;
+            if (dev_malloc(&lists.p, lists_cap * sizeof(int32_t)) == hipSuccess) {
+                CULSH_HIP(hipMemcpyAsync(lists.p, part->query_candidate_indices, found * sizeof(int32_t),
+                                         hipMemcpyDeviceToDevice, ctx->stream));
+                part->lists_in_place = true;  // (it keeps its own array until the parts are freed)
+            } else {
+                (void)hipGetLastError();
+                lists.p = nullptr;
+                lists_cap = 0;
+            }
+        }
+        if (lists.p && contiguous) {
+            if (part->lists_in_place || found == 0) lists_used += found;
+            else contiguous = false;  // this batch's lists sit elsewhere: the ones behind it cannot be placed yet
+        }
         parts.push_back(std::move(part));
         arena_rewind(ctx, mark);  // the batch's query has ended with the stream idle
     }
@@ -538,7 +582,7 @@ static culsh_status dense_query(culsh_ctx* ctx, Family fam, const T* Q, int nq, 
     result->device = ctx->device;
     std::vector<culsh_candidates*> raw;
     for (auto& p : parts) raw.push_back(p.get());
-    CULSH_TRY(concat_candidates(ctx, raw, result.get()));
+    CULSH_TRY(concat_candidates(ctx, raw, result.get(), &lists.p, lists_cap));
     CULSH_TRY(arena_end(ctx));  // parts are freed after the copies have run
     *out = result.release();
     return CULSH_OK;

@@ -180,6 +180,9 @@ struct culsh_candidates {
     int n_queries = 0;
     uint64_t n_total_candidates = 0;
     int device = 0;
+    // Batched queries only (a batch's result before the batches are put together): the lists were
+    // written straight into the caller's array, or have been copied there already.
+    bool lists_in_place = false;
 };
 
 namespace culsh_amd {
@@ -371,8 +374,11 @@ culsh_status launch_find_matching_buckets(culsh_ctx* ctx, const uint32_t* q_keys
 culsh_status query_from_matched(culsh_ctx* ctx, const int32_t* matched, int n_queries,
                                 const culsh_index* index, culsh_candidates* out);
 // lookup + candidate retrieval from key words [T][n_queries][key_w]
+// `lists_dst` (may be null): `lists_cap` elements of the caller's own, into which the lists are written when
+// that can be done without a copy and they fit (out->lists_in_place says so; out->query_candidate_indices stays
+// null then); else the result gets an array of its own as always.
 culsh_status query_from_keys(culsh_ctx* ctx, const uint32_t* q_keys, int n_queries, const culsh_index* index,
-                             culsh_candidates* out);
+                             culsh_candidates* out, int32_t* lists_dst = nullptr, uint64_t lists_cap = 0);
 
 // Most hash tables an index may have (every fit, load and query checks it): the query kernels give each
 // table of a query one thread of a workgroup.

@@ -855,7 +855,8 @@ culsh_status alloc_query_words(culsh_ctx* ctx, int n_queries, const DedupGeometr
 // candidates = sum of all span lengths.  Debug knobs: CULSH_DEDUP_TWO_PASS=1 forces the
 // count / scan / emit path, CULSH_DEDUP_TRACE=1 prints phase timers.
 culsh_status query_from_spans(culsh_ctx* ctx, const int2* spans, const unsigned long long* raw_total, int n_queries,
-                              const culsh_index* index, const DedupGeometry& g, culsh_candidates* out) {
+                              const culsh_index* index, const DedupGeometry& g, culsh_candidates* out,
+                              int32_t* lists_dst = nullptr, uint64_t lists_cap = 0) {
     const int T = index->n_hash_tables;
     const int n = index->n_total_candidates / T;
     const int wpt = g.wpt, n_chunks = g.n_chunks;
@@ -933,6 +934,10 @@ culsh_status query_from_spans(culsh_ctx* ctx, const int2* spans, const unsigned 
         bool guessed = attempt == 0 && guess_raw > 0.0;
         Path path = guessed ? choose_path(guess_raw, guess_uniq) : P_FUSED;
         if (path == P_PASSES) guessed = false;  // lists at raw-count spacing: R sizes the output
+        // The caller's array takes the lists when the kernel packs them itself and the size need not be
+        // known first (the guessed mode: a batch behind the first one); a batch that does not fit is
+        // redone with an array of its own.
+        const bool in_place = guessed && lists_dst != nullptr && lists_cap > 0;
         unsigned long long* words = const_cast<unsigned long long*>(raw_total);
         uint64_t R = 0;
         if (attempt == 1) {  // the guess was too small: R is known by now, the kernel's words start from zero again
@@ -959,6 +964,7 @@ culsh_status query_from_spans(culsh_ctx* ctx, const int2* spans, const unsigned 
         // overlap heavily.  Several bitmap passes: list q starts at the sum of the raw counts of the
         // queries before it, and the gaps are closed below.
         const uint64_t cap = path == P_PASSES ? R
+                             : in_place ? lists_cap
                              : guessed ? std::min<uint64_t>(bound, static_cast<uint64_t>(guess_uniq * n_queries * 1.25) + 1024)
                                        : std::min<uint64_t>(R, bound);
         unsigned int* err = reinterpret_cast<unsigned int*>(words + 1);  // [0] error flags, [1] ticket counter
@@ -976,9 +982,12 @@ culsh_status query_from_spans(culsh_ctx* ctx, const int2* spans, const unsigned 
             a.raw_offsets = raw_offsets;
             a.state = nullptr;
         }
-        int32_t* lists = nullptr;
-        CULSH_HIP(dev_malloc(&lists, cap * sizeof(int32_t)));
-        out->query_candidate_indices = lists;  // owned by `out` from here on, also if a later step fails
+        int32_t* lists = lists_dst;
+        if (!in_place) {
+            lists = nullptr;
+            CULSH_HIP(dev_malloc(&lists, cap * sizeof(int32_t)));
+            out->query_candidate_indices = lists;  // owned by `out` from here on, also if a later step fails
+        }
         a.out = lists;
         a.err = err;
         a.capacity = cap;
@@ -1035,7 +1044,8 @@ culsh_status query_from_spans(culsh_ctx* ctx, const int2* spans, const unsigned 
             slot->key = shape;
             slot->raw_per_query = static_cast<double>(ctx->pinned[2]) / n_queries;
         }
-        if (guessed && e == 2u) {  // the guess was too small and nothing else went wrong: once more with R
+        if (in_place) lists = nullptr;  // not this function's to free
+        if (guessed && e == 2u) {  // the guess (or the caller's array) was too small and nothing else went wrong: once more with R
             dev_free(lists);
             out->query_candidate_indices = nullptr;
             guess_raw = 0.0;
@@ -1049,6 +1059,9 @@ culsh_status query_from_spans(culsh_ctx* ctx, const int2* spans, const unsigned 
             dev_free(lists);
             out->query_candidate_indices = nullptr;
             slot->uniq_per_query = 0.0;
+        } else if (in_place) {
+            slot->uniq_per_query = static_cast<double>(U) / n_queries;
+            out->lists_in_place = true;
         } else if (path == P_PASSES) {
             slot->uniq_per_query = static_cast<double>(U) / n_queries;
             int32_t* packed = nullptr;
@@ -1150,7 +1163,7 @@ culsh_status query_from_matched(culsh_ctx* ctx, const int32_t* matched, int n_qu
 }
 
 culsh_status query_from_keys(culsh_ctx* ctx, const uint32_t* q_keys, int n_queries, const culsh_index* index,
-                             culsh_candidates* out) {
+                             culsh_candidates* out, int32_t* lists_dst, uint64_t lists_cap) {
     CULSH_TRY(check_query_args(n_queries, index));
     int2* spans = nullptr;
     unsigned long long* raw_total = nullptr;
@@ -1159,7 +1172,7 @@ culsh_status query_from_keys(culsh_ctx* ctx, const uint32_t* q_keys, int n_queri
     CULSH_TRY(dedup_geometry(ctx, index, &g));
     CULSH_TRY(alloc_query_words(ctx, n_queries, g, &raw_total));
     CULSH_TRY(launch_find_matching_buckets(ctx, q_keys, n_queries, index, nullptr, spans, raw_total));
-    return query_from_spans(ctx, spans, raw_total, n_queries, index, g, out);
+    return query_from_spans(ctx, spans, raw_total, n_queries, index, g, out, lists_dst, lists_cap);
 }
 
 }  // namespace culsh_amd

@@ -768,6 +768,38 @@ def test_rplsh_fit_query_path(ctx, dtype, n, d, T, H, nq):
     ctx.free_index(ih2)
 
 
+@pytest.mark.parametrize("order", ["few_first", "many_first", "none_first"])
+def test_batched_query_lists_written_in_place(ctx, order):
+    """A batched query puts the batches' lists into one array that is sized after the first batch: later
+    batches write behind what is there.  Batches that find far more per query than the first one do not
+    fit and get arrays of their own (everything is put together at the end); a first batch that finds far
+    more leaves the array oversized; a first batch without any candidate leaves none.  All equal the
+    unbatched result, for several batch sizes (also one that does not divide the number of queries)."""
+    _announce("batched_in_place", order)
+    from abi import assert_candidates_match  # noqa: F401
+
+    rng = np.random.default_rng(321)
+    n, d, T, H = 6000, 24, 6, 10
+    X = rng.standard_normal((n, d)).astype(np.float32)
+    X[:2500] = X[0] + 1e-4 * rng.standard_normal((2500, d)).astype(np.float32)   # one crowd: 2500 rows per bucket
+    P = rng.standard_normal((T * H, d)).astype(np.float32)
+    lone = rng.standard_normal((60, d)).astype(np.float32)                        # few candidates each
+    crowd = np.repeat(X[:1], 90, axis=0) + 1e-4 * rng.standard_normal((90, d)).astype(np.float32)
+    far = np.full((40, d), 0.0, np.float32)
+    far[:, 0] = -1e6 * np.sign(P[:, 0].sum() + 1e-9)                              # (whatever it hashes to: a third kind)
+    Q = {"few_first": np.concatenate([lone, crowd, lone[:7]]),
+         "many_first": np.concatenate([crowd, lone, crowd[:5]]),
+         "none_first": np.concatenate([far, lone, crowd])}[order]
+    ih = ctx.rplsh_fit(X, T, H, seed=1, P=P)
+    want = ctx.rplsh_query(Q, ih)
+    assert want["n_total_candidates"] > 2500 * 50
+    for bs in (50, 37, 20):
+        got = ctx.rplsh_query(Q, ih, batch_size=bs)
+        for k in ("counts", "offsets", "indices"):
+            np.testing.assert_array_equal(got[k], want[k])
+    ctx.free_index(ih)
+
+
 def test_rplsh_seeded_projection_matches_generator(ctx):
     """fit without an injected P draws it from the seed with the documented generator."""
     rng = np.random.default_rng(2)
