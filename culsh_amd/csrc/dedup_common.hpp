@@ -68,6 +68,43 @@ __device__ __forceinline__ void walk_candidates(const int32_t* __restrict__ cand
 // longer count how many younger loads may stay in flight at a use and would wait for all of them.
 // `f` is called for the lanes that hold a row only (never with -1).
 // THREADS: size of the workgroup (a multiple of 64); `tab` holds THREADS entries.
+// The piece table of the round that starts at piece r0: fills `tab` and hands every lane the entry of the
+// wavefront's lane-th piece (length 0: no such piece).  One barrier inside; all threads must call it.
+// THREADS: size of the workgroup (a multiple of 64); `tab` holds THREADS entries.
+template <int THREADS>
+__device__ __forceinline__ int2 piece_table(const int* s_start, const int* s_len, const uint32_t* s_ppref, int T,
+                                            uint32_t n_pieces, uint32_t r0, int2* tab) {
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const uint32_t pc = r0 + static_cast<uint32_t>(tid);
+    if (pc < n_pieces) {
+        int tl = 0, th = T;  // largest t with s_ppref[t] <= pc; that span owns the piece
+        while (th - tl > 1) {
+            const int mid = (tl + th) >> 1;
+            if (s_ppref[mid] <= pc) tl = mid; else th = mid;
+        }
+        const int first = static_cast<int>(pc - s_ppref[tl]) * 64;
+        tab[tid] = make_int2(s_start[tl] + first, min(64, s_len[tl] - first));
+    }
+    __syncthreads();
+    const uint32_t here = min(static_cast<uint32_t>(THREADS), n_pieces - r0);
+    const uint32_t pi = static_cast<uint32_t>(wave + lane * (THREADS / 64));
+    return pi < here ? tab[pi] : make_int2(0, 0);
+}
+
+// pieces of this wavefront in the round that starts at piece r0 (at most 64)
+template <int THREADS>
+__device__ __forceinline__ int pieces_of_wave(uint32_t n_pieces, uint32_t r0) {
+    const int wave = __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x) >> 6);
+    const uint32_t here = n_pieces > r0 ? min(static_cast<uint32_t>(THREADS), n_pieces - r0) : 0u;
+    return here > static_cast<uint32_t>(wave) ? static_cast<int>((here - wave + THREADS / 64 - 1) / (THREADS / 64)) : 0;
+}
+
+// the rows of the wavefront's k-th piece (k < 64, the same in all lanes): one load per lane, unconditional
+__device__ __forceinline__ int stream_fetch(const int32_t* __restrict__ cand, const int2& mine, int k) {
+    const int32_t* piece = cand + static_cast<uint32_t>(__builtin_amdgcn_readlane(mine.x, k));
+    return piece[threadIdx.x & 63];
+}
+
 // `kept` (optional): the caller's copy of the wavefront's table entries.  A walk of a single round
 // (n_pieces <= THREADS) leaves them there, and a later walk over the same spans that is handed them
 // back skips the piece table and its barrier (`reuse` = true; the caller places a barrier between the

@@ -32,6 +32,9 @@ namespace {
 
 constexpr int SP_STEP = 256;      // level-2 entries a wavefront reads per step (four per lane)
 constexpr int SP_MAX_STEPS = 4;   // steps per wavefront and rank range; bounds `cap` to NWAVES * 4 * 256 entries
+#ifndef SP_REG
+#define SP_REG 40                 // pieces per wavefront of a query whose rows stay in registers (49152 rows per query)
+#endif
 
 __global__ __launch_bounds__(DD_THREADS) void dedup_sparse_kernel(SparseDedupArgs a) {
     extern __shared__ uint32_t lds[];
@@ -162,13 +165,41 @@ __global__ __launch_bounds__(DD_THREADS) void dedup_sparse_kernel(SparseDedupArg
         SP_TICK(0)  // set-up
 
         // Level 1: every candidate row marks its block.
-        int2 kept = make_int2(0, 0);  // this lane's piece table entry, for the second walk
-        const bool one_round = n_pieces <= static_cast<uint32_t>(DD_THREADS);
-        stream_candidates<DD_THREADS>(a.cand, s_start, s_len, s_ppref, T, n_pieces, tab, [&](int row) {
+        // A query of at most SP_REG pieces per wavefront keeps its rows in registers between the two
+        // levels, so that they are read from memory once: one piece table, every load in flight at once
+        // (in groups of eight that are skipped as a whole beyond the wavefront's last piece), and both
+        // levels are marked from the registers.  Lane l holds the table entry of the wavefront's l-th
+        // piece; a piece's start and length reach the scalar registers through v_readlane, and a load is
+        // a scalar base plus the lane's fixed offset (lanes beyond a piece's end read what follows it in
+        // `cand`, which has CAND_PAD readable elements behind its last one, and skip the marks).
+        auto mark_block = [&](int row) {
             const uint32_t blk = static_cast<uint32_t>(row) >> 5;
             atomicOr(&l1[blk >> 5].x, 1u << (blk & 31u));
-        }, &kept);
-        if (n_pieces == 0) __syncthreads();  // (no barrier inside the walk then)
+        };
+        const bool in_regs = n_pieces <= static_cast<uint32_t>(SP_REG * NWAVES);
+        const bool one_round = n_pieces <= static_cast<uint32_t>(DD_THREADS);
+        int2 kept = make_int2(0, 0);  // this lane's piece table entry
+        int rows[SP_REG];
+        const int nk = pieces_of_wave<DD_THREADS>(n_pieces, 0u);
+        if (in_regs) {
+            kept = piece_table<DD_THREADS>(s_start, s_len, s_ppref, T, n_pieces, 0u, tab);
+            // all loads unconditionally (a piece beyond the wavefront's last one reads the start of `cand`):
+            // behind branches the compiler could not tell how many younger loads may stay in flight when
+            // the first rows are marked, and would wait for nearly all of them
+#pragma unroll
+            for (int u = 0; u < SP_REG; ++u) rows[u] = stream_fetch(a.cand, kept, u);
+#pragma unroll
+            for (int u0 = 0; u0 < SP_REG; u0 += 8) {
+                if (u0 < nk) {
+#pragma unroll
+                    for (int u = u0; u < u0 + 8; ++u)
+                        if (lane < __builtin_amdgcn_readlane(kept.y, u)) mark_block(rows[u]);
+                }
+            }
+            __syncthreads();
+        } else {
+            stream_candidates<DD_THREADS>(a.cand, s_start, s_len, s_ppref, T, n_pieces, tab, mark_block, &kept);
+        }
         SP_TICK(1)  // level-1 marks
 
         // Rank: thread `tid` owns the level-1 words [tid * k1, tid * k1 + k1).  Under it the previous
@@ -206,17 +237,31 @@ __global__ __launch_bounds__(DD_THREADS) void dedup_sparse_kernel(SparseDedupArg
         // Level 2, rank range that starts at p0: a row finds its block's rank and sets its bit in the
         // block's entry; the same 64-bit OR leaves the block number there (every row of a block ORs
         // the same number into a word that was zero).
-        auto mark_rows = [&](uint32_t p0) {
-            stream_candidates<DD_THREADS>(a.cand, s_start, s_len, s_ppref, T, n_pieces, tab, [&](int row) {
-                const uint32_t blk = static_cast<uint32_t>(row) >> 5;
-                const uint2 e = l1[blk >> 5];
-                const uint32_t r = e.y + __popc(e.x & ((1u << (blk & 31u)) - 1u)) - p0;
-                if (r < cap)
-                    atomicOr(reinterpret_cast<unsigned long long*>(&pb[r]),
-                             (static_cast<unsigned long long>(1u << (static_cast<uint32_t>(row) & 31u)) << 32) | blk);
-            }, &kept, one_round);
+        auto mark_row = [&](int row, uint32_t p0) {
+            const uint32_t blk = static_cast<uint32_t>(row) >> 5;
+            const uint2 e = l1[blk >> 5];
+            const uint32_t r = e.y + __popc(e.x & ((1u << (blk & 31u)) - 1u)) - p0;
+            if (r < cap)
+                atomicOr(reinterpret_cast<unsigned long long*>(&pb[r]),
+                         (static_cast<unsigned long long>(1u << (static_cast<uint32_t>(row) & 31u)) << 32) | blk);
+        };
+        auto mark_rows = [&](uint32_t p0) {  // a walk over the rows in memory; ends with a barrier
+            stream_candidates<DD_THREADS>(a.cand, s_start, s_len, s_ppref, T, n_pieces, tab,
+                                          [&](int row) { mark_row(row, p0); }, &kept, one_round);
             if (n_pieces == 0) __syncthreads();
         };
+        const bool from_regs = in_regs && n_pass == 1;
+        if (from_regs) {  // the rows in registers are used up here, before the read-out needs the registers
+#pragma unroll
+            for (int u0 = 0; u0 < SP_REG; u0 += 8) {
+                if (u0 < nk) {
+#pragma unroll
+                    for (int u = u0; u < u0 + 8; ++u)
+                        if (lane < __builtin_amdgcn_readlane(kept.y, u)) mark_row(rows[u], 0u);
+                }
+            }
+            __syncthreads();
+        }
 
         unsigned long long total = 0;
         if (n_pass > 1) {
@@ -249,7 +294,7 @@ __global__ __launch_bounds__(DD_THREADS) void dedup_sparse_kernel(SparseDedupArg
         for (uint32_t p = 0; p < n_pass; ++p) {
             const uint32_t p0 = p * cap, m = min(cap, n_blocks - p0);
             const bool last = p == n_pass - 1u;
-            mark_rows(p0);
+            if (!from_regs) mark_rows(p0);
             SP_TICK(4)  // level-2 marks
             if (last)  // level 1 is clean for the next query; nobody reads it during the read-out
                 for (int j = 0; j < k1; ++j) l1[tid * k1 + j] = make_uint2(0u, 0u);
@@ -258,37 +303,33 @@ __global__ __launch_bounds__(DD_THREADS) void dedup_sparse_kernel(SparseDedupArg
             // every lane takes four consecutive entries: list order = (wavefront, step, lane, entry, bit).
             const uint32_t pw = ((m + NWAVES - 1u) / NWAVES + (SP_STEP - 1u)) & ~static_cast<uint32_t>(SP_STEP - 1);
             const int steps = static_cast<int>(pw / SP_STEP);  // <= SP_MAX_STEPS
-            uint32_t blk[SP_MAX_STEPS][4], bits[SP_MAX_STEPS][4], c[SP_MAX_STEPS];
             unsigned int ticket_next = 0;
             if (last && tid == 0) ticket_next = atomicAdd(a.ticket, 1u);  // arrives while the rows are lined up
-#pragma unroll
-            for (int j = 0; j < SP_MAX_STEPS; ++j) {
-                uint4 v0 = make_uint4(0u, 0u, 0u, 0u), v1 = make_uint4(0u, 0u, 0u, 0u);
-                const uint32_t i0 = static_cast<uint32_t>(wave) * pw + static_cast<uint32_t>(j * SP_STEP + lane * 4);
-                if (j < steps && i0 < cap) {  // entries behind the range hold no bits
-                    v0 = *reinterpret_cast<const uint4*>(pb + i0);
-                    v1 = *reinterpret_cast<const uint4*>(pb + i0 + 2);
-                }
-                blk[j][0] = v0.x; bits[j][0] = v0.y; blk[j][1] = v0.z; bits[j][1] = v0.w;
-                blk[j][2] = v1.x; bits[j][2] = v1.y; blk[j][3] = v1.z; bits[j][3] = v1.w;
-                c[j] = __popc(bits[j][0]) + __popc(bits[j][1]) + __popc(bits[j][2]) + __popc(bits[j][3]);
-            }
-            // Line-up: a step's entries are in registers, which frees their place (two words per entry):
-            // the rows are written there in list order, ready for full-width stores.  A step with more
-            // rows than its place holds stays as it is.
+            // Line-up, step by step: a step's entries go to registers, which frees their place (two words
+            // per entry): the rows are written there in list order, ready for full-width stores.  A step
+            // with more rows than its place holds stays as it is.
             uint32_t st_total[SP_MAX_STEPS];
 #pragma unroll
             for (int j = 0; j < SP_MAX_STEPS; ++j) {
                 st_total[j] = 0u;
                 if (j >= steps) continue;
-                const uint32_t incl = wave_inclusive_sum_dpp(c[j]);
+                uint4 v0 = make_uint4(0u, 0u, 0u, 0u), v1 = make_uint4(0u, 0u, 0u, 0u);
+                const uint32_t i0 = static_cast<uint32_t>(wave) * pw + static_cast<uint32_t>(j * SP_STEP + lane * 4);
+                if (i0 < cap) {  // entries behind the range hold no bits
+                    v0 = *reinterpret_cast<const uint4*>(pb + i0);
+                    v1 = *reinterpret_cast<const uint4*>(pb + i0 + 2);
+                }
+                const uint32_t blk[4] = {v0.x, v0.z, v1.x, v1.z}, bits[4] = {v0.y, v0.w, v1.y, v1.w};
+                const uint32_t c = __popc(bits[0]) + __popc(bits[1]) + __popc(bits[2]) + __popc(bits[3]);
+                const uint32_t incl = wave_inclusive_sum_dpp(c);
                 st_total[j] = __shfl(incl, 63, 64);
                 if (st_total[j] <= step_room(pw, j)) {
-                    uint32_t* slot = reinterpret_cast<uint32_t*>(pb + static_cast<uint32_t>(wave) * pw + j * SP_STEP) + (incl - c[j]);
+                    __builtin_amdgcn_wave_barrier();  // every lane has its entries before the first row lands on them
+                    uint32_t* slot = reinterpret_cast<uint32_t*>(pb + static_cast<uint32_t>(wave) * pw + j * SP_STEP) + (incl - c);
 #pragma unroll
                     for (int k = 0; k < 4; ++k) {
-                        uint32_t left = bits[j][k];
-                        const uint32_t r0 = blk[j][k] << 5;
+                        uint32_t left = bits[k];
+                        const uint32_t r0 = blk[k] << 5;
                         while (left) {
                             *slot++ = r0 + static_cast<uint32_t>(__ffs(static_cast<int>(left)) - 1);
                             left &= left - 1u;
