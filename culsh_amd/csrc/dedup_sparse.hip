@@ -213,6 +213,7 @@ __global__ __launch_bounds__(DD_THREADS) void dedup_sparse_kernel(SparseDedupArg
             if (lane == 63) scratch[wave] = incl;
             if (pending && wave == 0) place_list(pend_q, pend_total);
             __syncthreads();
+            SP_TICK(2)  // block count and look-back of the previous query
 #pragma unroll
             for (int w = 0; w < NWAVES; ++w) {
                 const uint32_t v = scratch[w];

@@ -893,7 +893,9 @@ culsh_status query_from_spans(culsh_ctx* ctx, const int2* spans, const unsigned 
     bool fused = env_int("CULSH_DEDUP_TWO_PASS", 0) == 0;
     const bool several = n_chunks > 1;
     uint64_t U = 0;
-    // Which kernel.  Row ranges of one bitmap pass: the bitmap kernel.  Larger ones: the two-level
+    // Which kernel.  Row ranges of one bitmap pass: the bitmap kernel, unless the queries hold next to
+    // nothing (fewer than one raw candidate per 2048 rows: the sweep over the bitmap is then most of a
+    // query's time, and the two-level kernel sweeps a 32nd of it).  Larger ranges: the two-level
     // kernel (dedup_sparse.hip) when its level 1 fits and a query's distinct rows are expected to fit
     // its level 2, else the bitmap kernel with several passes per query.
     // CULSH_DEDUP_SPARSE (tests, tuning): 0 = never, 1 = whenever the geometry allows; CULSH_DEDUP_SPARSE_CAP
@@ -904,7 +906,7 @@ culsh_status query_from_spans(culsh_ctx* ctx, const int2* spans, const unsigned 
     const bool sparse_ok = sparse_knob != 0 && sparse_dedup_geometry(ctx, n, T, env_int("CULSH_DEDUP_SPARSE_CAP", 0), &sg);
     auto choose_path = [&](double raw_per_query, double uniq_per_query) {  // uniq_per_query < 0: not known
         if (sparse_ok && sparse_knob == 1) return P_SPARSE;
-        if (!several) return P_FUSED;
+        if (!several) return sparse_ok && sparse_knob != 0 && raw_per_query * 2048.0 <= static_cast<double>(n) ? P_SPARSE : P_FUSED;
         if (!sparse_ok) return P_PASSES;
         const bool fits = uniq_per_query >= 0.0 ? uniq_per_query <= 0.9 * sg.cap : raw_per_query <= 4.0 * sg.cap;
         return fits ? P_SPARSE : P_PASSES;
@@ -1124,7 +1126,7 @@ culsh_status query_from_spans(culsh_ctx* ctx, const int2* spans, const unsigned 
         uint64_t tk[8] = {0, 0, 0, 0, 0, 0, 0, 0};
         for (size_t i = 0; i < all.size(); ++i) tk[i & 7] += all[i];
         if (sparse_ok)
-            fprintf(stderr, "[two-level trace, if taken] set-up %llu level-1 %llu (unused) %llu rank+look-back+copy-out %llu level-2 %llu line-up %llu totals %llu tail %llu\n",
+            fprintf(stderr, "[two-level trace, if taken] set-up %llu level-1 %llu look-back %llu rank+copy-out %llu level-2 %llu line-up %llu totals %llu tail %llu\n",
                     (unsigned long long)tk[0], (unsigned long long)tk[1], (unsigned long long)tk[2], (unsigned long long)tk[3],
                     (unsigned long long)tk[4], (unsigned long long)tk[5], (unsigned long long)tk[6], (unsigned long long)tk[7]);
         fprintf(stderr, "[dedup trace] wpt=%d chunks=%d fused=%d | setup %llu gather %llu count %llu store %llu (ticks) | popc %llu line-up %llu look-back %llu barrier %llu\n",
