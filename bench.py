@@ -188,6 +188,9 @@ def other_configs(ctx, with_cpu: bool):
     sc_ms, sc_launches = _sum_ms(table_fit, "radix_scatter_kernel")
     roofs = [_roof("project_f32_kernel (fit launch)", "mfma", 2.0 * n * d * T * H, proj_ms, 1e12, PEAK_FP32_MFMA_TFLOPS,
                    "TFLOP/s", "2*n*d*T*H flop"),
+             # the same launch against the other roofline: it writes 4 bytes per hash, as many bytes as it reads
+             _roof("project_f32_kernel (fit launch)", "hbm", 4.0 * n * d + 4.0 * n * T * H, proj_ms, 1e9, PEAK_HBM_GBS,
+                   "GB/s", "X read once, one int32 hash per row, table and hash function written"),
              _roof("radix_scatter_kernel (all passes)", "hbm", _scatter_bytes(sc_launches, W, N), sc_ms, 1e9, PEAK_HBM_GBS,
                    "GB/s", f"{sc_launches} passes over {N} items of {W} key words and a row id")]
     parity = None
