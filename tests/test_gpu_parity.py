@@ -541,6 +541,57 @@ def test_core_query_two_level_bitmap_shapes(ctx, c_oracle, monkeypatch, T, n, nq
     ctx.free_index(ih)
 
 
+def _kernels_run(ctx, fn):
+    """Names of the library's kernels that `fn` launches (per-kernel event timing switched on around it)."""
+    import ctypes as C
+
+    from culsh_amd import _lib as L
+
+    L.check(ctx.lib.culsh_profile_enable(ctx.h, 1))
+    L.check(ctx.lib.culsh_profile_reset(ctx.h))
+    try:
+        result = fn()
+        names = set()
+        for i in range(ctx.lib.culsh_profile_count(ctx.h)):
+            name, ms, cnt = C.c_char_p(), C.c_double(), C.c_int64()
+            L.check(ctx.lib.culsh_profile_get(ctx.h, i, C.byref(name), C.byref(ms), C.byref(cnt)))
+            if cnt.value:
+                names.add(name.value.decode())
+    finally:
+        L.check(ctx.lib.culsh_profile_enable(ctx.h, 0))
+    return result, names
+
+
+def test_core_query_with_next_to_no_candidates_takes_the_two_level_kernel(ctx, c_oracle):
+    """Inside one bitmap pass the two-level kernel is chosen, unforced, when the queries bring fewer than
+    one raw candidate per 2048 rows (sweeping the bitmap would be most of such a query's time); the same
+    index queried with rows of a large bucket goes back to the bitmap kernel.  Both against the oracle."""
+    _announce("few_candidates_two_level")
+    rng = np.random.default_rng(77)
+    T, n, nq, H = 4, 200_000, 500, 3
+    sig = rng.integers(0, 40, size=(T, n, H)).astype(np.uint8)              # ~3 rows per bucket
+    sig[:, : n // 4, :] = 90                                                # and one bucket of 50,000 rows
+    qsig = rng.integers(0, 40, size=(T, nq, H)).astype(np.uint8)
+    qsig[:, ::5, :] = 200                                                   # no candidates
+    ih, _ = ctx.core_fit_index(sig, H)
+    from abi import assert_candidates_match
+
+    cix = c_oracle.fit_index_c(sig, H)
+    exp = c_oracle.query_index_c(qsig, cix)
+    for _ in range(2):                                                      # second call: path chosen from the first call's figures
+        got, names = _kernels_run(ctx, lambda: ctx.core_query_index(qsig, ih))
+        assert_candidates_match(got, exp)
+        assert "dedup_sparse_kernel" in names and not any(k.startswith("dedup_kernel") for k in names), names
+    heavy = qsig.copy()
+    heavy[:, ::2, :] = 90
+    exp_heavy = c_oracle.query_index_c(heavy, cix)
+    assert_candidates_match(ctx.core_query_index(heavy, ih), exp_heavy)     # outgrows what the earlier calls suggest: redone
+    got, names = _kernels_run(ctx, lambda: ctx.core_query_index(heavy, ih))
+    assert_candidates_match(got, exp_heavy)
+    assert "dedup_sparse_kernel" not in names, names
+    ctx.free_index(ih)
+
+
 def test_core_query_two_level_bitmap_look_back_gives_up(ctx, monkeypatch):
     """The two-level kernel with no polls allowed in its chained scan: the call is redone with the
     count / scan / emit launches."""
