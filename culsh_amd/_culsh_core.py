@@ -322,8 +322,27 @@ class PSLSHIndex(_DenseIndex):
                                       n_total_buckets, n_hash_tables, n_hashes, sig_nbytes, n_features, seed)
 
 
+MINHASH_PRIMES = (4294967291, 2147483647)  # the reference's 2^32 - 5 (minhash/hash.cuh:17) and 2^31 - 1
+
+
+def _check_prime(prime) -> Optional[int]:
+    if prime is None:
+        return None
+    if int(prime) not in MINHASH_PRIMES:
+        raise ValueError(f"prime must be one of {MINHASH_PRIMES}, got {prime}")
+    return int(prime)
+
+
 class MinHashIndex(_IndexBase):
     _KIND = L.KIND_MINHASH
+
+    @property
+    def prime(self) -> int:
+        """The prime the index's hash family is taken modulo (not part of the reference's index, whose
+        prime is fixed, minhash/hash.cuh:17)."""
+        v = C.c_uint32()
+        L.check(self._ctx._lib.culsh_index_minhash_prime(self._h, C.byref(v)))
+        return int(v.value)
 
     def get_hash_a(self) -> np.ndarray:
         return self._array(L.ARR_HASH_A, np.uint32)
@@ -334,14 +353,21 @@ class MinHashIndex(_IndexBase):
     @staticmethod
     def load(candidate_indices, bucket_signatures, bucket_candidate_offsets, table_bucket_offsets, hash_a, hash_b,
              n_total_candidates, n_total_buckets, n_hash_tables, n_hashes, sig_nbytes, n_features,
-             seed) -> "MinHashIndex":
+             seed, prime=None) -> "MinHashIndex":
+        """`prime` (an addition to bindings.cu:457-476): the prime the saved index was hashed with; None is the
+        reference's."""
         a = np.ascontiguousarray(hash_a, dtype=np.uint32).reshape(-1)
         b = np.ascontiguousarray(hash_b, dtype=np.uint32).reshape(-1)
         if a.size != n_hash_tables * n_hashes or b.size != a.size:
             raise RuntimeError("hash_a / hash_b do not match the index metadata")
-        return MinHashIndex._load(False, candidate_indices, bucket_signatures, bucket_candidate_offsets,
-                                  table_bucket_offsets, a, b, n_total_candidates, n_total_buckets, n_hash_tables,
-                                  n_hashes, sig_nbytes, n_features, seed)
+        ctx = _Ctx.default()  # the context the load below runs on: it hands its prime to the index
+        L.check(ctx._lib.culsh_ctx_set_minhash_prime(ctx.handle, _check_prime(prime) or MINHASH_PRIMES[0]))
+        try:
+            return MinHashIndex._load(False, candidate_indices, bucket_signatures, bucket_candidate_offsets,
+                                      table_bucket_offsets, a, b, n_total_candidates, n_total_buckets, n_hash_tables,
+                                      n_hashes, sig_nbytes, n_features, seed)
+        finally:
+            L.check(ctx._lib.culsh_ctx_set_minhash_prime(ctx.handle, MINHASH_PRIMES[0]))
 
 
 # --------------------------------------------------------------------------------------
@@ -442,7 +468,15 @@ class PSLSHCore(_DenseCore):
 
 
 class MinHashCore(_CoreBase):
-    """bindings.cu:118-168"""
+    """bindings.cu:118-168.  `prime` is an addition: the prime of the hash family, None = the reference's
+    4294967291 (minhash/hash.cuh:17)."""
+
+    def __init__(self, n_hash_tables: int, n_hashes: int, seed: int = 42, prime=None):
+        super().__init__(n_hash_tables, n_hashes, seed)
+        self._prime = _check_prime(prime) or MINHASH_PRIMES[0]
+        L.check(self._lib.culsh_ctx_set_minhash_prime(self._ctx.handle, self._prime))
+
+    prime = property(lambda self: self._prime)
 
     def _fit(self, indices, indptr, n_samples, n_features, hash_a, hash_b, query: bool):
         th = self._n_hash_tables * self._n_hashes

@@ -112,12 +112,18 @@ class LSHEstimator:
         settings then reuses the core's stream, scratch memory and seeded hash parameters (the
         reference builds a new core per fit, python/culsh/rp_lsh.py:119-121; the result is the same)."""
         hyper = self._hyper_values(rows)
-        key = (self._n_hash_tables, self._n_hashes, tuple(hyper[k] for k in self._family.hyper), self._seed)
+        extra = self._core_kwargs()
+        key = (self._n_hash_tables, self._n_hashes, tuple(hyper[k] for k in self._family.hyper), self._seed,
+               tuple(sorted(extra.items())))
         kept = getattr(self, "_kept_core", None)
         if kept is None or kept[0] != key:
-            kept = (key, self._family.core_cls(self._n_hash_tables, self._n_hashes, *key[2], self._seed))
+            kept = (key, self._family.core_cls(self._n_hash_tables, self._n_hashes, *key[2], self._seed, **extra))
             self._kept_core = kept
         return kept[1], hyper
+
+    def _core_kwargs(self) -> dict:
+        """Keyword arguments of the family's core beyond the reference's (none by default)."""
+        return {}
 
     def _fit(self, X):
         rows = _Rows(X, self._family.dense)
@@ -171,7 +177,18 @@ class LSHModel:
             fields["is_double"] = ix.is_double
         fields.update((k, getattr(ix, getter)()) for k, getter in _INDEX_ARRAYS.items())
         fields.update((k, getattr(ix, getter)()) for k, getter in fam.param_arrays)
+        fields.update(self._extra_fields())
         np.savez_compressed(path, **fields)
+
+    def _extra_fields(self) -> dict:
+        """Keys beyond the reference's that this model has to write to be read back as it is (none by
+        default, so that default files hold exactly the reference's keys)."""
+        return {}
+
+    @classmethod
+    def _extra_kwargs(cls, data) -> dict:
+        """Keyword arguments for the core and the index loader from such keys."""
+        return {}
 
     @classmethod
     def load(cls, path: str):
@@ -180,7 +197,8 @@ class LSHModel:
         data = np.load(path)
         ints = {k: int(data[k]) for k in ("n_hash_tables", "n_hashes", "n_features", "seed", *fam.hyper)}
         hyper = {k: ints[k] for k in fam.hyper}
-        core = fam.core_cls(ints["n_hash_tables"], ints["n_hashes"], *hyper.values(), ints["seed"])
+        extra = cls._extra_kwargs(data)
+        core = fam.core_cls(ints["n_hash_tables"], ints["n_hashes"], *hyper.values(), ints["seed"], **extra)
         if fam.dense:
             loader = fam.index_cls.load_double if data["is_double"] else fam.index_cls.load_float
         else:
@@ -188,6 +206,6 @@ class LSHModel:
         arrays = {k: data[k] for k in (*_INDEX_ARRAYS, *(k for k, _ in fam.param_arrays))}
         index = loader(**arrays, **{k: int(data[k]) for k in _INDEX_SCALARS},
                        n_hash_tables=ints["n_hash_tables"], n_hashes=ints["n_hashes"],
-                       n_features=ints["n_features"], seed=ints["seed"])
+                       n_features=ints["n_features"], seed=ints["seed"], **extra)
         return cls(n_hash_tables=ints["n_hash_tables"], n_hashes=ints["n_hashes"], **hyper,
                    n_features=ints["n_features"], core=core, index=index)

@@ -68,6 +68,10 @@ PROTOTYPES = {
     "culsh_generate_pslsh_params_f32": [_U64, _I, _I, _I, _P, _P],
     "culsh_generate_pslsh_params_f64": [_U64, _I, _I, _I, _P, _P],
     "culsh_generate_minhash_params": [_U64, _I, _P, _P],
+    "culsh_generate_minhash_params_mod": [_U64, _I, C.c_uint32, _P, _P],
+    "culsh_ctx_set_minhash_prime": [_P, C.c_uint32],
+    "culsh_ctx_get_minhash_prime": [_P, C.POINTER(C.c_uint32)],
+    "culsh_index_minhash_prime": [_P, C.POINTER(C.c_uint32)],
     "culsh_rplsh_fit_f32": [_P, _P, _I, _I, _I, _I, _U64, _P, _PP],
     "culsh_rplsh_fit_f64": [_P, _P, _I, _I, _I, _I, _U64, _P, _PP],
     "culsh_rplsh_query_f32": [_P, _P, _I, _P, _I, _PP],

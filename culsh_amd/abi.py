@@ -55,6 +55,15 @@ class Ctx:
     def __del__(self):
         self.close()
 
+    def set_minhash_prime(self, prime: int) -> None:
+        """The prime MinHash fits, loads and `minhash_compute` calls of this context hash with from now on."""
+        L.check(self.lib.culsh_ctx_set_minhash_prime(self.h, prime))
+
+    def index_minhash_prime(self, ih) -> int:
+        v = C.c_uint32()
+        L.check(self.lib.culsh_index_minhash_prime(ih, C.byref(v)))
+        return int(v.value)
+
     # ------------------------------------------------------------ objects
     def index_arrays(self, ih):
         """dict with the four core arrays + metadata of an index handle."""

@@ -224,7 +224,8 @@ def make_estimator(w: Workload, args):
         ws = args.window_size if args.window_size is not None else w.window_size
         ws = "auto" if ws in (None, 0) else ws
         return PStableLSH(n_hash_tables=T, n_hashes=H, window_size=ws, seed=args.seed), {"window_size": ws}
-    return MinHashLSH(n_hash_tables=T, n_hashes=H, seed=args.seed), {}
+    est = MinHashLSH(n_hash_tables=T, n_hashes=H, seed=args.seed, prime=args.prime)
+    return est, {"prime": est.prime}  # every report names the prime (the reference's unless --prime says otherwise)
 
 
 def run(args) -> dict:
@@ -298,6 +299,8 @@ def main(argv=None) -> int:
     ap.add_argument("-nh", "--n-hashes", type=int, default=None)
     ap.add_argument("-w", "--window-size", type=int, default=None, help="p-stable window (0 = 'auto')")
     ap.add_argument("-s", "--seed", type=int, default=42, help="seed of the hash parameters")
+    ap.add_argument("--prime", type=int, default=None,
+                    help="MinHash: prime of the hash family, 4294967291 (default, the reference's) or 2147483647")
     ap.add_argument("--data-seed", type=int, default=1234)
     ap.add_argument("-nq", "--n-queries", type=int, default=None)
     ap.add_argument("-ne", "--n-eval-queries", type=int, default=10)

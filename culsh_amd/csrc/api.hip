@@ -12,6 +12,7 @@
 #include <vector>
 
 #include "common.hpp"
+#include "mh_prime.hpp"
 
 namespace culsh_amd {
 
@@ -274,8 +275,8 @@ static void gen_bias(uint64_t seed, size_t count, T* b) {  // uniform in (0,1], 
         b[i] = static_cast<T>(static_cast<double>((r[i] >> 11) + 1) * (1.0 / 9007199254740992.0));
 }
 
-static void gen_minhash(uint64_t seed, size_t count, uint32_t* A, uint32_t* B) {
-    const uint64_t p = 4294967291ull;  // minhash/hash.cuh:17
+static void gen_minhash(uint64_t seed, size_t count, uint32_t* A, uint32_t* B, int prime_kind = MH_PRIME_2_32_M5) {
+    const uint64_t p = mh_prime_value(prime_kind);  // the reference's: minhash/hash.cuh:17
     std::vector<uint64_t> r(count);
     gen_raw_u64(seed, STREAM_HASH_A, count, r.data());
     for (size_t i = 0; i < count; ++i) A[i] = static_cast<uint32_t>(((r[i] >> 32) % (p - 1)) + 1);  // :27-28
@@ -687,17 +688,19 @@ static culsh_status minhash_fit_once(culsh_ctx* ctx, const int32_t* indices, con
     CULSH_REQUIRE(ix, CULSH_ERR_NOMEM, "host allocation failed");
     ix->device = ctx->device;
     ix->kind = CULSH_KIND_MINHASH;
+    ix->mh_prime_kind = ctx->mh_prime_kind;
     const size_t TH = static_cast<size_t>(nT) * H;
     {
         ctx->param_stage_off = 0;
         if (!A_host) {
             culsh_ctx::GenCache& gc = ctx->gen_cache;
-            constexpr int FAM_MINHASH_TAG = 100;
+            const int FAM_MINHASH_TAG = 100 + ctx->mh_prime_kind;
             if (!(gc.family == FAM_MINHASH_TAG && gc.seed == seed && gc.rows == TH)) {
                 gc.family = -1;
                 gc.p.resize(TH * sizeof(uint32_t));
                 gc.b.resize(TH * sizeof(uint32_t));
-                gen_minhash(seed, TH, reinterpret_cast<uint32_t*>(gc.p.data()), reinterpret_cast<uint32_t*>(gc.b.data()));
+                gen_minhash(seed, TH, reinterpret_cast<uint32_t*>(gc.p.data()), reinterpret_cast<uint32_t*>(gc.b.data()),
+                            ctx->mh_prime_kind);
                 gc.family = FAM_MINHASH_TAG;
                 gc.seed = seed;
                 gc.rows = TH;
@@ -726,7 +729,7 @@ static culsh_status minhash_fit_once(culsh_ctx* ctx, const int32_t* indices, con
         CULSH_TRY(launch_minhash_rank(ctx, indices, indptr, n, nT, H, ix.get(), ctx->aux_flag_dev, keys));
     } else {
         CULSH_TRY(arena_alloc_t(ctx, N * H, &keys));
-        CULSH_TRY(launch_minhash(ctx, indices, indptr, ix->A, ix->B, n, nT, H, true, keys));
+        CULSH_TRY(launch_minhash(ctx, indices, indptr, ix->A, ix->B, n, nT, H, true, keys, ix->mh_prime_kind));
     }
     CandPtr cands;
     if (cands_out) {
@@ -973,6 +976,36 @@ culsh_status culsh_generate_minhash_params(uint64_t seed, int n_rows, uint32_t* 
     gen_minhash(seed, n_rows, A, B);
     return CULSH_OK;
 }
+static bool prime_kind_of(uint32_t prime, int* kind) {
+    if (prime == mh_prime_value(MH_PRIME_2_32_M5)) { *kind = MH_PRIME_2_32_M5; return true; }
+    if (prime == mh_prime_value(MH_PRIME_2_31_M1)) { *kind = MH_PRIME_2_31_M1; return true; }
+    return false;
+}
+culsh_status culsh_generate_minhash_params_mod(uint64_t seed, int n_rows, uint32_t prime, uint32_t* A, uint32_t* B) {
+    int kind = 0;
+    CULSH_REQUIRE(A && B && n_rows > 0, CULSH_ERR_INVALID, "bad argument");
+    CULSH_REQUIRE(prime_kind_of(prime, &kind), CULSH_ERR_INVALID, "MinHash prime must be 4294967291 or 2147483647");
+    gen_minhash(seed, n_rows, A, B, kind);
+    return CULSH_OK;
+}
+culsh_status culsh_ctx_set_minhash_prime(culsh_ctx* ctx, uint32_t prime) {
+    int kind = 0;
+    CULSH_REQUIRE(ctx, CULSH_ERR_INVALID, "null argument");
+    CULSH_REQUIRE(prime_kind_of(prime, &kind), CULSH_ERR_INVALID, "MinHash prime must be 4294967291 or 2147483647");
+    ctx->mh_prime_kind = kind;
+    return CULSH_OK;
+}
+culsh_status culsh_ctx_get_minhash_prime(const culsh_ctx* ctx, uint32_t* prime) {
+    CULSH_REQUIRE(ctx && prime, CULSH_ERR_INVALID, "null argument");
+    *prime = mh_prime_value(ctx->mh_prime_kind);
+    return CULSH_OK;
+}
+culsh_status culsh_index_minhash_prime(const culsh_index* ix, uint32_t* prime) {
+    CULSH_REQUIRE(ix && prime, CULSH_ERR_INVALID, "null argument");
+    CULSH_REQUIRE(ix->kind == CULSH_KIND_MINHASH, CULSH_ERR_INVALID, "not a MinHash index");
+    *prime = mh_prime_value(ix->mh_prime_kind);
+    return CULSH_OK;
+}
 
 // ---- RPLSH
 culsh_status culsh_rplsh_fit_f32(culsh_ctx* ctx, const float* X, int n, int d, int T, int H, uint64_t seed,
@@ -1060,7 +1093,7 @@ culsh_status culsh_minhash_query(culsh_ctx* ctx, const int32_t* indices, const i
         CULSH_TRY(launch_minhash_rank(ctx, indices, indptr, nq, T, H, ix, nullptr, keys));
     } else {
         CULSH_TRY(arena_alloc_t(ctx, static_cast<size_t>(nq) * T * H, &keys));
-        CULSH_TRY(launch_minhash(ctx, indices, indptr, ix->A, ix->B, nq, T, H, true, keys));
+        CULSH_TRY(launch_minhash(ctx, indices, indptr, ix->A, ix->B, nq, T, H, true, keys, ix->mh_prime_kind));
     }
     CandPtr c(new (std::nothrow) culsh_candidates());
     CULSH_REQUIRE(c, CULSH_ERR_NOMEM, "host allocation failed");
@@ -1104,7 +1137,7 @@ culsh_status culsh_pslsh_hash_f64(culsh_ctx* ctx, const double* X, const double*
 culsh_status culsh_minhash_compute(culsh_ctx* ctx, const int32_t* indices, const int32_t* indptr, const uint32_t* A,
                                    const uint32_t* B, int n, int T, int H, uint32_t* sig) {
     STAGE_PROLOGUE();
-    CULSH_TRY(launch_minhash(ctx, indices, indptr, A, B, n, T, H, false, sig));
+    CULSH_TRY(launch_minhash(ctx, indices, indptr, A, B, n, T, H, false, sig, ctx->mh_prime_kind));
     return arena_end(ctx);
 }
 
@@ -1397,6 +1430,7 @@ culsh_status culsh_index_load(culsh_ctx* ctx, culsh_kind kind, int is_double, co
         }
     } else if (kind == CULSH_KIND_MINHASH) {
         CULSH_REQUIRE(param0 && param1, CULSH_ERR_INVALID, "hash_a and hash_b are required");
+        ix->mh_prime_kind = ctx->mh_prime_kind;  // the saved arrays do not name the prime: the context's is taken
         CULSH_TRY(upload(static_cast<const uint32_t*>(param0), TH, &ix->A));
         CULSH_TRY(upload(static_cast<const uint32_t*>(param1), TH, &ix->B));
     }

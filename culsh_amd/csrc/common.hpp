@@ -126,6 +126,7 @@ struct culsh_ctx {
     uint32_t* aux_flag_dev = nullptr;  // a family's own flag that travels with the end-of-build read-back, or null
     uint32_t aux_flag_host = 0;        // its value after that read-back
     bool sort_unchained = false;
+    int mh_prime_kind = 0;  // the prime MinHash fits of this context hash with (culsh_ctx_set_minhash_prime)
     // raw and distinct candidates per query of the last query calls, by the shape of the index they
     // went to (rows, buckets, tables, hashes): sizes the next call's output on an index of that shape
     // without a host round trip (query.hip).  A few shapes are kept, so that a caller who alternates
@@ -161,6 +162,7 @@ struct culsh_index {
     int key_w = 0;
     culsh_amd::PsCodec psc;  // enc == ENC_PSC only
     culsh_amd::MhCodec mhc;  // enc == ENC_MHR only
+    int mh_prime_kind = 0;   // MinHash: the prime the index was hashed with (mh_prime.hpp)
     // family parameters (device): rplsh/index.cuh, pslsh/index.cuh, minhash/index.cuh
     culsh_kind kind = CULSH_KIND_CORE;
     bool is_double = false;
@@ -281,9 +283,10 @@ culsh_status launch_project_f64(culsh_ctx* ctx, const double* X, const double* P
 
 // ---------------------------------------------------------------- minhash (minhash.hip)
 // as_keys: write byte-swapped values (ENC_BE key words) instead of the raw uint32.
+// prime_kind: which prime the family is taken modulo (mh_prime.hpp; 0 = the reference's 2^32 - 5).
 culsh_status launch_minhash(culsh_ctx* ctx, const int32_t* indices, const int32_t* indptr,
                             const uint32_t* A, const uint32_t* B, int n, int T, int H,
-                            bool as_keys, uint32_t* out);
+                            bool as_keys, uint32_t* out, int prime_kind);
 
 // ---------------------------------------------------------------- key codec (index.hip)
 // signature bytes [T][n][S] -> key words [T][n][W]

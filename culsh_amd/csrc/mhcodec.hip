@@ -16,50 +16,34 @@
 #include <algorithm>
 
 #include "common.hpp"
+#include "mh_prime.hpp"
 
 namespace culsh_amd {
 namespace {
 
-constexpr uint32_t PRIME = 4294967291u;  // minhash/hash.cuh:17 (2^32 - 5)
-
-// (a*x + b) mod (2^32 - 5) for a, x, b < 2^32, using 2^32 = 5 (mod p) twice.
-__device__ __forceinline__ uint32_t hash_mod_p(uint32_t a, uint32_t x, uint32_t b) {
-    const uint64_t v = static_cast<uint64_t>(a) * x + b;
-    const uint64_t v1 = 5ull * (v >> 32) + (v & 0xFFFFFFFFull);
-    const uint64_t v2 = 5ull * (v1 >> 32) + (v1 & 0xFFFFFFFFull);
-    return static_cast<uint32_t>(v2 >= PRIME ? v2 - PRIME : v2);
-}
-
-// The same for x < 2^25: a*x + b < 2^57, so the first fold leaves less than 2^32 + 5 * 2^25 and a
-// second fold could only add 5 once: it is merged with the final subtraction.
-__device__ __forceinline__ uint32_t hash_mod_p_small(uint32_t a, uint32_t x, uint32_t b) {
-    const uint64_t v = static_cast<uint64_t>(a) * x + b;
-    const uint64_t v1 = 5ull * (v >> 32) + (v & 0xFFFFFFFFull);
-    const uint32_t lo = static_cast<uint32_t>(v1);
-    return v1 >= PRIME ? lo + 5u : lo;
-}
-
 // ainv[c] = A[c]^(p-2) mod p: the inverse of the multiplier, with which the column that produced a
 // hash value is recovered from the value (the hash is a bijection of [0, p) unless A[c] = 0 mod p)
+template <int PK>
 __global__ __launch_bounds__(256) void mh_inverse_kernel(const uint32_t* __restrict__ A, int count,
                                                         uint32_t* __restrict__ ainv) {
     const int c = blockIdx.x * 256 + threadIdx.x;
     if (c >= count) return;
-    uint32_t base = hash_mod_p(A[c], 1u, 0u), acc = 1u;
-    for (uint32_t e = PRIME - 2u; e; e >>= 1) {
-        if (e & 1u) acc = hash_mod_p(acc, base, 0u);
-        base = hash_mod_p(base, base, 0u);
+    uint32_t base = MhPrime<PK>::hash(A[c], 1u, 0u), acc = 1u;
+    for (uint32_t e = MhPrime<PK>::P - 2u; e; e >>= 1) {
+        if (e & 1u) acc = MhPrime<PK>::hash(acc, base, 0u);
+        base = MhPrime<PK>::hash(base, base, 0u);
     }
     ainv[c] = acc;  // 0 for a multiplier that is 0 mod p (p - 2 is odd, so the first step already gives 0)
 }
 
 // keys[c][f] = byte-order form of hash_c(f): the sort then ranks columns in signature byte order
+template <int PK>
 __global__ __launch_bounds__(256) void mh_hash_columns_kernel(const uint32_t* __restrict__ A,
                                                              const uint32_t* __restrict__ B, int d,
                                                              uint32_t* __restrict__ keys) {
     const int c = blockIdx.y;
     const int f = blockIdx.x * 256 + threadIdx.x;
-    if (f < d) keys[static_cast<size_t>(c) * d + f] = __builtin_bswap32(hash_mod_p(A[c], static_cast<uint32_t>(f), B[c]));
+    if (f < d) keys[static_cast<size_t>(c) * d + f] = __builtin_bswap32(MhPrime<PK>::hash(A[c], static_cast<uint32_t>(f), B[c]));
 }
 
 // sorted_cols[c][r] = column of rank r; sorted_keys[c][r] = its byte-swapped hash
@@ -90,7 +74,7 @@ constexpr int NTHREADS = 256;
 // (row, hash) pairs with hashes fastest; besides the running minimum a thread keeps the column
 // that produced it.  SMALL: every column id is below 2^25; then only the minimum is kept and
 // its column is computed from it at the end, ainv * (min - b) mod p.
-template <bool SMALL>
+template <bool SMALL, int PK>
 __global__ __launch_bounds__(NTHREADS) void minhash_rank_kernel(const int32_t* __restrict__ indices,
                                                                const int32_t* __restrict__ indptr,
                                                                const uint32_t* __restrict__ A,
@@ -122,9 +106,9 @@ __global__ __launch_bounds__(NTHREADS) void minhash_rank_kernel(const int32_t* _
             uint32_t m = 0xFFFFFFFFu, col = 0xFFFFFFFFu;
             auto take = [&](uint32_t f) {
                 if (SMALL) {
-                    m = min(m, hash_mod_p_small(a, f, b));
+                    m = min(m, MhPrime<PK>::hash_small(a, f, b));
                 } else {
-                    const uint32_t h = hash_mod_p(a, f, b);
+                    const uint32_t h = MhPrime<PK>::hash(a, f, b);
                     const bool less = h < m;
                     m = less ? h : m;
                     col = less ? f : col;
@@ -142,9 +126,10 @@ __global__ __launch_bounds__(NTHREADS) void minhash_rank_kernel(const int32_t* _
             for (; j < e; ++j) take(static_cast<uint32_t>(indices[j]));
             if (SMALL && s < e) {
                 const uint32_t ai = ainv[c0 + c];
-                const uint32_t bp = b >= PRIME ? b - PRIME : b;
-                const uint32_t x = m - bp + (m < bp ? PRIME : 0u);  // (m - b) mod p; wraps to the exact value
-                col = ai ? hash_mod_p(ai, x, 0u) : static_cast<uint32_t>(indices[s]);  // all hashes equal: the first stays
+                constexpr uint32_t P = MhPrime<PK>::P;
+                const uint32_t bp = MhPrime<PK>::hash(1u, b, 0u);   // b mod p (an injected b may be any 32-bit value)
+                const uint32_t x = m - bp + (m < bp ? P : 0u);      // (m - b) mod p; wraps to the exact value
+                col = ai ? MhPrime<PK>::hash(ai, x, 0u) : static_cast<uint32_t>(indices[s]);  // all hashes equal: the first stays
             }
             uint32_t code = static_cast<uint32_t>(d);                      // empty row: sorts last
             if (s < e) code = col < static_cast<uint32_t>(d) ? rank[static_cast<size_t>(c0 + c) * d + col]
@@ -323,8 +308,13 @@ culsh_status mh_build_codec(culsh_ctx* ctx, int T, int H, int d, culsh_index* ix
     CULSH_TRY(arena_alloc_t(ctx, total, &keys_tmp));
     CULSH_TRY(arena_alloc_t(ctx, total, &cols_tmp));
     CULSH_TRY(arena_alloc_t(ctx, total, &cols));
-    CULSH_LAUNCH(ctx, mh_hash_columns_kernel, dim3(div_up(d, 256), static_cast<unsigned>(TH)), dim3(256), 0, ctx->stream,
-                 ix->A, ix->B, d, keys);
+    const bool mersenne = ix->mh_prime_kind == MH_PRIME_2_31_M1;
+    if (mersenne)
+        CULSH_LAUNCH(ctx, mh_hash_columns_kernel<MH_PRIME_2_31_M1>, dim3(div_up(d, 256), static_cast<unsigned>(TH)), dim3(256), 0,
+                     ctx->stream, ix->A, ix->B, d, keys);
+    else
+        CULSH_LAUNCH(ctx, mh_hash_columns_kernel<MH_PRIME_2_32_M5>, dim3(div_up(d, 256), static_cast<unsigned>(TH)), dim3(256), 0,
+                     ctx->stream, ix->A, ix->B, d, keys);
     CULSH_LAUNCH_CHECK();
     const uint32_t all_bits = 0xFFFFFFFFu;
     CULSH_TRY(sort_tables(ctx, keys, keys_tmp, cols_tmp, cols, d, static_cast<int>(TH), 1, &all_bits, &sorted));
@@ -335,8 +325,12 @@ culsh_status mh_build_codec(culsh_ctx* ctx, int T, int H, int d, culsh_index* ix
     CULSH_LAUNCH(ctx, mh_invert_kernel, dim3(div_up(total, 256)), dim3(256), 0, ctx->stream, cols, sorted, total, d,
                  mc.rank, mc.inv, static_cast<const uint32_t*>(ctx->sort_err_dev));
     CULSH_LAUNCH_CHECK();
-    CULSH_LAUNCH(ctx, mh_inverse_kernel, dim3(div_up(TH, 256)), dim3(256), 0, ctx->stream, ix->A, static_cast<int>(TH),
-                 mc.ainv);
+    if (mersenne)
+        CULSH_LAUNCH(ctx, mh_inverse_kernel<MH_PRIME_2_31_M1>, dim3(div_up(TH, 256)), dim3(256), 0, ctx->stream, ix->A,
+                     static_cast<int>(TH), mc.ainv);
+    else
+        CULSH_LAUNCH(ctx, mh_inverse_kernel<MH_PRIME_2_32_M5>, dim3(div_up(TH, 256)), dim3(256), 0, ctx->stream, ix->A,
+                     static_cast<int>(TH), mc.ainv);
     CULSH_LAUNCH_CHECK();
     if (ctx->sort_err_dev) {  // the column sort used the chained scan: its flag is settled here
         uint32_t gave_up = 0;
@@ -363,13 +357,17 @@ culsh_status launch_minhash_rank(culsh_ctx* ctx, const int32_t* indices, const i
     const int th_chunk = tables_per_chunk * H;
     const size_t lds = static_cast<size_t>(th_chunk) * rb * sizeof(uint32_t);
     const dim3 grid((n + rb - 1) / rb);
-    if (fit_flag && ix->mhc.d <= (1 << 25))
-        CULSH_LAUNCH(ctx, minhash_rank_kernel<true>, grid, dim3(NTHREADS), lds, ctx->stream, indices, indptr, ix->A, ix->B,
-                     ix->mhc.ainv, ix->mhc.rank, n, T, H, ix->mhc.d, ix->mhc.bits, ix->key_w, th_chunk, rb, keys, fit_flag);
-    else
-        CULSH_LAUNCH(ctx, minhash_rank_kernel<false>, grid, dim3(NTHREADS), lds, ctx->stream, indices, indptr, ix->A, ix->B,
-                     ix->mhc.ainv, ix->mhc.rank, n, T, H, ix->mhc.d, ix->mhc.bits, ix->key_w, th_chunk, rb, keys,
-                     static_cast<uint32_t*>(nullptr));
+    const bool small = fit_flag && ix->mhc.d <= (1 << 25);
+    uint32_t* flag = small ? fit_flag : nullptr;
+#define MH_RANK_CASE(S, PK)                                                                                              \
+    CULSH_LAUNCH(ctx, (minhash_rank_kernel<S, PK>), grid, dim3(NTHREADS), lds, ctx->stream, indices, indptr, ix->A, ix->B, \
+                 ix->mhc.ainv, ix->mhc.rank, n, T, H, ix->mhc.d, ix->mhc.bits, ix->key_w, th_chunk, rb, keys, flag)
+    if (ix->mh_prime_kind == MH_PRIME_2_31_M1) {
+        if (small) MH_RANK_CASE(true, MH_PRIME_2_31_M1); else MH_RANK_CASE(false, MH_PRIME_2_31_M1);
+    } else {
+        if (small) MH_RANK_CASE(true, MH_PRIME_2_32_M5); else MH_RANK_CASE(false, MH_PRIME_2_32_M5);
+    }
+#undef MH_RANK_CASE
     CULSH_LAUNCH_CHECK();
     return CULSH_OK;
 }

@@ -8,23 +8,16 @@
 // staged in LDS and written table-major so that each table receives RB*H consecutive
 // words.
 #include "common.hpp"
+#include "mh_prime.hpp"
 
 namespace culsh_amd {
 namespace {
 
-constexpr uint32_t PRIME = 4294967291u;  // minhash/hash.cuh:17 (2^32 - 5)
-constexpr int RB = 32;                   // rows per workgroup
+constexpr int RB = 32;  // rows per workgroup
 constexpr int NTHREADS = 256;
 
-// (a*x + b) mod (2^32 - 5) for a, x, b < 2^32, using 2^32 = 5 (mod p) twice.
-__device__ __forceinline__ uint32_t hash_mod_p(uint32_t a, uint32_t x, uint32_t b) {
-    const uint64_t v = static_cast<uint64_t>(a) * x + b;                 // < 2^64
-    const uint64_t v1 = 5ull * (v >> 32) + (v & 0xFFFFFFFFull);          // < 6 * 2^32
-    const uint64_t v2 = 5ull * (v1 >> 32) + (v1 & 0xFFFFFFFFull);        // < 2^32 + 25
-    return static_cast<uint32_t>(v2 >= PRIME ? v2 - PRIME : v2);
-}
-
-template <bool AS_KEYS>
+// PK: the prime of the hash family (mh_prime.hpp; the reference's is minhash/hash.cuh:17)
+template <bool AS_KEYS, int PK>
 __global__ __launch_bounds__(NTHREADS) void minhash_kernel(const int32_t* __restrict__ indices,
                                                           const int32_t* __restrict__ indptr,
                                                           const uint32_t* __restrict__ A,
@@ -46,10 +39,10 @@ __global__ __launch_bounds__(NTHREADS) void minhash_kernel(const int32_t* __rest
             for (; j + 4 <= e; j += 4) {  // four loads in flight, then four hash chains
                 const uint32_t f0 = static_cast<uint32_t>(indices[j]), f1 = static_cast<uint32_t>(indices[j + 1]);
                 const uint32_t f2 = static_cast<uint32_t>(indices[j + 2]), f3 = static_cast<uint32_t>(indices[j + 3]);
-                m = min(min(m, hash_mod_p(a, f0, b)), hash_mod_p(a, f1, b));
-                m = min(min(m, hash_mod_p(a, f2, b)), hash_mod_p(a, f3, b));
+                m = min(min(m, MhPrime<PK>::hash(a, f0, b)), MhPrime<PK>::hash(a, f1, b));
+                m = min(min(m, MhPrime<PK>::hash(a, f2, b)), MhPrime<PK>::hash(a, f3, b));
             }
-            for (; j < e; ++j) m = min(m, hash_mod_p(a, static_cast<uint32_t>(indices[j]), b));
+            for (; j < e; ++j) m = min(m, MhPrime<PK>::hash(a, static_cast<uint32_t>(indices[j]), b));
             stage[c * RB + r] = m;
         }
         __syncthreads();
@@ -73,7 +66,7 @@ __global__ __launch_bounds__(NTHREADS) void minhash_kernel(const int32_t* __rest
 
 culsh_status launch_minhash(culsh_ctx* ctx, const int32_t* indices, const int32_t* indptr,
                             const uint32_t* A, const uint32_t* B, int n, int T, int H, bool as_keys,
-                            uint32_t* out) {
+                            uint32_t* out, int prime_kind) {
     CULSH_REQUIRE(indptr && A && B && out, CULSH_ERR_INVALID, "minhash: null pointer");
     CULSH_REQUIRE(n > 0 && T > 0 && H > 0, CULSH_ERR_INVALID, "minhash: sizes must be positive");
     CULSH_REQUIRE(H <= 384, CULSH_ERR_LIMIT, "minhash: n_hashes > 384 is not supported");
@@ -84,10 +77,14 @@ culsh_status launch_minhash(culsh_ctx* ctx, const int32_t* indices, const int32_
     const int th_chunk = tables_per_chunk * H;
     const size_t lds = static_cast<size_t>(th_chunk) * RB * sizeof(uint32_t);
     dim3 grid((n + RB - 1) / RB), block(NTHREADS);
-    if (as_keys)
-        CULSH_LAUNCH(ctx, minhash_kernel<true>, grid, block, lds, ctx->stream, indices, indptr, A, B, n, T, H, th_chunk, out);
-    else
-        CULSH_LAUNCH(ctx, minhash_kernel<false>, grid, block, lds, ctx->stream, indices, indptr, A, B, n, T, H, th_chunk, out);
+#define MINHASH_CASE(K, PK)                                                                                          \
+    CULSH_LAUNCH(ctx, (minhash_kernel<K, PK>), grid, block, lds, ctx->stream, indices, indptr, A, B, n, T, H, th_chunk, out)
+    if (prime_kind == MH_PRIME_2_31_M1) {
+        if (as_keys) MINHASH_CASE(true, MH_PRIME_2_31_M1); else MINHASH_CASE(false, MH_PRIME_2_31_M1);
+    } else {
+        if (as_keys) MINHASH_CASE(true, MH_PRIME_2_32_M5); else MINHASH_CASE(false, MH_PRIME_2_32_M5);
+    }
+#undef MINHASH_CASE
     CULSH_LAUNCH_CHECK();
     return CULSH_OK;
 }

@@ -126,6 +126,8 @@ culsh_status culsh_generate_projection_f64(uint64_t seed, int n_rows, int n_feat
 culsh_status culsh_generate_pslsh_params_f32(uint64_t seed, int n_rows, int n_features, int window_size, float* P_host, float* b_host);
 culsh_status culsh_generate_pslsh_params_f64(uint64_t seed, int n_rows, int n_features, int window_size, double* P_host, double* b_host);
 culsh_status culsh_generate_minhash_params(uint64_t seed, int n_rows, uint32_t* A_host, uint32_t* B_host);
+/* The same normalised for another prime of the family (see culsh_ctx_set_minhash_prime). */
+culsh_status culsh_generate_minhash_params_mod(uint64_t seed, int n_rows, uint32_t prime, uint32_t* A_host, uint32_t* B_host);
 
 /* ---- RPLSH (rplsh/rplsh.cu) --------------------------------------------------------------
  * `P_host_opt`: NULL draws P from `seed`; otherwise a host array [T*H][n_features] of
@@ -153,7 +155,17 @@ culsh_status culsh_pslsh_fit_query_f64(culsh_ctx*, const double* X_dev, int n_sa
 /* ---- MinHash LSH (minhash/minhash.cu) -----------------------------------------------------
  * CSR column ids / row pointers are int32 device arrays; values are not read
  * (minhash_lsh.py:99-100).  `A_host_opt` / `B_host_opt` (both or neither) are already
- * normalised: A in [1,p-1], B in [0,p-1], p = 4294967291 (minhash/hash.cuh:17,26-32). */
+ * normalised: A in [1,p-1], B in [0,p-1], p = 4294967291 (minhash/hash.cuh:17,26-32).
+ *
+ * The prime is a parameter of the hashing kernels.  The reference fixes it at 4294967291 = 2^32 - 5
+ * (`MINHASH_PRIME`, minhash/hash.cuh:17), which is the default and what every parity statement refers to;
+ * culsh_ctx_set_minhash_prime switches the fits, `culsh_minhash_compute` calls and loads of a context to
+ * 2147483647 = 2^31 - 1, the other usual choice (no counterpart in the reference; any other value is
+ * refused).  An index keeps the prime it was fitted with and its queries hash with it; the saved arrays of
+ * the reference's format do not name it, so a load takes the context's. */
+culsh_status culsh_ctx_set_minhash_prime(culsh_ctx*, uint32_t prime);
+culsh_status culsh_ctx_get_minhash_prime(const culsh_ctx*, uint32_t* prime);
+culsh_status culsh_index_minhash_prime(const culsh_index*, uint32_t* prime);
 culsh_status culsh_minhash_fit(culsh_ctx*, const int32_t* indices_dev, const int32_t* indptr_dev, int n_samples, int n_features, int n_hash_tables, int n_hashes, uint64_t seed, const uint32_t* A_host_opt, const uint32_t* B_host_opt, culsh_index** out); /* minhash.cu:19-50 */
 culsh_status culsh_minhash_query(culsh_ctx*, const int32_t* indices_dev, const int32_t* indptr_dev, int n_queries, const culsh_index*, culsh_candidates** out); /* minhash.cu:52-74 */
 culsh_status culsh_minhash_fit_query(culsh_ctx*, const int32_t* indices_dev, const int32_t* indptr_dev, int n_samples, int n_features, int n_hash_tables, int n_hashes, uint64_t seed, const uint32_t* A_host_opt, const uint32_t* B_host_opt, culsh_candidates** out); /* minhash.cu:76-102 */

@@ -104,14 +104,14 @@ def pslsh_hash(X: np.ndarray, P: np.ndarray, b: np.ndarray, T: int, H: int) -> n
     return sig
 
 
-def minhash_hash(indices, indptr, A, B, T: int, H: int) -> np.ndarray:
+def minhash_hash(indices, indptr, A, B, T: int, H: int, prime: int = 4294967291) -> np.ndarray:
     n = len(indptr) - 1
     sig = np.empty((T, n, H), dtype=np.uint32)
     indices = np.ascontiguousarray(indices, dtype=np.int32)
     indptr = np.ascontiguousarray(indptr, dtype=np.int32)
     A = np.ascontiguousarray(A, dtype=np.uint32)
     B = np.ascontiguousarray(B, dtype=np.uint32)
-    lib().oracle_minhash(_p(indices), _p(indptr), _p(A), _p(B), n, T, H, _p(sig))
+    lib().oracle_minhash_mod(_p(indices), _p(indptr), _p(A), _p(B), n, T, H, C.c_uint64(prime), _p(sig))
     return sig
 
 

@@ -163,8 +163,8 @@ void oracle_pslsh_hash_f64(const double* X, const double* P, const double* b, in
 
 /* sig[t][row][h] = min_j ((uint64)A*idx_j + B) mod p, empty row -> 0xFFFFFFFF
  * (minhash/hash.cuh:86-127). */
-void oracle_minhash(const int32_t* indices, const int32_t* indptr, const uint32_t* A,
-                    const uint32_t* B, int n, int T, int H, uint32_t* sig) {
+void oracle_minhash_mod(const int32_t* indices, const int32_t* indptr, const uint32_t* A,
+                        const uint32_t* B, int n, int T, int H, uint64_t prime, uint32_t* sig) {
     const int TH = T * H;
 #pragma omp parallel for schedule(dynamic, 256)
     for (int r = 0; r < n; ++r) {
@@ -173,13 +173,19 @@ void oracle_minhash(const int32_t* indices, const int32_t* indptr, const uint32_
             uint32_t m = 0xFFFFFFFFu;
             for (int j = s; j < e; ++j) {
                 uint64_t v = (uint64_t)A[c] * (uint32_t)indices[j] + (uint64_t)B[c];
-                uint32_t hv = (uint32_t)(v % MINHASH_PRIME);
+                uint32_t hv = (uint32_t)(v % prime);
                 if (hv < m) m = hv;
             }
             int t = c / H, h = c % H;
             sig[(size_t)t * n * H + (size_t)r * H + h] = m;
         }
     }
+}
+
+/* the reference's prime */
+void oracle_minhash(const int32_t* indices, const int32_t* indptr, const uint32_t* A,
+                    const uint32_t* B, int n, int T, int H, uint32_t* sig) {
+    oracle_minhash_mod(indices, indptr, A, B, n, T, H, MINHASH_PRIME, sig);
 }
 
 /* ---------------------------------------------------------------- index build ------ */

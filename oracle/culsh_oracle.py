@@ -37,6 +37,10 @@ from typing import Optional
 import numpy as np
 
 MINHASH_PRIME = 4294967291  # minhash/hash.cuh:17 (largest 32-bit prime, 2**32 - 5)
+# The prime is a parameter of the functions below; the reference's is the default.  The library also
+# takes 2**31 - 1, for which there is no reference code: that case is pinned by big-integer arithmetic
+# only (tests/test_oracle.py).
+MINHASH_PRIME_MERSENNE = 2147483647
 
 _M64 = (1 << 64) - 1
 _GOLD = 0x9E3779B97F4A7C15
@@ -118,18 +122,18 @@ def generate_random_projections_biases(seed: int, n_rows: int, d: int, w: int, d
     return P, b.astype(dtype)
 
 
-def normalize_hash_integers(raw_a: np.ndarray, raw_b: np.ndarray):
+def normalize_hash_integers(raw_a: np.ndarray, raw_b: np.ndarray, prime: int = MINHASH_PRIME):
     """A = raw mod (p-1) + 1 in [1,p-1], B = raw mod p (minhash/hash.cuh:26-32)."""
-    A = (raw_a.astype(np.uint64) % np.uint64(MINHASH_PRIME - 1)) + np.uint64(1)
-    B = raw_b.astype(np.uint64) % np.uint64(MINHASH_PRIME)
+    A = (raw_a.astype(np.uint64) % np.uint64(prime - 1)) + np.uint64(1)
+    B = raw_b.astype(np.uint64) % np.uint64(prime)
     return A.astype(np.uint32), B.astype(np.uint32)
 
 
-def generate_hash_integers(seed: int, n: int):
+def generate_hash_integers(seed: int, n: int, prime: int = MINHASH_PRIME):
     """Seeded uint32 A, B, normalised as minhash/hash.cuh:42-54."""
     raw_a = (raw_u64(seed, STREAM_HASH_A, n) >> np.uint64(32)).astype(np.uint32)
     raw_b = (raw_u64(seed, STREAM_HASH_B, n) >> np.uint64(32)).astype(np.uint32)
-    return normalize_hash_integers(raw_a, raw_b)
+    return normalize_hash_integers(raw_a, raw_b, prime)
 
 
 # --------------------------------------------------------------------------------------
@@ -190,7 +194,7 @@ def pslsh_margin(X: np.ndarray, P: np.ndarray, b: np.ndarray, T: int, H: int) ->
 
 
 def minhash_hash(indices: np.ndarray, indptr: np.ndarray, A: np.ndarray, B: np.ndarray,
-                 T: int, H: int) -> np.ndarray:
+                 T: int, H: int, prime: int = MINHASH_PRIME) -> np.ndarray:
     """uint32 X_sig[T][n][H] = min_j ((uint64)A*idx_j + B) mod p; empty row -> 0xFFFFFFFF;
     CSR values are ignored (minhash/hash.cuh:69-128)."""
     n = len(indptr) - 1
@@ -204,7 +208,7 @@ def minhash_hash(indices: np.ndarray, indptr: np.ndarray, A: np.ndarray, B: np.n
     if len(nonempty) and len(idx64):
         # (A < 2^32) * (idx < 2^32) + (B < 2^32) < 2^64: no wrap in uint64
         for h in range(TH):
-            hashed = (A64[h] * idx64 + B64[h]) % np.uint64(MINHASH_PRIME)
+            hashed = (A64[h] * idx64 + B64[h]) % np.uint64(prime)
             mins = np.minimum.reduceat(hashed, indptr[nonempty].astype(np.int64))
             sig[nonempty, h] = mins.astype(np.uint32)
     return _table_major(sig, T, H)

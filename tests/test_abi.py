@@ -111,6 +111,16 @@ def test_minhash_generator_matches_definition():
     np.testing.assert_array_equal(A, A_ref)
     np.testing.assert_array_equal(B, B_ref)
     assert A.min() >= 1 and int(A.max()) <= o.MINHASH_PRIME - 1 and int(B.max()) <= o.MINHASH_PRIME - 1
+    # the same stream normalised for the other prime of the family; any third value is refused
+    p31 = o.MINHASH_PRIME_MERSENNE
+    assert lib.culsh_generate_minhash_params_mod(123, n, p31, _ptr(A), _ptr(B)) == L.OK
+    A_ref, B_ref = o.generate_hash_integers(123, n, p31)
+    np.testing.assert_array_equal(A, A_ref)
+    np.testing.assert_array_equal(B, B_ref)
+    assert A.min() >= 1 and int(A.max()) <= p31 - 1 and int(B.max()) <= p31 - 1
+    assert lib.culsh_generate_minhash_params_mod(123, n, o.MINHASH_PRIME, _ptr(A), _ptr(B)) == L.OK
+    np.testing.assert_array_equal(A, o.generate_hash_integers(123, n)[0])
+    assert lib.culsh_generate_minhash_params_mod(123, n, 4294967295, _ptr(A), _ptr(B)) != L.OK
 
 
 def test_header_is_plain_c_and_links_from_a_c_program(tmp_path):

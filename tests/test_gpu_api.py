@@ -331,6 +331,49 @@ def test_minhash_save_load_and_fit_query(tmp_path):
         lsh.fit(X64)
 
 
+def test_minhash_prime_is_a_parameter(tmp_path):
+    """`prime` (not in the reference, whose prime is fixed at 2^32 - 5, minhash/hash.cuh:17): a model fitted
+    modulo 2^31 - 1 follows the definition with that prime, names it in its file and comes back from the
+    file as it was; a default model's file holds the reference's keys only."""
+    from culsh_amd import MinHashLSH, MinHashLSHModel
+
+    p31 = o.MINHASH_PRIME_MERSENNE
+    X = sparse(1500, 300, 0.05)
+    T, H = 8, 3
+    with pytest.raises(ValueError, match="prime"):
+        MinHashLSH(n_hash_tables=T, n_hashes=H, seed=3, prime=4294967295)
+    lsh = MinHashLSH(n_hash_tables=T, n_hashes=H, seed=3, prime=p31)
+    model = lsh.fit(X)
+    assert lsh.prime == p31 and model.prime == p31 and model.index.prime == p31
+    A, B = model.index.get_hash_a(), model.index.get_hash_b()
+    np.testing.assert_array_equal(A, o.generate_hash_integers(3, T * H, p31)[0])
+    exp = o.fit_index(o.minhash_hash(X.indices, X.indptr, A, B, T, H, p31), H)
+    np.testing.assert_array_equal(model.index.get_candidate_indices(), exp.all_candidate_indices)
+    np.testing.assert_array_equal(model.index.get_bucket_signatures(), exp.all_bucket_signatures)
+    want = o.query_index(o.minhash_hash(X.indices, X.indptr, A, B, T, H, p31)[:, :200], exp)
+    got = model.query(X[:200])
+    np.testing.assert_array_equal(got.get_indices(), want.query_candidate_indices)
+    np.testing.assert_array_equal(got.get_offsets(), want.query_candidate_offsets)
+    path = os.path.join(tmp_path, "minhash_p31.npz")
+    model.save(path)
+    assert int(np.load(path)["prime"]) == p31
+    loaded = MinHashLSHModel.load(path)
+    assert loaded.prime == p31 and _key_form(loaded.index) == _key_form(model.index)
+    again = loaded.query(X[:200])
+    np.testing.assert_array_equal(again.get_indices(), got.get_indices())
+    np.testing.assert_array_equal(again.get_offsets(), got.get_offsets())
+    fq = lsh.fit_query(X)
+    full = model.query(X)
+    np.testing.assert_array_equal(fq.get_indices(), full.get_indices())
+    # the default: the reference's prime, and no key beyond the reference's in the file
+    plain = MinHashLSH(n_hash_tables=T, n_hashes=H, seed=3).fit(X)
+    assert plain.prime == o.MINHASH_PRIME
+    path2 = os.path.join(tmp_path, "minhash_default.npz")
+    plain.save(path2)
+    assert "prime" not in np.load(path2).files
+    assert MinHashLSHModel.load(path2).prime == o.MINHASH_PRIME
+
+
 def _key_form(index):
     """(key words per bucket, encoding) of an index object of the extension-module surface."""
     import ctypes as C

@@ -969,6 +969,83 @@ def test_minhash_fit_query_path(ctx):
     ctx.free_index(ih2)
 
 
+@pytest.mark.parametrize("n,d,T,H,nnz", [(500, 5000, 32, 4, 50), (77, 300, 5, 3, 8), (64, 100000, 2, 130, 20)])
+def test_minhash_compute_exact_mod_mersenne_prime(n, d, T, H, nnz):
+    """The prime is a parameter of the hashing kernels: 2^31 - 1 instead of the reference's 2^32 - 5,
+    against the oracle with the same prime; parameters at the ends of their ranges and parameters that are
+    not normalised at all (any 32-bit value may be injected)."""
+    _announce("minhash_mersenne", n, d, T, H, nnz)
+    from abi import Ctx
+
+    p31 = o.MINHASH_PRIME_MERSENNE
+    rng = np.random.default_rng(n + H)
+    indices, indptr = make_csr(rng, n, d, nnz, empty_rows=(0,))
+    A, B = o.generate_hash_integers(9, T * H, p31)
+    A[0], B[0] = p31 - 1, p31 - 1
+    if T * H > 2:
+        A[1], B[1] = 0xFFFFFFFF, 0xFFFFFFFE
+    own = Ctx(0)
+    try:
+        with pytest.raises(RuntimeError):
+            own.set_minhash_prime(4294967295)                     # neither of the two primes
+        own.set_minhash_prime(p31)
+        np.testing.assert_array_equal(own.minhash_compute(indices, indptr, A, B, T, H),
+                                      o.minhash_hash(indices, indptr, A, B, T, H, p31))
+        own.set_minhash_prime(o.MINHASH_PRIME)
+        np.testing.assert_array_equal(own.minhash_compute(indices, indptr, A, B, T, H),
+                                      o.minhash_hash(indices, indptr, A, B, T, H))
+    finally:
+        own.close()
+
+
+@pytest.mark.parametrize("beyond", [False, True])
+def test_minhash_fit_query_path_mod_mersenne_prime(c_oracle, beyond):
+    """Fit, query and fit_query with the family taken modulo 2^31 - 1: bucket tables and candidate lists
+    against the oracle on signatures of the same prime.  With rank keys (every column id below
+    n_features; the column of a minimum is recovered through the multiplier's inverse modulo that prime)
+    and with plain keys (`beyond`: some ids at or above n_features, found during the fit)."""
+    _announce("minhash_path_mersenne", beyond)
+    from abi import Ctx, assert_candidates_match, assert_index_matches
+
+    p31 = o.MINHASH_PRIME_MERSENNE
+    rng = np.random.default_rng(78)
+    n, d, T, H, nq = 6000, 3000, 16, 4, 200
+    indices, indptr = make_csr(rng, n, d, 25, empty_rows=(3, 9))
+    if beyond:
+        indices = indices.copy()
+        indices[rng.integers(0, len(indices), 40)] = d + 5
+    qrows = []
+    for i in range(nq):
+        r = indices[indptr[i]:indptr[i + 1]]
+        keep = r[rng.random(len(r)) > 0.1]
+        qrows.append(np.unique(np.concatenate([keep, rng.choice(d, 2)])))
+    qindptr = np.concatenate([[0], np.cumsum([len(r) for r in qrows])]).astype(np.int32)
+    qindices = np.concatenate(qrows).astype(np.int32)
+    own = Ctx(0)
+    try:
+        own.set_minhash_prime(p31)
+        ih = own.minhash_fit(indices, indptr, d, T, H, seed=42)   # seeded parameters, normalised for this prime
+        A, B = o.generate_hash_integers(42, T * H, p31)
+        np.testing.assert_array_equal(own.index_param(ih, 6, np.uint32), A)
+        np.testing.assert_array_equal(own.index_param(ih, 7, np.uint32), B)
+        assert own.index_minhash_prime(ih) == p31
+        sig = c_oracle.minhash_hash(indices, indptr, A, B, T, H, p31)
+        qsig = c_oracle.minhash_hash(qindices, qindptr, A, B, T, H, p31)
+        assert not np.array_equal(sig, c_oracle.minhash_hash(indices, indptr, A, B, T, H))   # the prime matters
+        cix = c_oracle.fit_index_c(sig, H)
+        assert_index_matches(own.index_arrays(ih), cix.to_numpy(n))
+        own.set_minhash_prime(o.MINHASH_PRIME)                    # a query hashes with its index's prime
+        got = own.minhash_query(qindices, qindptr, ih)
+        assert_candidates_match(got, c_oracle.query_index_c(qsig, cix))
+        assert got["n_total_candidates"] > nq // 2
+        own.set_minhash_prime(p31)
+        assert_candidates_match(own.minhash_fit_query(indices, indptr, d, T, H, seed=42, A=A, B=B),
+                                c_oracle.fit_query(sig, H))
+        own.free_index(ih)
+    finally:
+        own.close()
+
+
 def test_pslsh_query_values_never_seen_at_fit(ctx):
     """p-stable keys are stored as per-hash ranks of the values seen at fit time; a query
     hash outside that range (or inside it but never seen) must simply match no bucket."""

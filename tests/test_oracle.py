@@ -325,7 +325,9 @@ def test_pslsh_floor_known_answer():
     np.testing.assert_array_equal(sig[:, :, 0], [[0, -1, 0], [3, -1, 1]])
 
 
-def test_minhash_matches_bigint(c_oracle):
+@pytest.mark.parametrize("prime", [4294967291, 2147483647])
+def test_minhash_matches_bigint(c_oracle, prime):
+    """Both primes the library takes: the reference's 2^32 - 5 (minhash/hash.cuh:17) and 2^31 - 1."""
     rng = np.random.default_rng(8)
     T, H, n, d = 3, 4, 40, 1000
     rows = [np.sort(rng.choice(d, size=rng.integers(0, 12), replace=False)) for _ in range(n)]
@@ -334,16 +336,20 @@ def test_minhash_matches_bigint(c_oracle):
     rows[5] = np.array([2**31 - 1])                              # largest int32 column id
     indptr = np.concatenate([[0], np.cumsum([len(r) for r in rows])]).astype(np.int32)
     indices = np.concatenate(rows).astype(np.int32)
-    A = rng.integers(1, o.MINHASH_PRIME, size=T * H, dtype=np.uint64).astype(np.uint32)
-    B = rng.integers(0, o.MINHASH_PRIME, size=T * H, dtype=np.uint64).astype(np.uint32)
-    A[0], B[0] = o.MINHASH_PRIME - 1, o.MINHASH_PRIME - 1        # extremes of the ranges
+    A = rng.integers(1, prime, size=T * H, dtype=np.uint64).astype(np.uint32)
+    B = rng.integers(0, prime, size=T * H, dtype=np.uint64).astype(np.uint32)
+    A[0], B[0] = prime - 1, prime - 1                            # extremes of the ranges
+    A[1], B[1] = 0xFFFFFFFF, 0xFFFFFFFF                          # injected parameters need not be normalised
     expected = np.empty((T, n, H), dtype=np.uint32)
     for i, r in enumerate(rows):
         for c in range(T * H):
-            vals = [(int(A[c]) * int(x) + int(B[c])) % 4294967291 for x in r]
+            vals = [(int(A[c]) * int(x) + int(B[c])) % prime for x in r]
             expected[c // H, i, c % H] = min(vals) if vals else 0xFFFFFFFF
-    np.testing.assert_array_equal(o.minhash_hash(indices, indptr, A, B, T, H), expected)
-    np.testing.assert_array_equal(c_oracle.minhash_hash(indices, indptr, A, B, T, H), expected)
+    np.testing.assert_array_equal(o.minhash_hash(indices, indptr, A, B, T, H, prime), expected)
+    np.testing.assert_array_equal(c_oracle.minhash_hash(indices, indptr, A, B, T, H, prime), expected)
+    if prime == o.MINHASH_PRIME:                                 # the default is the reference's prime
+        np.testing.assert_array_equal(o.minhash_hash(indices, indptr, A, B, T, H), expected)
+        np.testing.assert_array_equal(c_oracle.minhash_hash(indices, indptr, A, B, T, H), expected)
 
 
 def test_minhash_jaccard_estimate():
