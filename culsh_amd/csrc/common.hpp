@@ -409,7 +409,17 @@ struct SparseDedupArgs {
     int cap;                      // level-2 entries (SparseDedupGeometry)
     int spin_limit;               // polls of an unpublished predecessor before giving up
     unsigned long long* ticks;    // optional [workgroups][8] phase timers (wall clock ticks of thread 0), or null
+    // Optional: only the queries that matched a bucket at all are worked on.  `active` lists them in ascending
+    // order, `*n_active` says how many; the chained scan then runs over positions in that list, `counts` of
+    // the other queries are zero already, and `offsets` are left to a scan over `counts` afterwards.
+    const int32_t* active = nullptr;
+    const unsigned int* n_active = nullptr;
 };
+// Fills `active` / `*n_active` for SparseDedupArgs from the spans of `n_queries` (<= MAX_COMPACT_QUERIES)
+// queries and zeroes `counts`.
+constexpr int MAX_COMPACT_QUERIES = 1 << 18;
+culsh_status launch_active_queries(culsh_ctx* ctx, const void* spans, int n_queries, int T, int32_t* active,
+                                   unsigned int* n_active, uint64_t* counts);
 struct SparseDedupGeometry {
     int l1_per_thread = 0, cap = 0;
     size_t lds_bytes = 0;

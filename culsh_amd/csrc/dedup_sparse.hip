@@ -70,10 +70,13 @@ __global__ __launch_bounds__(DD_THREADS) void dedup_sparse_kernel(SparseDedupArg
         for (int i = tid; i < n16; i += DD_THREADS) z[i] = make_uint4(0u, 0u, 0u, 0u);
     }
     __syncthreads();
+    // `q` numbers the units of the chained scan: queries, or positions in the list of active queries
+    const int n_units = a.active ? static_cast<int>(*a.n_active) : a.n_queries;
+    auto query_of = [&](int unit) { return a.active ? a.active[unit] : unit; };
     int q = *sh_q;
-    if (q >= a.n_queries) return;
+    if (q >= n_units) return;
     int2 sp = make_int2(0, 0);
-    if (tid < T) sp = spans[static_cast<size_t>(q) * T + tid];
+    if (tid < T) sp = spans[static_cast<size_t>(query_of(q)) * T + tid];
 
     // The query whose rows are lined up in level 2 and wait for the position of their list.
     bool pending = false;
@@ -95,9 +98,12 @@ __global__ __launch_bounds__(DD_THREADS) void dedup_sparse_kernel(SparseDedupArg
                 b = ~0ull;
             }
             *sh_base = b;
-            a.counts[qq] = total;
-            a.offsets[qq] = excl;
-            if (qq == a.n_queries - 1) a.offsets[a.n_queries] = excl + total;
+            const int id = query_of(qq);
+            a.counts[id] = total;
+            if (!a.active) {  // (with a list of active queries the offsets come from a scan over the counts)
+                a.offsets[id] = excl;
+                if (qq == n_units - 1) a.offsets[a.n_queries] = excl + total;
+            }
         }
     };
     // Stores this wavefront's steps of a rank range whose rows are lined up (or, for a step with more
@@ -153,7 +159,7 @@ __global__ __launch_bounds__(DD_THREADS) void dedup_sparse_kernel(SparseDedupArg
     };
 
     for (;;) {
-        int q_next = a.n_queries;
+        int q_next = n_units;
         int2 sp_next = make_int2(0, 0);
         if (tid < T) {
             s_start[tid] = sp.x;
@@ -340,8 +346,8 @@ __global__ __launch_bounds__(DD_THREADS) void dedup_sparse_kernel(SparseDedupArg
             }
             if (lane == 0) wtot[wave] = st_total[0] + st_total[1] + st_total[2] + st_total[3];
             if (last && wave == 0) {
-                const int qn = min(static_cast<int>(__shfl(ticket_next, 0, 64)), a.n_queries);
-                if (T <= 64 && qn < a.n_queries && lane < T) sp_next = spans[static_cast<size_t>(qn) * T + lane];
+                const int qn = min(static_cast<int>(__shfl(ticket_next, 0, 64)), n_units);
+                if (T <= 64 && qn < n_units && lane < T) sp_next = spans[static_cast<size_t>(query_of(qn)) * T + lane];
                 if (lane == 0) *sh_q = qn;
             }
             SP_TICK(5)  // load, line-up
@@ -377,18 +383,67 @@ __global__ __launch_bounds__(DD_THREADS) void dedup_sparse_kernel(SparseDedupArg
             SP_TICK(6)  // totals
             if (last) q_next = *sh_q;
         }
-        if (q_next >= a.n_queries) break;
+        if (q_next >= n_units) break;
         q = q_next;
         if (T <= 64) {
             sp = sp_next;  // zero outside the first T lanes
         } else {
             sp = make_int2(0, 0);
-            if (tid < T) sp = spans[static_cast<size_t>(q) * T + tid];
+            if (tid < T) sp = spans[static_cast<size_t>(query_of(q)) * T + tid];
         }
     }
     if (pending) flush_pending();
     SP_TICK(7)
 #undef SP_TICK
+}
+
+// The queries with at least one non-empty span, in ascending order.  First every query is looked at (one thread
+// each, `flags[q]` = it has a candidate; `counts[q]` is zeroed on the way), then a single workgroup writes the
+// list: that keeps the order without a scan across workgroups, and reading one flag per query is short work.
+__global__ __launch_bounds__(256) void active_flags_kernel(const int2* __restrict__ spans, int n_queries, int T,
+                                                          uint32_t* __restrict__ flags, uint64_t* __restrict__ counts) {
+    const int q = blockIdx.x * 256 + threadIdx.x;
+    if (q >= n_queries) return;
+    const int2* s = spans + static_cast<size_t>(q) * T;
+    int most = 0;
+    for (int t = 0; t < T; ++t) most = max(most, s[t].y);
+    flags[q] = most > 0 ? 1u : 0u;
+    counts[q] = 0;
+}
+
+constexpr int AQ_PER_THREAD = 4;
+__global__ __launch_bounds__(DD_THREADS) void active_queries_kernel(const uint32_t* __restrict__ flags, int n_queries,
+                                                                   int32_t* __restrict__ active,
+                                                                   unsigned int* __restrict__ n_active) {
+    __shared__ uint32_t wave_count[NWAVES];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    uint32_t done = 0;  // active queries before this round's
+    for (int base = 0; base < n_queries; base += DD_THREADS * AQ_PER_THREAD) {
+        // thread `tid` looks at AQ_PER_THREAD consecutive queries, so that list order = thread order
+        const int q0 = base + tid * AQ_PER_THREAD;
+        uint32_t mask = 0;
+#pragma unroll
+        for (int j = 0; j < AQ_PER_THREAD; ++j)
+            if (q0 + j < n_queries && flags[q0 + j]) mask |= 1u << j;
+        const uint32_t mine = __popc(mask);
+        const uint32_t incl = wave_inclusive_sum_dpp(mine);
+        if (lane == 63) wave_count[wave] = incl;
+        __syncthreads();
+        uint32_t before = done, total = 0;
+#pragma unroll
+        for (int w = 0; w < NWAVES; ++w) {
+            const uint32_t v = wave_count[w];
+            before += (w < wave) ? v : 0u;
+            total += v;
+        }
+        uint32_t pos = before + incl - mine;
+#pragma unroll
+        for (int j = 0; j < AQ_PER_THREAD; ++j)
+            if (mask & (1u << j)) active[pos++] = q0 + j;
+        done += total;
+        __syncthreads();  // wave_count is rewritten in the next round
+    }
+    if (tid == 0) *n_active = done;
 }
 
 size_t fixed_lds(int T) {
@@ -412,6 +467,20 @@ bool sparse_dedup_geometry(const culsh_ctx* ctx, int n_rows, int T, int cap_limi
     g->cap = static_cast<int>(cap);
     g->lds_bytes = l1_bytes + cap * sizeof(uint2) + fixed;
     return true;
+}
+
+culsh_status launch_active_queries(culsh_ctx* ctx, const void* spans, int n_queries, int T, int32_t* active,
+                                   unsigned int* n_active, uint64_t* counts) {
+    CULSH_REQUIRE(spans && active && n_active && counts && n_queries > 0 && n_queries <= MAX_COMPACT_QUERIES && T > 0,
+                  CULSH_ERR_INTERNAL, "active queries: bad argument");
+    uint32_t* flags = nullptr;
+    CULSH_TRY(arena_alloc_t(ctx, static_cast<size_t>(n_queries), &flags));
+    CULSH_LAUNCH(ctx, active_flags_kernel, dim3(div_up(static_cast<size_t>(n_queries), 256)), dim3(256), 0, ctx->stream,
+                 static_cast<const int2*>(spans), n_queries, T, flags, counts);
+    CULSH_LAUNCH_CHECK();
+    CULSH_LAUNCH(ctx, active_queries_kernel, dim3(1), dim3(DD_THREADS), 0, ctx->stream, flags, n_queries, active, n_active);
+    CULSH_LAUNCH_CHECK();
+    return CULSH_OK;
 }
 
 culsh_status launch_dedup_sparse(culsh_ctx* ctx, const SparseDedupArgs& a, const SparseDedupGeometry& g) {

@@ -984,6 +984,7 @@ culsh_status query_from_spans(culsh_ctx* ctx, const int2* spans, const unsigned 
             a.raw_offsets = raw_offsets;
             a.state = nullptr;
         }
+        bool compacted = false;  // the two-level kernel works on the queries that matched a bucket only
         int32_t* lists = lists_dst;
         if (!in_place) {
             lists = nullptr;
@@ -1010,6 +1011,19 @@ culsh_status query_from_spans(culsh_ctx* ctx, const int2* spans, const unsigned 
             s.cap = sg.cap;
             s.spin_limit = a.spin_limit;
             s.ticks = ticks_dev;
+            // Inside one bitmap pass this kernel is only taken for queries with next to no candidates, and
+            // most of those match no bucket at all: they are left out (their counts are zero, a query
+            // costs the kernel several barriers whatever it holds) and the offsets come from a scan.
+            compacted = !several && n_queries <= MAX_COMPACT_QUERIES && env_int("CULSH_DEDUP_COMPACT", 1) != 0;
+            if (compacted) {
+                int32_t* active = nullptr;
+                unsigned int* n_active = nullptr;
+                CULSH_TRY(arena_alloc_t(ctx, static_cast<size_t>(n_queries), &active));
+                CULSH_TRY(arena_alloc_t(ctx, 1, &n_active));
+                CULSH_TRY(launch_active_queries(ctx, spans, n_queries, T, active, n_active, out->query_candidate_counts));
+                s.active = active;
+                s.n_active = n_active;
+            }
             CULSH_TRY(launch_dedup_sparse(ctx, s, sg));
         } else {
             {   // more LDS than a launch may ask for by default: allowed once per kernel and device, not per call
@@ -1033,7 +1047,8 @@ culsh_status query_from_spans(culsh_ctx* ctx, const int2* spans, const unsigned 
                              ctx->stream, a);
             CULSH_LAUNCH_CHECK();
         }
-        if (path == P_PASSES) CULSH_TRY(exclusive_scan_u64(ctx, out->query_candidate_counts, out->query_candidate_offsets, n_queries));
+        if (path == P_PASSES || compacted)
+            CULSH_TRY(exclusive_scan_u64(ctx, out->query_candidate_counts, out->query_candidate_offsets, n_queries));
         CULSH_HIP(hipMemcpyAsync(&ctx->pinned[0], out->query_candidate_offsets + n_queries, sizeof(uint64_t),
                                  hipMemcpyDeviceToHost, ctx->stream));
         CULSH_HIP(hipMemcpyAsync(&ctx->pinned[1], err, sizeof(unsigned int), hipMemcpyDeviceToHost, ctx->stream));

@@ -481,17 +481,21 @@ def test_core_query_sparse_passes_at_full_bitmap_size(ctx, c_oracle):
     ctx.free_index(ih)
 
 
+@pytest.mark.parametrize("compact", [1, 0])
 @pytest.mark.parametrize("cap", [0, 64, 8])
 @pytest.mark.parametrize("n", [3000, 70_000])
-def test_core_query_two_level_bitmap(ctx, c_oracle, monkeypatch, n, cap):
+def test_core_query_two_level_bitmap(ctx, c_oracle, monkeypatch, n, cap, compact):
     """The de-duplication kernel for queries with few candidates for the row range, forced on a small
     index: one bit per block of 32 rows, the non-empty blocks ranked, one word of row bits per ranked
     block.  Rows at both ends of a block, of a level-1 word (1024 rows) and of the index; a bucket of
     consecutive rows (blocks filled completely: a read-out step with more rows than its place holds is
     stored from registers); queries without candidates; tables that repeat each other's rows.  With a
-    level 2 of 64 or 8 entries the queries take many rank ranges (counted first, then stored)."""
-    _announce("two_level_bitmap", n, cap)
+    level 2 of 64 or 8 entries the queries take many rank ranges (counted first, then stored).  `compact`:
+    the kernel is handed the list of queries that matched a bucket (the way it runs inside one bitmap
+    pass) or every query."""
+    _announce("two_level_bitmap", n, cap, compact)
     monkeypatch.setenv("CULSH_DEDUP_SPARSE", "1")
+    monkeypatch.setenv("CULSH_DEDUP_COMPACT", str(compact))
     if cap:
         monkeypatch.setenv("CULSH_DEDUP_SPARSE_CAP", str(cap))
     rng = np.random.default_rng(1000 + n + cap)
