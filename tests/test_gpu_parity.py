@@ -596,6 +596,40 @@ def test_core_query_with_next_to_no_candidates_takes_the_two_level_kernel(ctx, c
     ctx.free_index(ih)
 
 
+@pytest.mark.parametrize("seed", range(6))
+def test_core_query_every_path_on_random_shapes(ctx, c_oracle, monkeypatch, seed):
+    """One seeded random index and query set (tables, rows, bucket sizes, share of queries without a match
+    and of repeated rows all drawn) through every de-duplication path the library has: the choice it makes
+    by itself, the bitmap kernel with several passes, the two-level kernel with and without the list of
+    matched queries and with a small level 2, and the count / scan / emit launches.  All against the oracle."""
+    _announce("every_path", seed)
+    rng = np.random.default_rng(4000 + seed)
+    T = int(rng.choice([1, 3, 17, 64, 65, 130]))
+    n = int(rng.choice([700, 5000, 40_000, 150_000]))
+    H = 2
+    values = int(rng.choice([3, 12, 40]))                                    # n / values^2 rows per bucket
+    nq = int(rng.integers(1, 400))
+    sig = rng.integers(0, values, size=(T, n, H)).astype(np.uint8)
+    if T > 1:
+        sig[T // 2] = sig[0]                                                 # two tables with the same buckets
+    qsig = rng.integers(0, values, size=(T, nq, H)).astype(np.uint8)
+    qsig[:, rng.random(nq) < rng.choice([0.0, 0.5, 0.95]), :] = 250          # queries that match nothing
+    ih, _ = ctx.core_fit_index(sig, H)
+    from abi import assert_candidates_match
+
+    exp = c_oracle.query_index_c(qsig, c_oracle.fit_index_c(sig, H))
+    paths = [{}, {"CULSH_DEDUP_WPT": "1"}, {"CULSH_DEDUP_SPARSE": "1"}, {"CULSH_DEDUP_SPARSE": "1", "CULSH_DEDUP_COMPACT": "0"},
+             {"CULSH_DEDUP_SPARSE": "1", "CULSH_DEDUP_SPARSE_CAP": "32"}, {"CULSH_DEDUP_TWO_PASS": "1"},
+             {"CULSH_QUERY_RAW_GUESS": "0"}]
+    for env in paths:
+        with monkeypatch.context() as m:
+            for k, v in env.items():
+                m.setenv(k, v)
+            for _ in range(2):                                               # the second call sizes its output from the first
+                assert_candidates_match(ctx.core_query_index(qsig, ih), exp)
+    ctx.free_index(ih)
+
+
 def test_core_query_two_level_bitmap_look_back_gives_up(ctx, monkeypatch):
     """The two-level kernel with no polls allowed in its chained scan: the call is redone with the
     count / scan / emit launches."""
