@@ -12,6 +12,7 @@ pytestmark = pytest.mark.gpu
     ["--config", "c1", "--fit-query", "--host-inputs", "--repeats", "0", "-ne", "3", "-k", "10"],
     ["--config", "c3", "-n", "20000", "-nq", "200", "--repeats", "1", "-ne", "4", "-k", "10", "-bs", "64"],
     ["--config", "c4", "-n", "5000", "-nq", "100", "--repeats", "1", "-ne", "4", "-k", "10"],
+    ["--config", "c4", "-n", "5000", "-nq", "100", "--repeats", "1", "-ne", "4", "-k", "10", "--prime", "2147483647"],
 ])
 def test_benchmark_report(argv, capsys):
     from culsh_amd import benchmark
@@ -27,6 +28,8 @@ def test_benchmark_report(argv, capsys):
         assert report["runtimes"]["fit_time"] > 0 and report["runtimes"]["query_time"] > 0
         assert report["throughput"]["fit_mvec_per_s"] > 0
         assert report["index"]["n_total_buckets"] > 0
+    if report["algorithm"] == "MinHashLSH":  # every MinHash report names its prime
+        assert report["params"]["prime"] == (2147483647 if "--prime" in argv else 4294967291)
     rec = report["recall_evaluation"]
     for k, v in rec["recall_at_k"].items():
         assert 0.0 <= v <= 1.0
