@@ -889,6 +889,31 @@ def test_batched_query_lists_written_in_place(ctx, order):
     ctx.free_index(ih)
 
 
+@pytest.mark.parametrize("forced", ["", "sparse"])
+def test_batched_query_with_next_to_no_candidates(ctx, monkeypatch, forced):
+    """Batches whose queries mostly match nothing: inside a batch the two-level kernel works on the list of
+    matched queries and takes its offsets from a scan, while the batches' lists still go into one array one
+    behind the other.  Batched equals unbatched for several batch sizes; `sparse` forces that kernel for every
+    batch, also the ones the library would give to the bitmap kernel."""
+    _announce("batched_few_candidates", forced)
+    if forced:
+        monkeypatch.setenv("CULSH_DEDUP_SPARSE", "1")
+    rng = np.random.default_rng(99)
+    n, d, T, H = 150_000, 16, 5, 40                        # 40 hash bits per table: nearly every row alone in its bucket
+    X = rng.standard_normal((n, d)).astype(np.float32)
+    P = rng.standard_normal((T * H, d)).astype(np.float32)
+    Q = rng.standard_normal((900, d)).astype(np.float32)   # matches nothing, mostly
+    Q[::9] = X[rng.integers(0, n, 100)]                    # every ninth query is a fitted row: at least itself
+    ih = ctx.rplsh_fit(X, T, H, seed=1, P=P)
+    want = ctx.rplsh_query(Q, ih)
+    assert 100 <= want["n_total_candidates"] < 5000 and (want["counts"] == 0).sum() > 500
+    for bs in (300, 128, 77):
+        got = ctx.rplsh_query(Q, ih, batch_size=bs)
+        for k in ("counts", "offsets", "indices"):
+            np.testing.assert_array_equal(got[k], want[k])
+    ctx.free_index(ih)
+
+
 def test_rplsh_seeded_projection_matches_generator(ctx):
     """fit without an injected P draws it from the seed with the documented generator."""
     rng = np.random.default_rng(2)
