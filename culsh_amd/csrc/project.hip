@@ -95,11 +95,17 @@ __global__ __launch_bounds__(NTHREADS, (BK <= 8 ? 5 : (BK <= 16 ? 4 : 3))) void 
     // robin to the 8 XCDs; ids are arranged so that all column tiles of one row tile land
     // on the same XCD (same id mod 8) and close in time, so the X tile is fetched from HBM
     // once and served from that XCD's L2 afterwards.
+    //
+    // A workgroup takes the tiles w, w + G, w + 2G, ... of that numbering, G (the grid) being a multiple
+    // of 8 * n_col_tiles: its column tile and XCD never change, and a tile's first stage is fetched under
+    // the last stage of the tile before.  The host launches one workgroup per tile (G = all tiles) or, for
+    // launches of a single column tile, as many workgroups as stay resident.
     const int nct = a.n_col_tiles;
     const int per_group = 8 * nct;
-    const int g = blockIdx.x / per_group, rem = blockIdx.x - g * per_group;
+    const int g0 = blockIdx.x / per_group, rem = blockIdx.x - g0 * per_group;
     const int ct = rem >> 3, slot = rem & 7;
-    const int rt = g * 8 + slot;
+    const int g_step = gridDim.x / per_group;       // row-tile groups between two tiles of this workgroup
+    int rt = g0 * 8 + slot;                           // the tile being multiplied
     if (rt >= a.n_row_tiles) return;
 
     const int tid = threadIdx.x;
@@ -112,16 +118,23 @@ __global__ __launch_bounds__(NTHREADS, (BK <= 8 ? 5 : (BK <= 16 ? 4 : 3))) void 
     // global -> LDS staging: thread loads float4 number (tid + 256*i), i < 4, of each tile.
     // Addresses are a wavefront-uniform tile base plus a 32-bit element offset per thread.
     const int lrow = tid / F4, c4 = (tid % F4) * 4;
-    const float* xbase = a.X + static_cast<size_t>(rt) * BM * d;
+    const float* xbase = nullptr;  // of the tile being fetched (the next one during a tile's last stage)
     uint32_t xoff[NLD], poff[NLD];
     bool xok[NLD], pok[NLD];
+    auto fetch_from_tile = [&](int rt_f) {
+        xbase = a.X + static_cast<size_t>(rt_f) * BM * d;
+#pragma unroll
+        for (int i = 0; i < NLD; ++i) {
+            const int lr = lrow + RSTEP * i;  // row inside the tile
+            xok[i] = rt_f * BM + lr < n;
+            // VEC reads a valid row instead of predicating: the last row of X for rows past the end
+            xoff[i] = static_cast<uint32_t>(VEC ? min(lr, n - 1 - rt_f * BM) : lr) * static_cast<uint32_t>(d);
+        }
+    };
+    fetch_from_tile(rt);
 #pragma unroll
     for (int i = 0; i < NLD; ++i) {
         const int lr = lrow + RSTEP * i;  // row inside the tile
-        const int row = rt * BM + lr;
-        xok[i] = row < n;
-        // VEC reads a valid row instead of predicating: the last row of X for rows past the end
-        xoff[i] = static_cast<uint32_t>(VEC ? min(lr, n - 1 - rt * BM) : lr) * static_cast<uint32_t>(d);
         const int vc = ct * BN + lr;
         const int prow = (EPI == EPI_SIGN_KEYS) ? sign_vcol_to_prow(vc, T, H) : (vc < TH ? vc : -1);
         pok[i] = prow >= 0;
@@ -156,214 +169,241 @@ __global__ __launch_bounds__(NTHREADS, (BK <= 8 ? 5 : (BK <= 16 ? 4 : 3))) void 
         }
     };
 
-    f32x16 acc[2][2];
-#pragma unroll
-    for (int i = 0; i < 2; ++i)
-#pragma unroll
-        for (int j = 0; j < 2; ++j)
-#pragma unroll
-            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
-
     float4 ra[NLD], rb[NLD];
-    fetch(c4, ra, rb);
-
-    const int nk = (d + BK - 1) / BK;
-    for (int kt = 0; kt < nk; ++kt) {
+    auto stage_to_lds = [&]() {
 #pragma unroll
         for (int i = 0; i < NLD; ++i) {
             *reinterpret_cast<float4*>(&As[(lrow + RSTEP * i) * PITCH + c4]) = ra[i];
             *reinterpret_cast<float4*>(&Bs[(lrow + RSTEP * i) * PITCH + c4]) = rb[i];
         }
-        __syncthreads();
-        if (kt + 1 < nk) fetch((kt + 1) * BK + c4, ra, rb);
-        // The 32x32x2 MFMA takes, per lane, A[row = lane%32][k = lane/32] and
-        // B[k = lane/32][col = lane%32].  Any pairing of k between A and B that covers each
-        // feature once is a valid dot product, so lanes 0-31 walk features 0..15 of the
-        // stage and lanes 32-63 features BK/2..BK-1: each lane reads BK/2 consecutive floats.
-        constexpr int KH = BK / 2;  // features per lane and stage
-        float af[2][KH], bf[2][KH];
-#pragma unroll
-        for (int i = 0; i < 2; ++i) {
-            const float* pa = &As[(wm * 64 + i * 32 + r32) * PITCH + half * KH];
-            const float* pb = &Bs[(wn * 64 + i * 32 + r32) * PITCH + half * KH];
-#pragma unroll
-            for (int q = 0; q < KH / 4; ++q) {
-                const float4 va = *reinterpret_cast<const float4*>(pa + 4 * q);
-                const float4 vb = *reinterpret_cast<const float4*>(pb + 4 * q);
-                af[i][4 * q + 0] = va.x; af[i][4 * q + 1] = va.y;
-                af[i][4 * q + 2] = va.z; af[i][4 * q + 3] = va.w;
-                bf[i][4 * q + 0] = vb.x; bf[i][4 * q + 1] = vb.y;
-                bf[i][4 * q + 2] = vb.z; bf[i][4 * q + 3] = vb.w;
-            }
-        }
-#pragma unroll
-        for (int k = 0; k < KH; ++k)
-#pragma unroll
-            for (int i = 0; i < 2; ++i)
-#pragma unroll
-                for (int j = 0; j < 2; ++j)
-                    // The key epilogue wants a lane to hold one column of its tile, the others one row
-                    // (four neighbouring hashes per register quad): those swap the operands and get
-                    // the transposed tile.
-                    acc[i][j] = (EPI == EPI_SIGN_KEYS)
-                                    ? __builtin_amdgcn_mfma_f32_32x32x2f32(af[i][k], bf[j][k], acc[i][j], 0, 0, 0)
-                                    : __builtin_amdgcn_mfma_f32_32x32x2f32(bf[j][k], af[i][k], acc[i][j], 0, 0, 0);
-        __syncthreads();
-    }
+    };
+    fetch(c4, ra, rb);
+    stage_to_lds();
+    __syncthreads();
 
-    // Accumulator layout of the 32x32 tile: register v of lane l holds
-    // row 8*(v/4) + 4*(l/32) + v%4, column l%32 of (first operand) x (second operand).
-    if (EPI == EPI_SIGN_KEYS) {
+    const int nk = (d + BK - 1) / BK;
+    for (;;) {  // tiles of this workgroup
+        const int rt_next = rt + 8 * g_step;
+        const bool has_next = rt_next < a.n_row_tiles;
+        f32x16 acc[2][2];
 #pragma unroll
         for (int i = 0; i < 2; ++i)
 #pragma unroll
-            for (int j = 0; j < 2; ++j) {
-                int mine = 0;
+            for (int j = 0; j < 2; ++j)
 #pragma unroll
-                for (int v = 0; v < 16; ++v) {
-                    // hash bit = 1 iff the sign bit is clear (rplsh/hash.cuh:47)
-                    const unsigned long long m =
-                        __builtin_amdgcn_ballot_w64((__float_as_uint(acc[i][j][v]) >> 31) == 0u);
-                    // the low half of the ballot is the word of row rlo, the high half that of row
-                    // rlo + 4: each goes to the lane of that number
-                    const int rlo = 8 * (v >> 2) + (v & 3);
-                    const uint32_t m_lo = static_cast<uint32_t>(m), m_hi = static_cast<uint32_t>(m >> 32);
-                    // (on gfx950 a vector instruction may not read an SGPR in the two issue slots after
-                    // the vector compare that wrote it; the compiler does not pad inline assembly)
-                    asm("s_nop 1\n\tv_writelane_b32 %0, %1, %3\n\tv_writelane_b32 %0, %2, %4"
-                        : "+v"(mine)
-                        : "s"(m_lo), "s"(m_hi), "n"(rlo), "n"(rlo + 4));
-                }
-                if (lane < 32) tw[(wm * 64 + i * 32 + lane) * (BN / 32) + (wn * 2 + j)] = static_cast<uint32_t>(mine);
+                for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+
+        for (int kt = 0; kt < nk; ++kt) {
+            // LDS holds stage kt.  The next stage is fetched under this one's products: the tile's own, or
+            // after its last stage the first one of the workgroup's next tile.
+            const bool more = kt + 1 < nk;
+            if (more) {
+                fetch((kt + 1) * BK + c4, ra, rb);
+            } else if (has_next) {
+                fetch_from_tile(rt_next);
+                fetch(c4, ra, rb);
             }
-        __syncthreads();
-        uint32_t* keys = static_cast<uint32_t*>(a.out);
-        if (H <= 32) {
-            const int tpt = 32 / H;
-            const uint32_t mask = (H == 32) ? 0xFFFFFFFFu : ((1u << H) - 1u);
-            // (table slot tl, row) pairs, rows fastest: a thread keeps its row and steps tl by
-            // NTHREADS / BM, carrying (tc, sub) = (tl / tpt, tl % tpt) along without dividing
-            constexpr int TL_STEP = NTHREADS / BM;
-            const int row = tid % BM, grow = rt * BM + row;
-            int tl = tid / BM;
-            int tc = tl / tpt, sub = tl - tc * tpt;
-            for (; tl < (BN / 32) * tpt; tl += TL_STEP) {
-                const int table = (ct * (BN / 32) + tc) * tpt + sub;
-                if (table < T && grow < n) {
-                    const uint32_t field = (tw[row * (BN / 32) + tc] >> (sub * H)) & mask;
-                    keys[static_cast<size_t>(table) * n + grow] = field << (32 - H);
+            // The 32x32x2 MFMA takes, per lane, A[row = lane%32][k = lane/32] and
+            // B[k = lane/32][col = lane%32].  Any pairing of k between A and B that covers each
+            // feature once is a valid dot product, so lanes 0-31 walk features 0..15 of the
+            // stage and lanes 32-63 features BK/2..BK-1: each lane reads BK/2 consecutive floats.
+            constexpr int KH = BK / 2;  // features per lane and stage
+            float af[2][KH], bf[2][KH];
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+                const float* pa = &As[(wm * 64 + i * 32 + r32) * PITCH + half * KH];
+                const float* pb = &Bs[(wn * 64 + i * 32 + r32) * PITCH + half * KH];
+#pragma unroll
+                for (int q = 0; q < KH / 4; ++q) {
+                    const float4 va = *reinterpret_cast<const float4*>(pa + 4 * q);
+                    const float4 vb = *reinterpret_cast<const float4*>(pb + 4 * q);
+                    af[i][4 * q + 0] = va.x; af[i][4 * q + 1] = va.y;
+                    af[i][4 * q + 2] = va.z; af[i][4 * q + 3] = va.w;
+                    bf[i][4 * q + 0] = vb.x; bf[i][4 * q + 1] = vb.y;
+                    bf[i][4 * q + 2] = vb.z; bf[i][4 * q + 3] = vb.w;
                 }
-                sub += TL_STEP;
-                while (sub >= tpt) { sub -= tpt; ++tc; }
+            }
+#pragma unroll
+            for (int k = 0; k < KH; ++k)
+#pragma unroll
+                for (int i = 0; i < 2; ++i)
+#pragma unroll
+                    for (int j = 0; j < 2; ++j)
+                        // The key epilogue wants a lane to hold one column of its tile, the others one row
+                        // (four neighbouring hashes per register quad): those swap the operands and get
+                        // the transposed tile.
+                        acc[i][j] = (EPI == EPI_SIGN_KEYS)
+                                        ? __builtin_amdgcn_mfma_f32_32x32x2f32(af[i][k], bf[j][k], acc[i][j], 0, 0, 0)
+                                        : __builtin_amdgcn_mfma_f32_32x32x2f32(bf[j][k], af[i][k], acc[i][j], 0, 0, 0);
+            __syncthreads();  // every wavefront has its fragments: the stage may be overwritten
+            if (more || has_next) stage_to_lds();
+            __syncthreads();
+        }
+
+        // The epilogue's indices are derived again for every tile from a value the compiler cannot see
+        // through: hoisted out of the tile loop as the loop invariants they are, they would sit in registers
+        // all through the stage loop, which has none to spare.
+        int e_tid = tid;
+        asm volatile("" : "+v"(e_tid));
+        const int e_lane = e_tid & 63, e_wave = e_tid >> 6;
+        const int e_wm = e_wave >> 1, e_wn = e_wave & 1;
+        const int e_r32 = e_lane & 31, e_half = e_lane >> 5;
+        // Accumulator layout of the 32x32 tile: register v of e_lane l holds
+        // row 8*(v/4) + 4*(l/32) + v%4, column l%32 of (first operand) x (second operand).
+        if (EPI == EPI_SIGN_KEYS) {
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+#pragma unroll
+                for (int j = 0; j < 2; ++j) {
+                    int mine = 0;
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) {
+                        // hash bit = 1 iff the sign bit is clear (rplsh/hash.cuh:47)
+                        const unsigned long long m =
+                            __builtin_amdgcn_ballot_w64((__float_as_uint(acc[i][j][v]) >> 31) == 0u);
+                        // the low e_half of the ballot is the word of row rlo, the high e_half that of row
+                        // rlo + 4: each goes to the e_lane of that number
+                        const int rlo = 8 * (v >> 2) + (v & 3);
+                        const uint32_t m_lo = static_cast<uint32_t>(m), m_hi = static_cast<uint32_t>(m >> 32);
+                        // (on gfx950 a vector instruction may not read an SGPR in the two issue slots after
+                        // the vector compare that wrote it; the compiler does not pad inline assembly)
+                        asm("s_nop 1\n\tv_writelane_b32 %0, %1, %3\n\tv_writelane_b32 %0, %2, %4"
+                            : "+v"(mine)
+                            : "s"(m_lo), "s"(m_hi), "n"(rlo), "n"(rlo + 4));
+                    }
+                    if (e_lane < 32) tw[(e_wm * 64 + i * 32 + e_lane) * (BN / 32) + (e_wn * 2 + j)] = static_cast<uint32_t>(mine);
+                }
+            __syncthreads();
+            uint32_t* keys = static_cast<uint32_t*>(a.out);
+            if (H <= 32) {
+                const int tpt = 32 / H;
+                const uint32_t mask = (H == 32) ? 0xFFFFFFFFu : ((1u << H) - 1u);
+                // (table slot tl, row) pairs, rows fastest: a thread keeps its row and steps tl by
+                // NTHREADS / BM, carrying (tc, sub) = (tl / tpt, tl % tpt) along without dividing
+                constexpr int TL_STEP = NTHREADS / BM;
+                const int row = e_tid % BM, grow = rt * BM + row;
+                int tl = e_tid / BM;
+                int tc = tl / tpt, sub = tl - tc * tpt;
+                for (; tl < (BN / 32) * tpt; tl += TL_STEP) {
+                    const int table = (ct * (BN / 32) + tc) * tpt + sub;
+                    if (table < T && grow < n) {
+                        const uint32_t field = (tw[row * (BN / 32) + tc] >> (sub * H)) & mask;
+                        keys[static_cast<size_t>(table) * n + grow] = field << (32 - H);
+                    }
+                    sub += TL_STEP;
+                    while (sub >= tpt) { sub -= tpt; ++tc; }
+                }
+            } else {
+                const int wt = (H + 31) >> 5;
+                for (int idx = e_tid; idx < (BN / 32) * BM; idx += NTHREADS) {
+                    const int tc = idx / BM, row = idx - tc * BM;
+                    const int tile = ct * (BN / 32) + tc;
+                    const int table = tile / wt, w = tile - table * wt;
+                    const int grow = rt * BM + row;
+                    if (table < T && grow < n) {
+                        const int nbits = min(32, H - 32 * w);
+                        const uint32_t mask = (nbits == 32) ? 0xFFFFFFFFu : (0xFFFFFFFFu << (32 - nbits));
+                        keys[(static_cast<size_t>(table) * n + grow) * wt + w] = tw[row * (BN / 32) + tc] & mask;
+                    }
+                }
             }
         } else {
-            const int wt = (H + 31) >> 5;
-            for (int idx = tid; idx < (BN / 32) * BM; idx += NTHREADS) {
-                const int tc = idx / BM, row = idx - tc * BM;
-                const int tile = ct * (BN / 32) + tc;
-                const int table = tile / wt, w = tile - table * wt;
-                const int grow = rt * BM + row;
-                if (table < T && grow < n) {
-                    const int nbits = min(32, H - 32 * w);
-                    const uint32_t mask = (nbits == 32) ? 0xFFFFFFFFu : (0xFFFFFFFFu << (32 - nbits));
-                    keys[(static_cast<size_t>(table) * n + grow) * wt + w] = tw[row * (BN / 32) + tc] & mask;
-                }
-            }
-        }
-    } else {
-        // Transposed tiles: registers 4g..4g+3 of lane l hold row l%32, columns 8g + 4*(l/32) + 0..3.
-        // When H is a multiple of 4 those are four neighbouring hashes of one table, stored at once;
-        // the 32 lanes of a half wave then cover 32 consecutive rows, H * 4 bytes apart.
-        const bool quad = (H & 3) == 0 && (reinterpret_cast<uintptr_t>(a.out) & 15) == 0 &&
-                          (!FLOOR || (reinterpret_cast<uintptr_t>(a.b) & 15) == 0);
+            // Transposed tiles: registers 4g..4g+3 of e_lane l hold row l%32, columns 8g + 4*(l/32) + 0..3.
+            // When H is a multiple of 4 those are four neighbouring hashes of one table, stored at once;
+            // the 32 lanes of a e_half wave then cover 32 consecutive rows, H * 4 bytes apart.
+            const bool quad = (H & 3) == 0 && (reinterpret_cast<uintptr_t>(a.out) & 15) == 0 &&
+                              (!FLOOR || (reinterpret_cast<uintptr_t>(a.b) & 15) == 0);
 #pragma unroll
-        for (int j = 0; j < 2; ++j) {
-            const int cb = ct * BN + wn * 64 + j * 32 + 4 * half;  // column of register 0
-            int t = cb / H, h = cb - t * H;
+            for (int j = 0; j < 2; ++j) {
+                const int cb = ct * BN + e_wn * 64 + j * 32 + 4 * e_half;  // column of register 0
+                int t = cb / H, h = cb - t * H;
 #pragma unroll
-            for (int g = 0; g < 4; ++g) {
-                const int c0 = cb + 8 * g;
-                if (quad) {
-                    if (c0 < TH) {
-                        float4 bias = make_float4(0.f, 0.f, 0.f, 0.f);
-                        if (FLOOR) bias = *reinterpret_cast<const float4*>(a.b + c0);
-                        int4 lo = make_int4(INT_MAX, INT_MAX, INT_MAX, INT_MAX), hi = make_int4(INT_MIN, INT_MIN, INT_MIN, INT_MIN);
-#pragma unroll
-                        for (int i = 0; i < 2; ++i) {
-                            const int row = rt * BM + wm * 64 + i * 32 + r32;
-                            if (row >= n) continue;
-                            const size_t off = (static_cast<size_t>(t) * n + row) * H + h;
-                            const float x0 = acc[i][j][4 * g], x1 = acc[i][j][4 * g + 1];
-                            const float x2 = acc[i][j][4 * g + 2], x3 = acc[i][j][4 * g + 3];
-                            if (EPI == EPI_SIGN_BYTES) {
-                                const uint32_t bytes = ((__float_as_uint(x0) >> 31) ^ 1u) |
-                                                       (((__float_as_uint(x1) >> 31) ^ 1u) << 8) |
-                                                       (((__float_as_uint(x2) >> 31) ^ 1u) << 16) |
-                                                       (((__float_as_uint(x3) >> 31) ^ 1u) << 24);
-                                *reinterpret_cast<uint32_t*>(static_cast<uint8_t*>(a.out) + off) = bytes;
-                            } else {  // pslsh/hash.cuh:46
-                                const int4 v = make_int4(static_cast<int32_t>(floorf(x0 + bias.x)),
-                                                         static_cast<int32_t>(floorf(x1 + bias.y)),
-                                                         static_cast<int32_t>(floorf(x2 + bias.z)),
-                                                         static_cast<int32_t>(floorf(x3 + bias.w)));
-                                *reinterpret_cast<int4*>(static_cast<int32_t*>(a.out) + off) = v;
-                                if (FOLD_MM) {
-                                    lo.x = min(lo.x, v.x); lo.y = min(lo.y, v.y); lo.z = min(lo.z, v.z); lo.w = min(lo.w, v.w);
-                                    hi.x = max(hi.x, v.x); hi.y = max(hi.y, v.y); hi.z = max(hi.z, v.z); hi.w = max(hi.w, v.w);
-                                }
-                            }
-                        }
-                        if (FOLD_MM) {
-                            // the 32 lanes of a half wave hold 32 rows of the same four columns; eight copies of
-                            // the ranges (one per row residue, rows of MM_PITCH words: different banks) keep the
-                            // lanes that meet at one word down to four (sixteen copies measured no faster)
-                            int32_t* mn = &cmin[(r32 & 7) * MM_PITCH + (c0 - ct * BN)];
-                            int32_t* mx = &cmax[(r32 & 7) * MM_PITCH + (c0 - ct * BN)];
-                            atomicMin(mn, lo.x); atomicMin(mn + 1, lo.y); atomicMin(mn + 2, lo.z); atomicMin(mn + 3, lo.w);
-                            atomicMax(mx, hi.x); atomicMax(mx + 1, hi.y); atomicMax(mx + 2, hi.z); atomicMax(mx + 3, hi.w);
-                        }
-                    }
-                } else {
-                    int tq = t, hq = h;
-#pragma unroll
-                    for (int q = 0; q < 4; ++q) {
-                        if (c0 + q < TH) {
-                            const float bias = FLOOR ? a.b[c0 + q] : 0.f;
+                for (int g = 0; g < 4; ++g) {
+                    const int c0 = cb + 8 * g;
+                    if (quad) {
+                        if (c0 < TH) {
+                            float4 bias = make_float4(0.f, 0.f, 0.f, 0.f);
+                            if (FLOOR) bias = *reinterpret_cast<const float4*>(a.b + c0);
+                            int4 lo = make_int4(INT_MAX, INT_MAX, INT_MAX, INT_MAX), hi = make_int4(INT_MIN, INT_MIN, INT_MIN, INT_MIN);
 #pragma unroll
                             for (int i = 0; i < 2; ++i) {
-                                const int row = rt * BM + wm * 64 + i * 32 + r32;
+                                const int row = rt * BM + e_wm * 64 + i * 32 + e_r32;
                                 if (row >= n) continue;
-                                const size_t off = (static_cast<size_t>(tq) * n + row) * H + hq;
-                                const float x = acc[i][j][4 * g + q];
+                                const size_t off = (static_cast<size_t>(t) * n + row) * H + h;
+                                const float x0 = acc[i][j][4 * g], x1 = acc[i][j][4 * g + 1];
+                                const float x2 = acc[i][j][4 * g + 2], x3 = acc[i][j][4 * g + 3];
                                 if (EPI == EPI_SIGN_BYTES) {
-                                    static_cast<uint8_t*>(a.out)[off] =
-                                        static_cast<uint8_t>((__float_as_uint(x) >> 31) ^ 1u);
-                                } else {
-                                    static_cast<int32_t*>(a.out)[off] = static_cast<int32_t>(floorf(x + bias));
+                                    const uint32_t bytes = ((__float_as_uint(x0) >> 31) ^ 1u) |
+                                                           (((__float_as_uint(x1) >> 31) ^ 1u) << 8) |
+                                                           (((__float_as_uint(x2) >> 31) ^ 1u) << 16) |
+                                                           (((__float_as_uint(x3) >> 31) ^ 1u) << 24);
+                                    *reinterpret_cast<uint32_t*>(static_cast<uint8_t*>(a.out) + off) = bytes;
+                                } else {  // pslsh/hash.cuh:46
+                                    const int4 v = make_int4(static_cast<int32_t>(floorf(x0 + bias.x)),
+                                                             static_cast<int32_t>(floorf(x1 + bias.y)),
+                                                             static_cast<int32_t>(floorf(x2 + bias.z)),
+                                                             static_cast<int32_t>(floorf(x3 + bias.w)));
+                                    *reinterpret_cast<int4*>(static_cast<int32_t*>(a.out) + off) = v;
+                                    if (FOLD_MM) {
+                                        lo.x = min(lo.x, v.x); lo.y = min(lo.y, v.y); lo.z = min(lo.z, v.z); lo.w = min(lo.w, v.w);
+                                        hi.x = max(hi.x, v.x); hi.y = max(hi.y, v.y); hi.z = max(hi.z, v.z); hi.w = max(hi.w, v.w);
+                                    }
                                 }
                             }
+                            if (FOLD_MM) {
+                                // the 32 lanes of a e_half wave hold 32 rows of the same four columns; eight copies of
+                                // the ranges (one per row residue, rows of MM_PITCH words: different banks) keep the
+                                // lanes that meet at one word down to four (sixteen copies measured no faster)
+                                int32_t* mn = &cmin[(e_r32 & 7) * MM_PITCH + (c0 - ct * BN)];
+                                int32_t* mx = &cmax[(e_r32 & 7) * MM_PITCH + (c0 - ct * BN)];
+                                atomicMin(mn, lo.x); atomicMin(mn + 1, lo.y); atomicMin(mn + 2, lo.z); atomicMin(mn + 3, lo.w);
+                                atomicMax(mx, hi.x); atomicMax(mx + 1, hi.y); atomicMax(mx + 2, hi.z); atomicMax(mx + 3, hi.w);
+                            }
                         }
-                        if (++hq == H) { hq = 0; ++tq; }
+                    } else {
+                        int tq = t, hq = h;
+#pragma unroll
+                        for (int q = 0; q < 4; ++q) {
+                            if (c0 + q < TH) {
+                                const float bias = FLOOR ? a.b[c0 + q] : 0.f;
+#pragma unroll
+                                for (int i = 0; i < 2; ++i) {
+                                    const int row = rt * BM + e_wm * 64 + i * 32 + e_r32;
+                                    if (row >= n) continue;
+                                    const size_t off = (static_cast<size_t>(tq) * n + row) * H + hq;
+                                    const float x = acc[i][j][4 * g + q];
+                                    if (EPI == EPI_SIGN_BYTES) {
+                                        static_cast<uint8_t*>(a.out)[off] =
+                                            static_cast<uint8_t>((__float_as_uint(x) >> 31) ^ 1u);
+                                    } else {
+                                        static_cast<int32_t*>(a.out)[off] = static_cast<int32_t>(floorf(x + bias));
+                                    }
+                                }
+                            }
+                            if (++hq == H) { hq = 0; ++tq; }
+                        }
                     }
+                    h += 8;
+                    while (h >= H) { h -= H; ++t; }
                 }
-                h += 8;
-                while (h >= H) { h -= H; ++t; }
             }
         }
-        if (FOLD_MM) {  // the tile's ranges into the table's, again only where they would change
-            __syncthreads();
-            const int c = ct * BN + tid;
-            if (tid < BN && c < TH) {
-                int32_t lo = INT_MAX, hi = INT_MIN;
+        if (!has_next) break;
+        rt = rt_next;
+    }
+    if (FOLD_MM) {  // the tile's ranges into the table's, again only where they would change
+        __syncthreads();
+        const int c = ct * BN + tid;
+        if (tid < BN && c < TH) {
+            int32_t lo = INT_MAX, hi = INT_MIN;
 #pragma unroll
-                for (int k = 0; k < 8; ++k) {
-                    lo = min(lo, cmin[k * MM_PITCH + tid]);
-                    hi = max(hi, cmax[k * MM_PITCH + tid]);
-                }
-                if (lo <= hi) {
-                    if (lo < a.mm[2 * c]) atomicMin(&a.mm[2 * c], lo);
-                    if (hi > a.mm[2 * c + 1]) atomicMax(&a.mm[2 * c + 1], hi);
-                }
+            for (int k = 0; k < 8; ++k) {
+                lo = min(lo, cmin[k * MM_PITCH + tid]);
+                hi = max(hi, cmax[k * MM_PITCH + tid]);
+            }
+            if (lo <= hi) {
+                if (lo < a.mm[2 * c]) atomicMin(&a.mm[2 * c], lo);
+                if (hi > a.mm[2 * c + 1]) atomicMax(&a.mm[2 * c + 1], hi);
             }
         }
     }
@@ -607,10 +647,18 @@ culsh_status launch_project_f32(culsh_ctx* ctx, const float* X, const float* P, 
     a.mm = minmax;
     const bool fold_mm = floor_epi && minmax && minmax_folded && H % 4 == 0 &&
                          reinterpret_cast<uintptr_t>(out) % 16 == 0 && reinterpret_cast<uintptr_t>(b) % 16 == 0;
+    // With one column tile (T * H <= 128) workgroups stay and walk over row tiles (see the kernel): as many
+    // as fit on the device at once, in whole groups of 8.  With several column tiles every tile gets a
+    // workgroup of its own: the dispatch order then keeps the column tiles of a row tile close in time, which
+    // workgroups that each go their own way over hundreds of tiles do not (4M x 768 x 1024: 0.87 of the fp32
+    // MFMA peak against 0.83 with resident workgroups; 1M x 128 x 512: no difference; 1M x 128 x 128 with the
+    // floor epilogue: 0.55 against 0.59).
     const long long groups = (a.n_row_tiles + 7) / 8;
-    const long long blocks = groups * 8 * a.n_col_tiles;
-    CULSH_REQUIRE(blocks < (1ll << 31), CULSH_ERR_LIMIT, "projection grid too large");
-    dim3 grid(static_cast<unsigned>(blocks)), block(NTHREADS);
+    const long long per_group = 8ll * a.n_col_tiles;
+    const long long resident_groups = std::max(1ll, (static_cast<long long>(ctx->n_cus) * 4) / per_group);
+    const long long launched = a.n_col_tiles == 1 ? std::min(groups, resident_groups) : groups;
+    CULSH_REQUIRE(launched * per_group < (1ll << 31), CULSH_ERR_LIMIT, "projection grid too large");
+    dim3 grid(static_cast<unsigned>(launched * per_group)), block(NTHREADS);
     const bool vec = a.vec_x && a.vec_p;
     // 16 features per stage keep the kernel at 124 registers, i.e. 4 workgroups per CU instead of
     // the 3 that 32 features per stage allow: measured 1.06 ms against 1.14 ms at 1M x 128 x 512
