@@ -506,8 +506,9 @@ static culsh_status concat_candidates(culsh_ctx* ctx, const std::vector<culsh_ca
 
 // query over key words that are already in the arena
 static culsh_status query_keys(culsh_ctx* ctx, const uint32_t* q_keys, int nq, const culsh_index* ix,
-                               culsh_candidates* out, int32_t* lists_dst = nullptr, uint64_t lists_cap = 0) {
-    return query_from_keys(ctx, q_keys, nq, ix, out, lists_dst, lists_cap);
+                               culsh_candidates* out, int32_t* lists_dst = nullptr, uint64_t lists_cap = 0,
+                               int key_rows = 0, int key_first = 0) {
+    return query_from_keys(ctx, q_keys, nq, ix, out, lists_dst, lists_cap, key_rows, key_first);
 }
 
 template <typename T>
@@ -539,19 +540,31 @@ static culsh_status dense_query(culsh_ctx* ctx, Family fam, const T* Q, int nq, 
     struct Lists { int32_t* p = nullptr; ~Lists() { dev_free(p); } } lists;
     uint64_t lists_cap = 0, lists_used = 0;
     bool contiguous = true;  // all lists so far are (or can be put) in `lists` one behind the other
+    // The queries of all batches are hashed in one launch when their key words are a modest amount of memory
+    // (the batches bound the candidates, which are what is large): a batch of some thousand rows fills a
+    // fraction of the device, 10,000 rows x 768 x 1024 run at 0.62 of the fp32 MFMA peak against 0.87 for
+    // 100,000.  Every batch then looks its rows up in the key array of all queries.
+    uint32_t* all_keys = nullptr;
+    int W_all = 0;
+    // (p-stable hashing also holds the int32 hashes of all rows until the keys are made)
+    const size_t key_bytes = static_cast<size_t>(nq) * nT * (static_cast<size_t>(std::max(1, ix->key_w)) + (fam == FAM_RPLSH ? 0 : H)) *
+                             sizeof(uint32_t);
+    if (batch_size < nq && key_bytes <= (size_t(1) << 30))
+        CULSH_TRY(hash_dense_to_keys<T>(ctx, fam, Q, nq, d, nT, H, ix->P, ix->b, nullptr, ix, &all_keys, &W_all));
     for (int start = 0; start < nq; start += batch_size) {
         const int bn = std::min(batch_size, nq - start);
         const ArenaMark mark = arena_mark(ctx);
-        uint32_t* keys = nullptr;
-        int W = 0;
-        CULSH_TRY(hash_dense_to_keys<T>(ctx, fam, Q + static_cast<size_t>(start) * d, bn, d, nT, H, ix->P, ix->b,
-                                        nullptr, ix, &keys, &W));
+        uint32_t* keys = all_keys;
+        int W = W_all;
+        if (!all_keys)
+            CULSH_TRY(hash_dense_to_keys<T>(ctx, fam, Q + static_cast<size_t>(start) * d, bn, d, nT, H, ix->P, ix->b,
+                                            nullptr, ix, &keys, &W));
         CandPtr part(new (std::nothrow) culsh_candidates());
         CULSH_REQUIRE(part, CULSH_ERR_NOMEM, "host allocation failed");
         part->device = ctx->device;
         const bool room = lists.p && contiguous && lists_used < lists_cap;
         CULSH_TRY(query_keys(ctx, keys, bn, ix, part.get(), room ? lists.p + lists_used : nullptr,
-                             room ? lists_cap - lists_used : 0));
+                             room ? lists_cap - lists_used : 0, all_keys ? nq : 0, all_keys ? start : 0));
         const uint64_t found = part->n_total_candidates;
         if (start == 0 && bn < nq && found > 0) {
             const double per_query = static_cast<double>(found) / bn;

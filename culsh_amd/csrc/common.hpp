@@ -373,15 +373,18 @@ culsh_status build_key_directory(culsh_ctx* ctx, culsh_index* index, size_t buck
 
 culsh_status launch_find_matching_buckets(culsh_ctx* ctx, const uint32_t* q_keys, int n_queries,
                                           const culsh_index* index, int32_t* matched, void* spans = nullptr,
-                                          unsigned long long* raw_total = nullptr);
+                                          unsigned long long* raw_total = nullptr, int key_rows = 0, int key_first = 0);
 culsh_status query_from_matched(culsh_ctx* ctx, const int32_t* matched, int n_queries,
                                 const culsh_index* index, culsh_candidates* out);
 // lookup + candidate retrieval from key words [T][n_queries][key_w]
 // `lists_dst` (may be null): `lists_cap` elements of the caller's own, into which the lists are written when
 // that can be done without a copy and they fit (out->lists_in_place says so; out->query_candidate_indices stays
 // null then); else the result gets an array of its own as always.
+// `key_rows` > 0: the key array holds `key_rows` rows per table and this call's queries are the rows
+// key_first .. key_first + n_queries of every table (a batch out of keys that were hashed in one go).
 culsh_status query_from_keys(culsh_ctx* ctx, const uint32_t* q_keys, int n_queries, const culsh_index* index,
-                             culsh_candidates* out, int32_t* lists_dst = nullptr, uint64_t lists_cap = 0);
+                             culsh_candidates* out, int32_t* lists_dst = nullptr, uint64_t lists_cap = 0,
+                             int key_rows = 0, int key_first = 0);
 
 // Most hash tables an index may have (every fit, load and query checks it): the query kernels give each
 // table of a query one thread of a workgroup.

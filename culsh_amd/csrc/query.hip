@@ -123,7 +123,8 @@ __global__ __launch_bounds__(256) void lookup_kernel(const uint32_t* __restrict_
                                                     const int32_t* __restrict__ bucket_candidate_offsets,
                                                     int n_queries, int T, int W, int32_t* __restrict__ matched,
                                                     int2* __restrict__ spans,
-                                                    unsigned long long* __restrict__ raw_total) {
+                                                    unsigned long long* __restrict__ raw_total, int key_rows,
+                                                    int key_first) {
     __shared__ unsigned long long block_raw;
     if (threadIdx.x == 0) block_raw = 0ull;
     __syncthreads();
@@ -133,7 +134,8 @@ __global__ __launch_bounds__(256) void lookup_kernel(const uint32_t* __restrict_
     // they walk the same table's directory and buckets); results are stored per query
     const int t = live ? static_cast<int>(idx / n_queries) : 0, q = live ? static_cast<int>(idx - static_cast<size_t>(t) * n_queries) : 0;
     const size_t slot = static_cast<size_t>(q) * T + t;
-    const uint32_t* key = q_keys + (static_cast<size_t>(t) * n_queries + q) * W;
+    // the keys are [T][key_rows][W]; the queries of this call are the rows key_first .. key_first + n_queries of every table
+    const uint32_t* key = q_keys + (static_cast<size_t>(t) * key_rows + key_first + q) * W;
     int lo = live ? table_bucket_offsets[t] : 0, hi = live ? table_bucket_offsets[t + 1] - 1 : -1;
     if (live && dir) {
         const uint32_t lead = key[0] >> key_dir_shift(dir[0]);
@@ -791,13 +793,15 @@ culsh_status build_key_directory(culsh_ctx* ctx, culsh_index* index, size_t buck
 
 culsh_status launch_find_matching_buckets(culsh_ctx* ctx, const uint32_t* q_keys, int n_queries,
                                           const culsh_index* index, int32_t* matched, void* spans,
-                                          unsigned long long* raw_total) {
+                                          unsigned long long* raw_total, int key_rows, int key_first) {
+    if (key_rows <= 0) { key_rows = n_queries; key_first = 0; }
+    CULSH_REQUIRE(key_first >= 0 && key_first + n_queries <= key_rows, CULSH_ERR_INTERNAL, "lookup: queries outside the key array");
     const size_t pairs = static_cast<size_t>(n_queries) * index->n_hash_tables;
     CULSH_REQUIRE(pairs / 256 < (1ull << 31), CULSH_ERR_LIMIT, "too many (query, table) pairs");
     CULSH_REQUIRE(!spans || raw_total, CULSH_ERR_INTERNAL, "spans need a raw candidate counter");
     CULSH_LAUNCH(ctx, lookup_kernel, dim3(div_up(pairs, 256)), dim3(256), 0, ctx->stream, q_keys,
                  index->bucket_keys, index->key_dir, index->table_bucket_offsets, index->bucket_candidate_offsets, n_queries,
-                 index->n_hash_tables, index->key_w, matched, static_cast<int2*>(spans), raw_total);
+                 index->n_hash_tables, index->key_w, matched, static_cast<int2*>(spans), raw_total, key_rows, key_first);
     CULSH_LAUNCH_CHECK();
     return CULSH_OK;
 }
@@ -1180,7 +1184,7 @@ culsh_status query_from_matched(culsh_ctx* ctx, const int32_t* matched, int n_qu
 }
 
 culsh_status query_from_keys(culsh_ctx* ctx, const uint32_t* q_keys, int n_queries, const culsh_index* index,
-                             culsh_candidates* out, int32_t* lists_dst, uint64_t lists_cap) {
+                             culsh_candidates* out, int32_t* lists_dst, uint64_t lists_cap, int key_rows, int key_first) {
     CULSH_TRY(check_query_args(n_queries, index));
     int2* spans = nullptr;
     unsigned long long* raw_total = nullptr;
@@ -1188,7 +1192,7 @@ culsh_status query_from_keys(culsh_ctx* ctx, const uint32_t* q_keys, int n_queri
     DedupGeometry g;
     CULSH_TRY(dedup_geometry(ctx, index, &g));
     CULSH_TRY(alloc_query_words(ctx, n_queries, g, &raw_total));
-    CULSH_TRY(launch_find_matching_buckets(ctx, q_keys, n_queries, index, nullptr, spans, raw_total));
+    CULSH_TRY(launch_find_matching_buckets(ctx, q_keys, n_queries, index, nullptr, spans, raw_total, key_rows, key_first));
     return query_from_spans(ctx, spans, raw_total, n_queries, index, g, out, lists_dst, lists_cap);
 }
 
